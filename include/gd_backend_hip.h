@@ -1,0 +1,357 @@
+/*
+ * gd_backend_hip.h - C-ABI of the MI355X (gfx950) backend for the gradients.c
+ * inference decode path.
+ *
+ * Every `gd_backend_*` symbol declared in part 1-3 has the name, argument order,
+ * struct layout and status behaviour of the symbol of the same name in the
+ * reference's backend boundary, reference file `src/core/backend.h` (one backend
+ * is linked per build there; this library is that backend for HIP).  Each
+ * declaration cites the reference lines it replaces.  Part 4 holds entry points
+ * that have no counterpart in the reference (device argmax, fused operators,
+ * stream timing, graph capture); they use the same view structs.
+ *
+ * Conventions (reference src/core/backend.h:132-140, src/ops/op_common.h:60-94):
+ *   - tensors are borrowed `gd_backend_tensor_view`s: buffer + BYTE offset,
+ *     element count, dtype code, rank, shape, strides in ELEMENTS; all views the
+ *     decode path passes are contiguous;
+ *   - matrices are `gd_backend_matrix_view`s with a row pitch in bytes;
+ *   - outputs are pre-allocated by the caller, the backend writes in place;
+ *   - argument structs are read during the call only;
+ *   - between gd_backend_scope_begin and gd_backend_record_fence operators are
+ *     enqueued asynchronously in order on one HIP stream; outside a scope each
+ *     operator returns after its work has completed;
+ *   - device-side invalid cache positions are skipped silently, never trap.
+ */
+#ifndef GD_BACKEND_HIP_H
+#define GD_BACKEND_HIP_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- part 1: status, dtype codes, handles, views ------------------------- */
+
+/* reference include/gradients/status.h:8-19 (same numeric values). */
+#ifndef GRADIENTS_STATUS_H
+typedef enum gd_status {
+    GD_OK = 0,
+    GD_ERR_INVALID_ARGUMENT = -1,
+    GD_ERR_OUT_OF_MEMORY = -2,
+    GD_ERR_FROZEN = -3,
+    GD_ERR_BUSY = -4,
+    GD_ERR_BAD_STATE = -5,
+    GD_ERR_UNSUPPORTED = -6,
+    GD_ERR_INTERNAL = -7,
+    GD_ERR_NOT_IMPLEMENTED = -8,
+    GD_ERR_IO = -9
+} gd_status;
+#endif
+
+/* dtype codes carried in view.dtype: reference include/gradients/tensor.h:49-57. */
+#define GD_BACKEND_DTYPE_F16 1u
+#define GD_BACKEND_DTYPE_BF16 2u
+#define GD_BACKEND_DTYPE_F32 3u
+#define GD_BACKEND_DTYPE_I32 4u
+#define GD_BACKEND_DTYPE_U8 5u
+#define GD_BACKEND_DTYPE_U16 6u
+
+#define GD_BACKEND_MAX_DIMS 8u
+
+typedef struct gd_backend gd_backend;               /* backend.h:10 */
+typedef struct gd_backend_buffer gd_backend_buffer; /* backend.h:11 */
+
+/* backend.h:13-15 */
+typedef struct gd_backend_fence {
+    void *handle;
+} gd_backend_fence;
+
+/* backend.h:17-19; the reference defines only METAL = 1. */
+typedef enum gd_backend_kind {
+    GD_BACKEND_METAL = 1,
+    GD_BACKEND_HIP = 2
+} gd_backend_kind;
+
+/* backend.h:21-28 */
+typedef struct gd_backend_matrix_view {
+    gd_backend_buffer *buffer;
+    size_t offset;    /* bytes */
+    uint32_t rows;
+    uint32_t cols;
+    size_t row_bytes; /* pitch */
+    uint32_t dtype;
+} gd_backend_matrix_view;
+
+/* backend.h:45-50 */
+typedef struct gd_backend_vector_view {
+    gd_backend_buffer *buffer;
+    size_t offset;
+    uint32_t length;
+    uint32_t dtype;
+} gd_backend_vector_view;
+
+/* backend.h:132-140 */
+typedef struct gd_backend_tensor_view {
+    gd_backend_buffer *buffer;
+    size_t offset; /* bytes */
+    size_t count;  /* elements */
+    uint32_t dtype;
+    uint32_t rank;
+    int64_t shape[8];
+    int64_t strides[8]; /* elements */
+} gd_backend_tensor_view;
+
+/* ---- part 2: lifecycle, buffers, scope, transfers ------------------------ */
+
+/* backend.h:144-148.  GD_ERR_UNSUPPORTED when no HIP device is present. */
+gd_status gd_backend_create_default(gd_backend **out_backend);
+void gd_backend_destroy(gd_backend *backend);
+gd_backend_kind gd_backend_kind_query(const gd_backend *backend);
+const char *gd_backend_name(const gd_backend *backend);
+
+/* backend.h:150-156.  Buffers are HBM allocations; host_ptr is NULL and
+ * is_host_visible false unless the backend was created with the environment
+ * variable GD_HIP_HOST_VISIBLE=1 (pinned host memory mapped into the device,
+ * for running an unmodified reference core; not for performance). */
+gd_status gd_backend_buffer_create(gd_backend *backend, size_t nbytes, gd_backend_buffer **out_buffer);
+void gd_backend_buffer_destroy(gd_backend_buffer *buffer);
+size_t gd_backend_buffer_nbytes(const gd_backend_buffer *buffer);
+void *gd_backend_buffer_host_ptr(gd_backend_buffer *buffer);
+bool gd_backend_buffer_is_host_visible(const gd_backend_buffer *buffer);
+
+/* backend.h:158-159.  scope_begin: GD_ERR_BAD_STATE when nested (reference
+ * src/backends/metal/backend_metal.m:541-544).  flush = submit + block. */
+gd_status gd_backend_scope_begin(gd_backend *backend);
+gd_status gd_backend_flush(gd_backend *backend);
+
+/* backend.h:161-170; synchronous, ordered after all enqueued work. */
+gd_status gd_backend_upload(gd_backend *backend, gd_backend_buffer *buffer, size_t offset,
+                            const void *src, size_t nbytes);
+gd_status gd_backend_download(gd_backend *backend, gd_backend_buffer *buffer, size_t offset,
+                              void *dst, size_t nbytes);
+
+/* backend.h:172-177; elem_size in {1,2,4}, pattern's low bytes repeated. */
+gd_status gd_backend_fill(gd_backend *backend, gd_backend_buffer *buffer, size_t offset,
+                          size_t count, size_t elem_size, uint32_t pattern);
+
+/* backend.h:788-791.  record_fence closes the scope opened by scope_begin. */
+gd_status gd_backend_record_fence(gd_backend *backend, gd_backend_fence *out_fence);
+void gd_backend_fence_destroy(gd_backend_fence *fence);
+bool gd_backend_fence_is_complete(gd_backend_fence *fence);
+gd_status gd_backend_fence_wait(gd_backend_fence *fence);
+
+/* ---- part 3: operators on the decode path -------------------------------- */
+
+/* backend.h:301-312.  out[i,:] = table[ids[i],:]; id out of range -> NaN row
+ * (reference src/ops/embedding/metal_embedding.metal:26-30). */
+typedef struct gd_backend_embedding_args {
+    uint64_t ids_count;
+    uint64_t vocab;
+    uint64_t dim;
+} gd_backend_embedding_args;
+gd_status gd_backend_embedding_forward(gd_backend *backend, const gd_backend_tensor_view *table,
+                                       const gd_backend_tensor_view *ids,
+                                       const gd_backend_tensor_view *out,
+                                       const gd_backend_embedding_args *args);
+
+/* backend.h:528-544.  Only rows, cols, eps are read by the forward. */
+typedef struct gd_backend_rms_norm_args {
+    uint64_t rows;
+    uint64_t cols;
+    uint64_t row_blocks;
+    float eps;
+    uint32_t simdgroups;
+    uint32_t wgrad_simdgroups;
+    uint32_t wgrad_row_block;
+    uint32_t reserved0;
+} gd_backend_rms_norm_args;
+gd_status gd_backend_rms_norm_forward(gd_backend *backend, const gd_backend_tensor_view *x,
+                                      const gd_backend_tensor_view *weight,
+                                      const gd_backend_tensor_view *out,
+                                      const gd_backend_rms_norm_args *args);
+
+/* backend.h:187-195.  F16 operands, F32 accumulate, one F16 rounding.
+ * matmul: y[M,N] = x[M,K] w[K,N].  matmul_nt: y = x w^T with w stored [N,K]. */
+gd_status gd_backend_matmul(gd_backend *backend, const gd_backend_matrix_view *x,
+                            const gd_backend_matrix_view *w, const gd_backend_matrix_view *y);
+gd_status gd_backend_matmul_nt(gd_backend *backend, const gd_backend_matrix_view *x,
+                               const gd_backend_matrix_view *w, const gd_backend_matrix_view *y);
+/* backend.h:215-219.  y = x w + bias, bias added in F32 before the rounding
+ * (reference src/ops/_shared/gemm/metal_gemm_common.h:125-132). */
+gd_status gd_backend_linear(gd_backend *backend, const gd_backend_matrix_view *x,
+                            const gd_backend_matrix_view *w, const gd_backend_vector_view *bias,
+                            const gd_backend_matrix_view *y);
+
+/* reference src/core/backend_generated.h:14-17.  F16 add with NumPy-style
+ * right-aligned broadcasting of contiguous operands; residual adds (same shape)
+ * and bias adds ([rows,N] + [N]) are the shapes the decode path uses. */
+gd_status gd_backend_add(gd_backend *backend, const gd_backend_tensor_view *x,
+                         const gd_backend_tensor_view *y, const gd_backend_tensor_view *out);
+
+/* backend.h:321-325, 341-349.  qkv [N, 3*H*D] -> q,k rotated, v copied, each
+ * [N,H,D]; full-head rotation only (n_dims == head_dim). */
+typedef struct gd_backend_rope_args {
+    float theta;
+    uint32_t n_dims;
+    uint32_t interleaved;
+} gd_backend_rope_args;
+gd_status gd_backend_qkv_split_rope_forward(gd_backend *backend, const gd_backend_tensor_view *qkv,
+                                            const gd_backend_tensor_view *pos_ids,
+                                            const gd_backend_tensor_view *q,
+                                            const gd_backend_tensor_view *k,
+                                            const gd_backend_tensor_view *v, uint32_t n_heads,
+                                            uint32_t head_dim, const gd_backend_rope_args *args);
+
+/* backend.h:520-522.  out[r,c] = x12[r,c] * silu(x12[r,H+c]). */
+gd_status gd_backend_swiglu_split_forward(gd_backend *backend, const gd_backend_tensor_view *x12,
+                                          const gd_backend_tensor_view *out);
+
+/* backend.h:671-698.  Packed causal attention over cu_seqlens; stats may be
+ * NULL (inference).  Head dim up to 128 (the reference stops at 64). */
+typedef struct gd_backend_sdpa_varlen_args {
+    float scale;
+    uint32_t causal;
+    uint32_t sliding_window;
+    uint32_t prefix_len;
+    uint32_t max_seqlen;
+    uint32_t use_forward_stats;
+} gd_backend_sdpa_varlen_args;
+gd_status gd_backend_sdpa_varlen(gd_backend *backend, const gd_backend_tensor_view *q,
+                                 const gd_backend_tensor_view *k, const gd_backend_tensor_view *v,
+                                 const gd_backend_tensor_view *cu_seqlens,
+                                 const gd_backend_tensor_view *out,
+                                 const gd_backend_tensor_view *stats,
+                                 const gd_backend_sdpa_varlen_args *args);
+
+/* backend.h:680-685, 710-729.  q/out [B,Tq,Hq,D], caches [B,Tmax,Hkv,D].
+ * `sdpa_decode` takes a rank-0 I32 position tensor, `_at` a host scalar in
+ * args->cache_pos, `_positions` an I32 [B] tensor.  A negative position leaves
+ * that batch row of `out` untouched. */
+typedef struct gd_backend_sdpa_decode_args {
+    float scale;
+    uint32_t sliding_window;
+    uint32_t prefix_len;
+    int32_t cache_pos;
+} gd_backend_sdpa_decode_args;
+gd_status gd_backend_sdpa_decode(gd_backend *backend, const gd_backend_tensor_view *q,
+                                 const gd_backend_tensor_view *k_cache,
+                                 const gd_backend_tensor_view *v_cache,
+                                 const gd_backend_tensor_view *cache_pos,
+                                 const gd_backend_tensor_view *out,
+                                 const gd_backend_sdpa_decode_args *args);
+gd_status gd_backend_sdpa_decode_at(gd_backend *backend, const gd_backend_tensor_view *q,
+                                    const gd_backend_tensor_view *k_cache,
+                                    const gd_backend_tensor_view *v_cache,
+                                    const gd_backend_tensor_view *out,
+                                    const gd_backend_sdpa_decode_args *args);
+gd_status gd_backend_sdpa_decode_positions(gd_backend *backend, const gd_backend_tensor_view *q,
+                                           const gd_backend_tensor_view *k_cache,
+                                           const gd_backend_tensor_view *v_cache,
+                                           const gd_backend_tensor_view *cache_pos,
+                                           const gd_backend_tensor_view *out,
+                                           const gd_backend_sdpa_decode_args *args);
+
+/* backend.h:687-689, 730-750.  cache[b, pos_b + t] = new[b, t]; rows whose
+ * position is negative or whose span would pass Tmax are skipped on the device
+ * (reference src/ops/kv_cache_append/metal_kv_cache_append.metal:52-54,102-113). */
+typedef struct gd_backend_kv_cache_append_args {
+    int32_t cache_pos;
+} gd_backend_kv_cache_append_args;
+gd_status gd_backend_kv_cache_append_at(gd_backend *backend, const gd_backend_tensor_view *k_cache,
+                                        const gd_backend_tensor_view *v_cache,
+                                        const gd_backend_tensor_view *k_new,
+                                        const gd_backend_tensor_view *v_new,
+                                        const gd_backend_kv_cache_append_args *args);
+gd_status gd_backend_kv_cache_append_positions(gd_backend *backend,
+                                               const gd_backend_tensor_view *k_cache,
+                                               const gd_backend_tensor_view *v_cache,
+                                               const gd_backend_tensor_view *cache_pos,
+                                               const gd_backend_tensor_view *k_new,
+                                               const gd_backend_tensor_view *v_new,
+                                               const gd_backend_kv_cache_append_args *args);
+gd_status gd_backend_kv_cache_append_packed(gd_backend *backend,
+                                            const gd_backend_tensor_view *k_cache,
+                                            const gd_backend_tensor_view *v_cache,
+                                            const gd_backend_tensor_view *cache_pos,
+                                            const gd_backend_tensor_view *cu_seqlens,
+                                            const gd_backend_tensor_view *k_new,
+                                            const gd_backend_tensor_view *v_new,
+                                            const gd_backend_kv_cache_append_args *args);
+
+/* ---- part 4: entry points without a counterpart in the reference --------- */
+
+/* Greedy next token on the device.  The reference downloads the logits and
+ * scans them on the host (examples/gpt_lm/gpt_lm_shared.c:1388-1400): index of
+ * the largest finite value, first occurrence wins, 0 when no value is finite.
+ * logits F16 or F32 [rows, cols]; ids I32 [rows]; gap (optional, may be NULL)
+ * F32 [rows] = best - second best finite value (+inf when fewer than two). */
+gd_status gd_backend_argmax_rows(gd_backend *backend, const gd_backend_tensor_view *logits,
+                                 const gd_backend_tensor_view *ids,
+                                 const gd_backend_tensor_view *gap);
+
+/* Fused form of the reference's two-step gd_swiglu_split + gd_linear
+ * (src/ops/swiglu_split_linear/core_swiglu_split_linear.c:260-263):
+ * y = half(half(x12[:, :H] * silu(x12[:, H:])) @ w[H,N] + bias).  The F16
+ * rounding of the activation is kept.  bias may be NULL. */
+gd_status gd_backend_swiglu_split_linear(gd_backend *backend, const gd_backend_matrix_view *x12,
+                                         const gd_backend_matrix_view *w,
+                                         const gd_backend_vector_view *bias,
+                                         const gd_backend_matrix_view *y);
+
+/* y = half(half(x w^T) + bias): matmul_nt followed by the bias add in one
+ * launch, keeping both F16 roundings of the reference's two-kernel sequence
+ * (src/ops/linear_transposed_weight/core_linear_transposed_weight.c:51,76).
+ * bias may be NULL (then identical to gd_backend_matmul_nt). */
+gd_status gd_backend_linear_nt(gd_backend *backend, const gd_backend_matrix_view *x,
+                               const gd_backend_matrix_view *w, const gd_backend_vector_view *bias,
+                               const gd_backend_matrix_view *y);
+
+/* out[i,:] = src[rows[i],:]; replaces the reference's per-sequence slice +
+ * concat when the last prompt rows are selected
+ * (examples/gpt_lm/gpt_lm_shared.c:1117-1169).  Row index out of range -> row
+ * left untouched. */
+gd_status gd_backend_gather_rows(gd_backend *backend, const gd_backend_tensor_view *src,
+                                 const gd_backend_tensor_view *rows,
+                                 const gd_backend_tensor_view *out);
+
+/* dst[i] = src[i] + delta for contiguous I32 tensors (device-resident cache
+ * positions advance without a host round trip). */
+gd_status gd_backend_add_scalar_i32(gd_backend *backend, const gd_backend_tensor_view *src,
+                                    const gd_backend_tensor_view *dst, int32_t delta);
+
+/* Device copy between buffers, enqueued like an operator. */
+gd_status gd_backend_copy(gd_backend *backend, gd_backend_buffer *dst, size_t dst_offset,
+                          gd_backend_buffer *src, size_t src_offset, size_t nbytes);
+
+/* Stream timers: events recorded on the backend's own stream. */
+typedef struct gd_backend_timer gd_backend_timer;
+gd_status gd_backend_timer_create(gd_backend *backend, gd_backend_timer **out_timer);
+void gd_backend_timer_destroy(gd_backend_timer *timer);
+gd_status gd_backend_timer_start(gd_backend_timer *timer);
+gd_status gd_backend_timer_stop(gd_backend_timer *timer);
+/* Blocks until the stop event has completed. */
+gd_status gd_backend_timer_elapsed_ms(gd_backend_timer *timer, float *out_ms);
+
+/* Graph capture of the operators enqueued between begin and end (must be
+ * inside a scope); launch replays them on the backend stream. */
+typedef struct gd_backend_graph gd_backend_graph;
+gd_status gd_backend_graph_begin_capture(gd_backend *backend);
+gd_status gd_backend_graph_end_capture(gd_backend *backend, gd_backend_graph **out_graph);
+gd_status gd_backend_graph_launch(gd_backend *backend, gd_backend_graph *graph);
+void gd_backend_graph_destroy(gd_backend_graph *graph);
+
+/* Device facts for benchmarks: name, compute units, total global memory. */
+gd_status gd_backend_device_info(const gd_backend *backend, char *name, size_t name_len,
+                                 int32_t *compute_units, uint64_t *global_mem_bytes);
+
+/* Raw device address of a buffer (base of the allocation). */
+void *gd_backend_buffer_device_ptr(gd_backend_buffer *buffer);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* GD_BACKEND_HIP_H */
