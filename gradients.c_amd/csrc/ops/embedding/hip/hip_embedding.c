@@ -1,0 +1,56 @@
+/*
+ * Host dispatch of gd_backend_embedding_forward (reference src/core/backend.h:301-312),
+ * gd_backend_gather_rows and gd_backend_add_scalar_i32.
+ */
+#include "../../../backends/hip/backend_hip_internal.h"
+
+int gd_hip_launch_gather_rows(hipStream_t stream, const void *table, const int32_t *ids, void *out,
+                              uint64_t n_ids, uint64_t vocab, uint64_t row_bytes, uint32_t elem_size,
+                              int aligned16, int nan_on_invalid);
+int gd_hip_launch_add_scalar_i32(hipStream_t stream, const int32_t *src, int32_t *dst, uint64_t n, int32_t delta);
+
+static gd_status gather(gd_backend *backend, const gd_backend_tensor_view *table, const gd_backend_tensor_view *ids,
+                        const gd_backend_tensor_view *out, uint64_t n_ids, uint64_t vocab, uint64_t dim, int nan)
+{
+    size_t es;
+    if (table->dtype != GD_BACKEND_DTYPE_F16 && table->dtype != GD_BACKEND_DTYPE_F32) return GD_ERR_UNSUPPORTED;
+    if (out->dtype != table->dtype || ids->dtype != GD_BACKEND_DTYPE_I32) return GD_ERR_UNSUPPORTED;
+    if (n_ids == 0u || vocab == 0u || dim == 0u || vocab > SIZE_MAX / dim || n_ids > SIZE_MAX / dim ||
+        table->count != (size_t)(vocab * dim) || ids->count != (size_t)n_ids || out->count != (size_t)(n_ids * dim) ||
+        (ids->offset & 3u) != 0u || vocab > 0x7fffffffu || n_ids * dim > 0x7fffffffull * 256u)
+        return GD_ERR_INVALID_ARGUMENT;
+    es = gd_hip_dtype_size(table->dtype);
+    return gd_hip_finish_op(backend, gd_hip_launch_gather_rows(
+        backend->stream, gd_hip_view_ptr(table), (const int32_t *)gd_hip_view_ptr(ids), gd_hip_view_ptr(out),
+        n_ids, vocab, dim * es, (uint32_t)es, ((table->offset | out->offset) & 15u) == 0u, nan));
+}
+
+gd_status gd_backend_embedding_forward(gd_backend *backend, const gd_backend_tensor_view *table,
+                                       const gd_backend_tensor_view *ids, const gd_backend_tensor_view *out,
+                                       const gd_backend_embedding_args *args)
+{
+    if (backend == NULL || args == NULL || !gd_hip_view_ok(table) || !gd_hip_view_ok(ids) || !gd_hip_view_ok(out))
+        return GD_ERR_INVALID_ARGUMENT;
+    return gather(backend, table, ids, out, args->ids_count, args->vocab, args->dim, 1);
+}
+
+gd_status gd_backend_gather_rows(gd_backend *backend, const gd_backend_tensor_view *src,
+                                 const gd_backend_tensor_view *rows, const gd_backend_tensor_view *out)
+{
+    if (backend == NULL || !gd_hip_view_ok(src) || !gd_hip_view_ok(rows) || !gd_hip_view_ok(out) ||
+        src->rank != 2u || out->rank != 2u || rows->rank != 1u || out->shape[0] != rows->shape[0] ||
+        out->shape[1] != src->shape[1])
+        return GD_ERR_INVALID_ARGUMENT;
+    return gather(backend, src, rows, out, (uint64_t)rows->shape[0], (uint64_t)src->shape[0],
+                  (uint64_t)src->shape[1], 0);
+}
+
+gd_status gd_backend_add_scalar_i32(gd_backend *backend, const gd_backend_tensor_view *src,
+                                    const gd_backend_tensor_view *dst, int32_t delta)
+{
+    if (backend == NULL || !gd_hip_view_ok(src) || !gd_hip_view_ok(dst) || src->dtype != GD_BACKEND_DTYPE_I32 ||
+        dst->dtype != GD_BACKEND_DTYPE_I32 || src->count != dst->count || ((src->offset | dst->offset) & 3u) != 0u)
+        return GD_ERR_INVALID_ARGUMENT;
+    return gd_hip_finish_op(backend, gd_hip_launch_add_scalar_i32(
+        backend->stream, (const int32_t *)gd_hip_view_ptr(src), (int32_t *)gd_hip_view_ptr(dst), src->count, delta));
+}

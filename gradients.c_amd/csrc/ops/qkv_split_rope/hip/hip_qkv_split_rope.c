@@ -1,0 +1,41 @@
+/*
+ * Host dispatch of gd_backend_qkv_split_rope_forward.  Checks restate the reference
+ * src/ops/qkv_split_rope/metal_qkv_split_rope.m:195-216 (shapes, even head size, full-head
+ * rotation only).
+ */
+#include "../../../backends/hip/backend_hip_internal.h"
+
+int gd_hip_launch_qkv_split_rope(hipStream_t stream, const void *qkv, const int32_t *pos, void *q, void *k,
+                                 void *v, uint64_t tokens, uint32_t heads, uint32_t head_dim, float theta,
+                                 uint32_t interleaved, int aligned16);
+
+static bool out_ok(const gd_backend_tensor_view *t, int64_t tokens, uint32_t heads, uint32_t head_dim)
+{
+    return gd_hip_view_ok(t) && t->dtype == GD_BACKEND_DTYPE_F16 && t->rank == 3u && t->shape[0] == tokens &&
+           t->shape[1] == (int64_t)heads && t->shape[2] == (int64_t)head_dim;
+}
+
+gd_status gd_backend_qkv_split_rope_forward(gd_backend *backend, const gd_backend_tensor_view *qkv,
+                                            const gd_backend_tensor_view *pos_ids,
+                                            const gd_backend_tensor_view *q, const gd_backend_tensor_view *k,
+                                            const gd_backend_tensor_view *v, uint32_t n_heads, uint32_t head_dim,
+                                            const gd_backend_rope_args *args)
+{
+    int64_t tokens;
+    uint64_t area;
+    if (backend == NULL || args == NULL || !gd_hip_view_ok(qkv) || !gd_hip_view_ok(pos_ids) || n_heads == 0u ||
+        head_dim == 0u || qkv->rank != 2u || qkv->dtype != GD_BACKEND_DTYPE_F16 ||
+        pos_ids->dtype != GD_BACKEND_DTYPE_I32 || pos_ids->rank != 1u || (pos_ids->offset & 3u) != 0u)
+        return GD_ERR_INVALID_ARGUMENT;
+    tokens = qkv->shape[0];
+    area = (uint64_t)n_heads * head_dim;
+    if (tokens <= 0 || pos_ids->shape[0] != tokens || (uint64_t)qkv->shape[1] != area * 3u ||
+        !out_ok(q, tokens, n_heads, head_dim) || !out_ok(k, tokens, n_heads, head_dim) ||
+        !out_ok(v, tokens, n_heads, head_dim) || (head_dim & 1u) != 0u || !(args->theta > 0.0f) ||
+        args->n_dims != head_dim || (uint64_t)tokens * area / 2u > 0x7fffffffull * 256u)
+        return GD_ERR_INVALID_ARGUMENT;
+    return gd_hip_finish_op(backend, gd_hip_launch_qkv_split_rope(
+        backend->stream, gd_hip_view_ptr(qkv), (const int32_t *)gd_hip_view_ptr(pos_ids), gd_hip_view_ptr(q),
+        gd_hip_view_ptr(k), gd_hip_view_ptr(v), (uint64_t)tokens, n_heads, head_dim, args->theta,
+        args->interleaved, ((qkv->offset | q->offset | k->offset | v->offset) & 15u) == 0u));
+}

@@ -1,0 +1,133 @@
+/*
+ * Host dispatch of gd_backend_sdpa_decode{,_at,_positions}.  Validation restates the
+ * reference dispatch src/ops/sdpa_decode/metal_sdpa_decode.m:60-150 with the head-size
+ * limit raised from 64 to 128 for the split-KV kernel (256 for the generic one).
+ */
+#include <math.h>
+
+#include "../../../backends/hip/backend_hip_internal.h"
+#include "hip_sdpa_decode_types.h"
+
+int gd_hip_launch_sdpa_decode_split(hipStream_t stream, const void *q, const void *k, const void *v,
+                                    const int32_t *pos, void *out, float *ws,
+                                    const gd_hip_sdpa_decode_params *params);
+int gd_hip_launch_sdpa_decode_generic(hipStream_t stream, const void *q, const void *k, const void *v,
+                                      const int32_t *pos, void *out, const gd_hip_sdpa_decode_params *params);
+
+#define GD_HIP_SDPA_MAX_DH 256
+
+static bool common_ok(const gd_backend_tensor_view *q, const gd_backend_tensor_view *k,
+                      const gd_backend_tensor_view *v, const gd_backend_tensor_view *out)
+{
+    uint32_t i;
+    if (!gd_hip_view_ok(q) || !gd_hip_view_ok(k) || !gd_hip_view_ok(v) || !gd_hip_view_ok(out)) return false;
+    if ((q->dtype != GD_BACKEND_DTYPE_F16 && q->dtype != GD_BACKEND_DTYPE_F32) || k->dtype != q->dtype ||
+        v->dtype != q->dtype || out->dtype != q->dtype || q->rank != 4u || k->rank != 4u || v->rank != 4u ||
+        out->rank != 4u)
+        return false;
+    for (i = 0u; i < 4u; ++i) {
+        if (k->shape[i] != v->shape[i] || out->shape[i] != q->shape[i]) return false;
+    }
+    return q->shape[0] == k->shape[0] && q->shape[3] == k->shape[3] && (q->shape[2] % k->shape[2]) == 0 &&
+           q->shape[0] <= (int64_t)INT32_MAX && q->shape[1] <= (int64_t)INT32_MAX &&
+           k->shape[1] <= (int64_t)INT32_MAX && q->shape[2] <= 65535 && k->shape[2] <= 65535 &&
+           q->shape[3] <= GD_HIP_SDPA_MAX_DH;
+}
+
+static bool args_ok(const gd_backend_sdpa_decode_args *a, const gd_backend_tensor_view *k)
+{
+    return a != NULL && a->scale == a->scale && a->scale > 0.0f && isfinite(a->scale) &&
+           (int64_t)a->prefix_len <= k->shape[1] && a->sliding_window <= (uint32_t)INT32_MAX;
+}
+
+static gd_status dispatch(gd_backend *backend, const gd_backend_tensor_view *q, const gd_backend_tensor_view *k,
+                          const gd_backend_tensor_view *v, const gd_backend_tensor_view *pos,
+                          const gd_backend_tensor_view *out, const gd_backend_sdpa_decode_args *args,
+                          uint32_t pos_mode)
+{
+    gd_hip_sdpa_decode_params p;
+    const int32_t *pos_ptr = pos != NULL ? (const int32_t *)gd_hip_view_ptr(pos) : NULL;
+    uint32_t group;
+    p.batch = (uint32_t)q->shape[0];
+    p.tq = (uint32_t)q->shape[1];
+    p.tmax = (uint32_t)k->shape[1];
+    p.hq = (uint32_t)q->shape[2];
+    p.hkv = (uint32_t)k->shape[2];
+    p.dh = (uint32_t)q->shape[3];
+    p.window = args->sliding_window;
+    p.prefix_len = args->prefix_len;
+    p.pos_mode = pos_mode;
+    p.cache_pos = args->cache_pos;
+    p.scale = args->scale;
+    p.dtype = q->dtype;
+    p.chunk = 0u;
+    p.nsplit = 1u;
+    group = p.hq / p.hkv;
+    if (q->dtype == GD_BACKEND_DTYPE_F16 && p.tq == 1u && (p.dh == 64u || p.dh == 128u) && p.prefix_len == 0u &&
+        (group == 1u || group == 2u || group == 4u || group == 8u) &&
+        ((q->offset | k->offset | v->offset | out->offset) & 15u) == 0u && p.batch <= 65535u) {
+        /* longest key range a row can have */
+        uint32_t span = p.window > 0u && p.window < p.tmax ? p.window : p.tmax;
+        uint32_t chunk = (uint32_t)backend->sdpa_chunk;
+        gd_status st;
+        if (chunk == 0u) {
+            /* aim at >= 4 workgroups per compute unit, never less than 256 keys per workgroup */
+            const uint64_t pairs = (uint64_t)p.batch * p.hkv;
+            const uint64_t want = ((uint64_t)backend->compute_units * 4u + pairs - 1u) / pairs;
+            chunk = (uint32_t)((span + want - 1u) / want);
+            if (chunk < 256u) chunk = 256u;
+        }
+        chunk = (chunk + 31u) & ~31u;
+        if (chunk > span) chunk = (span + 31u) & ~31u;
+        p.chunk = chunk;
+        p.nsplit = (span + chunk - 1u) / chunk;
+        if (p.nsplit > 1u) {
+            st = gd_hip_reserve_attn_ws(backend, (size_t)p.batch * p.hq * p.nsplit * (p.dh + 2u) * sizeof(float));
+            if (st != GD_OK) return st;
+        }
+        return gd_hip_finish_op(backend, gd_hip_launch_sdpa_decode_split(
+            backend->stream, gd_hip_view_ptr(q), gd_hip_view_ptr(k), gd_hip_view_ptr(v), pos_ptr,
+            gd_hip_view_ptr(out), (float *)backend->attn_ws, &p));
+    }
+    if ((uint64_t)p.batch * p.hq * p.tq > 0x7fffffffu) return GD_ERR_UNSUPPORTED;
+    return gd_hip_finish_op(backend, gd_hip_launch_sdpa_decode_generic(
+        backend->stream, gd_hip_view_ptr(q), gd_hip_view_ptr(k), gd_hip_view_ptr(v), pos_ptr,
+        gd_hip_view_ptr(out), &p));
+}
+
+gd_status gd_backend_sdpa_decode(gd_backend *backend, const gd_backend_tensor_view *q,
+                                 const gd_backend_tensor_view *k_cache, const gd_backend_tensor_view *v_cache,
+                                 const gd_backend_tensor_view *cache_pos, const gd_backend_tensor_view *out,
+                                 const gd_backend_sdpa_decode_args *args)
+{
+    if (backend == NULL || !common_ok(q, k_cache, v_cache, out) || !gd_hip_view_ok(cache_pos) ||
+        cache_pos->dtype != GD_BACKEND_DTYPE_I32 || cache_pos->rank != 0u || cache_pos->count != 1u ||
+        (cache_pos->offset & 3u) != 0u || !args_ok(args, k_cache))
+        return GD_ERR_INVALID_ARGUMENT;
+    return dispatch(backend, q, k_cache, v_cache, cache_pos, out, args, GD_HIP_SDPA_POS_TENSOR0);
+}
+
+gd_status gd_backend_sdpa_decode_at(gd_backend *backend, const gd_backend_tensor_view *q,
+                                    const gd_backend_tensor_view *k_cache, const gd_backend_tensor_view *v_cache,
+                                    const gd_backend_tensor_view *out, const gd_backend_sdpa_decode_args *args)
+{
+    if (backend == NULL || !common_ok(q, k_cache, v_cache, out) || !args_ok(args, k_cache) ||
+        args->cache_pos < 0 || (int64_t)args->cache_pos > k_cache->shape[1] ||
+        q->shape[1] > k_cache->shape[1] - (int64_t)args->cache_pos)
+        return GD_ERR_INVALID_ARGUMENT;
+    return dispatch(backend, q, k_cache, v_cache, NULL, out, args, GD_HIP_SDPA_POS_SCALAR);
+}
+
+gd_status gd_backend_sdpa_decode_positions(gd_backend *backend, const gd_backend_tensor_view *q,
+                                           const gd_backend_tensor_view *k_cache,
+                                           const gd_backend_tensor_view *v_cache,
+                                           const gd_backend_tensor_view *cache_pos,
+                                           const gd_backend_tensor_view *out,
+                                           const gd_backend_sdpa_decode_args *args)
+{
+    if (backend == NULL || !common_ok(q, k_cache, v_cache, out) || !gd_hip_view_ok(cache_pos) ||
+        cache_pos->dtype != GD_BACKEND_DTYPE_I32 || cache_pos->rank != 1u || cache_pos->shape[0] != q->shape[0] ||
+        (cache_pos->offset & 3u) != 0u || !args_ok(args, k_cache))
+        return GD_ERR_INVALID_ARGUMENT;
+    return dispatch(backend, q, k_cache, v_cache, cache_pos, out, args, GD_HIP_SDPA_POS_VECTOR);
+}

@@ -1,0 +1,20 @@
+#ifndef GD_HIP_SDPA_DECODE_TYPES_H
+#define GD_HIP_SDPA_DECODE_TYPES_H
+#include <stdint.h>
+
+#define GD_HIP_SDPA_POS_SCALAR 0u  /* params.cache_pos */
+#define GD_HIP_SDPA_POS_TENSOR0 1u /* pos[0] for every batch row */
+#define GD_HIP_SDPA_POS_VECTOR 2u  /* pos[b] */
+
+typedef struct gd_hip_sdpa_decode_params {
+    uint32_t batch, tq, tmax, hq, hkv, dh;
+    uint32_t window, prefix_len;
+    uint32_t pos_mode;
+    int32_t cache_pos;
+    float scale;
+    uint32_t chunk;  /* keys per workgroup (split-KV kernel) */
+    uint32_t nsplit; /* workgroups per (batch, kv head) */
+    uint32_t dtype;  /* GD_BACKEND_DTYPE_F16 or _F32 (generic kernel) */
+} gd_hip_sdpa_decode_params;
+
+#endif

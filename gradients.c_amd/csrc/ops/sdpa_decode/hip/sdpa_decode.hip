@@ -1,0 +1,352 @@
+/*
+ * sdpa_decode for gfx950: attention of the newest query token(s) over the K/V cache.
+ *
+ * Replaces the reference kernels src/ops/sdpa_decode/metal_sdpa_decode.metal:86-175
+ * (Tq=1 window fast path) and :177-281 (general path, one active thread per query).
+ *
+ * The path is HBM-bound: every live K and V row is read once (algorithmic bytes =
+ * sum_b T_b * Hkv * D * 2 * 2 + q/out).  Split-KV kernel, F16, Tq == 1:
+ *   - grid (nsplit, Hkv, B); a workgroup of 4 wavefronts owns `chunk` consecutive keys of one
+ *     (batch, kv head) and all G = Hq/Hkv query heads that share it, so K/V bytes are read once;
+ *   - a wavefront load covers 64 lanes x 16 B = 1 KiB: D/8 lanes hold one key row (8 halfs each),
+ *     so one instruction fetches 8 (D=64) or 4 (D=128) whole rows, each a full 128/256-byte line;
+ *   - the dot product is reduced over the D/8 lanes of a row with shuffles; every row slot keeps
+ *     its own running max/sum (online softmax in the exp2 domain) and an F32 accumulator for its
+ *     8 channels, so the inner loop has no cross-slot traffic;
+ *   - slots are merged with shuffles, wavefronts through LDS; with nsplit == 1 the result is
+ *     normalised and stored as F16 directly, otherwise (max, sum, acc) partials go to a
+ *     workspace and a small combine kernel finishes.
+ * Everything else (F32 caches, Tq > 1, prefix masks, other head sizes) takes the generic
+ * kernel: one wavefront per query row, lane-per-key scores, lane-per-channel accumulation.
+ *
+ * Semantics (both kernels): live = min(pos + Tq, Tmax), query position pos + i, mask
+ * reference metal_sdpa_decode.metal:30-53, out = 0 when no key is visible, rows with a
+ * negative position are left untouched.
+ */
+#include "../../_shared/hip_device.h"
+#include "hip_sdpa_decode_types.h"
+
+#define GD_NEG_INF (-__builtin_inff())
+
+__device__ __forceinline__ bool gd_attn_allowed(int qpos, int j, int window, int prefix_len)
+{
+    if (prefix_len > 0) {
+        if (qpos < prefix_len) {
+            if (j >= prefix_len) return false;
+        } else if (j > qpos) {
+            return false;
+        }
+    } else if (j > qpos) {
+        return false;
+    }
+    if (window > 0) {
+        if (prefix_len > 0) {
+            if (qpos >= prefix_len && j >= prefix_len && (qpos - j) >= window) return false;
+        } else if ((qpos - j) >= window) {
+            return false;
+        }
+    }
+    return true;
+}
+
+__device__ __forceinline__ int gd_decode_pos(const int32_t *pos, const gd_hip_sdpa_decode_params &p, int b)
+{
+    if (p.pos_mode == GD_HIP_SDPA_POS_SCALAR) return p.cache_pos;
+    return pos[p.pos_mode == GD_HIP_SDPA_POS_VECTOR ? b : 0];
+}
+
+/* ---- split-KV kernel ----------------------------------------------------------- */
+
+#define GD_SDPA_WAVES 4
+
+template <int D, int G>
+__global__ void __launch_bounds__(GD_SDPA_WAVES * 64)
+gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__restrict__ kc,
+                            const gd_half *__restrict__ vc, const int32_t *__restrict__ pos_ptr,
+                            gd_half *__restrict__ out, float *__restrict__ ws, gd_hip_sdpa_decode_params p)
+{
+    constexpr int LPK = D / 8;      /* lanes per key row */
+    constexpr int KPW = 64 / LPK;   /* key rows per wavefront load */
+    constexpr int KPB = KPW * GD_SDPA_WAVES;
+    constexpr int UNROLL = 4;
+    const int split = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int slot = lane / LPK, sub = lane % LPK;
+
+    const int pos = gd_decode_pos(pos_ptr, p, b);
+    if (pos < 0) return;
+    const int live = min(pos + 1, (int)p.tmax);
+    const int first = p.window > 0u ? max(0, pos - (int)p.window + 1) : 0;
+    const int r0 = first + split * (int)p.chunk;
+    const int r1 = min(r0 + (int)p.chunk, live);
+    float *ws_row = ws + (((size_t)b * p.hq + (size_t)hkv * G) * p.nsplit + split) * (D + 2);
+    if (r0 >= r1) {
+        if (p.nsplit > 1u) {
+            if (threadIdx.x < G) {
+                float *w = ws_row + (size_t)threadIdx.x * p.nsplit * (D + 2);
+                w[0] = GD_NEG_INF;
+                w[1] = 0.f;
+            }
+        } else {
+            for (int idx = threadIdx.x; idx < G * D; idx += GD_SDPA_WAVES * 64)
+                out[((size_t)b * p.hq + (size_t)hkv * G) * D + idx] = (gd_half)0.f;
+        }
+        return;
+    }
+
+    /* query rows of the G heads that share this kv head, pre-scaled into the exp2 domain */
+    const float qscale = p.scale * 1.4426950408889634f;
+    float qf[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const gd_half8 qv = *reinterpret_cast<const gd_half8 *>(q + ((size_t)b * p.hq + (size_t)hkv * G + g) * D + sub * 8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qf[g][e] = (float)qv[e] * qscale;
+    }
+
+    float m[G], l[G], acc[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        m[g] = GD_NEG_INF;
+        l[g] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
+    }
+
+    const size_t row_stride = (size_t)p.hkv * D; /* elements between consecutive keys */
+    const gd_half *kbase = kc + ((size_t)b * p.tmax * p.hkv + hkv) * D + sub * 8;
+    const gd_half *vbase = vc + ((size_t)b * p.tmax * p.hkv + hkv) * D + sub * 8;
+
+    for (int j0 = r0 + wave * KPW + slot; j0 < r1 + 0; j0 += KPB * UNROLL) {
+        gd_half8 kv[UNROLL], vv[UNROLL];
+        bool ok[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int j = j0 + u * KPB;
+            ok[u] = j < r1;
+            const int jj = ok[u] ? j : (r1 - 1);
+            kv[u] = *reinterpret_cast<const gd_half8 *>(kbase + (size_t)jj * row_stride);
+            vv[u] = *reinterpret_cast<const gd_half8 *>(vbase + (size_t)jj * row_stride);
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            float kf[8], vf[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                kf[e] = (float)kv[u][e];
+                vf[e] = (float)vv[u][e];
+            }
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                float s = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) s = fmaf(qf[g][e], kf[e], s);
+#pragma unroll
+                for (int off = 1; off < LPK; off <<= 1) s += __shfl_xor(s, off, 64);
+                if (ok[u]) {
+                    const float mn = fmaxf(m[g], s);
+                    const float corr = exp2f(m[g] - mn); /* exp2(-inf) = 0 on the first key */
+                    const float pr = exp2f(s - mn);
+                    l[g] = l[g] * corr + pr;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[g][e] = acc[g][e] * corr + pr * vf[e];
+                    m[g] = mn;
+                }
+            }
+        }
+    }
+
+    /* merge the KPW row slots of the wavefront */
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int off = LPK; off < 64; off <<= 1) {
+            const float mo = __shfl_xor(m[g], off, 64);
+            const float lo = __shfl_xor(l[g], off, 64);
+            const float mn = fmaxf(m[g], mo);
+            const float c1 = (m[g] == GD_NEG_INF) ? 0.f : exp2f(m[g] - mn);
+            const float c2 = (mo == GD_NEG_INF) ? 0.f : exp2f(mo - mn);
+            l[g] = l[g] * c1 + lo * c2;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float ao = __shfl_xor(acc[g][e], off, 64);
+                acc[g][e] = acc[g][e] * c1 + ao * c2;
+            }
+            m[g] = mn;
+        }
+    }
+
+    /* merge the wavefronts through LDS */
+    __shared__ float sm_acc[GD_SDPA_WAVES][G][D];
+    __shared__ float sm_m[GD_SDPA_WAVES][G], sm_l[GD_SDPA_WAVES][G];
+    if (slot == 0) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sm_acc[wave][g][sub * 8 + e] = acc[g][e];
+            if (sub == 0) {
+                sm_m[wave][g] = m[g];
+                sm_l[wave][g] = l[g];
+            }
+        }
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < G * D; idx += GD_SDPA_WAVES * 64) {
+        const int g = idx / D, c = idx % D;
+        float mm = GD_NEG_INF;
+#pragma unroll
+        for (int w = 0; w < GD_SDPA_WAVES; ++w) mm = fmaxf(mm, sm_m[w][g]);
+        float ll = 0.f, aa = 0.f;
+#pragma unroll
+        for (int w = 0; w < GD_SDPA_WAVES; ++w) {
+            const float cw = (sm_m[w][g] == GD_NEG_INF) ? 0.f : exp2f(sm_m[w][g] - mm);
+            ll += sm_l[w][g] * cw;
+            aa += sm_acc[w][g][c] * cw;
+        }
+        if (p.nsplit > 1u) {
+            float *w = ws_row + (size_t)g * p.nsplit * (D + 2);
+            w[2 + c] = aa;
+            if (c == 0) {
+                w[0] = mm;
+                w[1] = ll;
+            }
+        } else {
+            out[((size_t)b * p.hq + (size_t)hkv * G + g) * D + c] = (gd_half)(ll > 0.f ? aa / ll : 0.f);
+        }
+    }
+}
+
+template <int D>
+__global__ void __launch_bounds__(D)
+gd_sdpa_decode_combine_kernel(const float *__restrict__ ws, const int32_t *__restrict__ pos_ptr,
+                              gd_half *__restrict__ out, gd_hip_sdpa_decode_params p)
+{
+    const int hq = blockIdx.x, b = blockIdx.y, c = threadIdx.x;
+    if (gd_decode_pos(pos_ptr, p, b) < 0) return;
+    const float *w = ws + ((size_t)b * p.hq + hq) * p.nsplit * (D + 2);
+    float mm = GD_NEG_INF;
+    for (uint32_t s = 0; s < p.nsplit; ++s) mm = fmaxf(mm, w[(size_t)s * (D + 2)]);
+    float ll = 0.f, aa = 0.f;
+    for (uint32_t s = 0; s < p.nsplit; ++s) {
+        const float ms = w[(size_t)s * (D + 2)];
+        if (ms == GD_NEG_INF) continue;
+        const float cw = exp2f(ms - mm);
+        ll += w[(size_t)s * (D + 2) + 1] * cw;
+        aa += w[(size_t)s * (D + 2) + 2 + c] * cw;
+    }
+    out[((size_t)b * p.hq + hq) * D + c] = (gd_half)(ll > 0.f ? aa / ll : 0.f);
+}
+
+/* ---- generic kernel -------------------------------------------------------------- */
+
+template <typename T>
+__global__ void __launch_bounds__(64)
+gd_sdpa_decode_generic_kernel(const T *__restrict__ q, const T *__restrict__ kc, const T *__restrict__ vc,
+                              const int32_t *__restrict__ pos_ptr, T *__restrict__ out,
+                              gd_hip_sdpa_decode_params p)
+{
+    __shared__ float qs[256];
+    __shared__ float ps[64];
+    const int lane = threadIdx.x;
+    int r = blockIdx.x;
+    const int i = r % (int)p.tq;
+    r /= (int)p.tq;
+    const int hq = r % (int)p.hq;
+    const int b = r / (int)p.hq;
+    const int pos = gd_decode_pos(pos_ptr, p, b);
+    if (pos < 0) return;
+    const int D = (int)p.dh;
+    const int hkv = hq / (int)(p.hq / p.hkv);
+    const int live = (int)min((long long)pos + (long long)p.tq, (long long)p.tmax);
+    const int qpos = pos + i;
+    const size_t qbase = (((size_t)b * p.tq + i) * p.hq + hq) * D;
+    for (int c = lane; c < D; c += 64) qs[c] = (float)q[qbase + c];
+    __syncthreads();
+
+    float m = GD_NEG_INF, l = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};
+    int jstart = 0;
+    if (p.window > 0u && p.prefix_len == 0u) jstart = max(0, qpos - (int)p.window + 1) & ~63;
+    for (int j0 = jstart; j0 < live; j0 += 64) {
+        const int j = j0 + lane;
+        const bool ok = j < live && gd_attn_allowed(qpos, j, (int)p.window, (int)p.prefix_len);
+        float s = GD_NEG_INF;
+        if (ok) {
+            const T *kr = kc + (((size_t)b * p.tmax + j) * p.hkv + hkv) * D;
+            float dot = 0.f;
+            for (int c = 0; c < D; ++c) dot = fmaf(qs[c], (float)kr[c], dot);
+            s = dot * p.scale;
+        }
+        const float cm = gd_wave_max(s);
+        if (cm == GD_NEG_INF) continue; /* uniform across the wavefront */
+        const float mn = fmaxf(m, cm);
+        const float corr = (m == GD_NEG_INF) ? 0.f : expf(m - mn);
+        const float pr = ok ? expf(s - mn) : 0.f;
+        l = l * corr + gd_wave_sum(pr);
+        __syncthreads();
+        ps[lane] = pr;
+        __syncthreads();
+        const int n = min(64, live - j0);
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+            const int c = lane + 64 * rr;
+            if (c < D) {
+                float a = acc[rr] * corr;
+                const T *vr = vc + (((size_t)b * p.tmax + j0) * p.hkv + hkv) * D + c;
+                for (int jj = 0; jj < n; ++jj) a = fmaf(ps[jj], (float)vr[(size_t)jj * p.hkv * D], a);
+                acc[rr] = a;
+            }
+        }
+        m = mn;
+    }
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+        const int c = lane + 64 * rr;
+        if (c < D) out[qbase + c] = (T)(acc[rr] * inv);
+    }
+}
+
+/* ---- launchers ----------------------------------------------------------------------- */
+
+template <int D, int G>
+static int launch_split(hipStream_t stream, const void *q, const void *k, const void *v, const int32_t *pos,
+                        void *out, float *ws, const gd_hip_sdpa_decode_params &p)
+{
+    dim3 grid(p.nsplit, p.hkv, p.batch);
+    gd_sdpa_decode_split_kernel<D, G><<<grid, GD_SDPA_WAVES * 64, 0, stream>>>(
+        (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, pos, (gd_half *)out, ws, p);
+    if (p.nsplit > 1u) {
+        dim3 cgrid(p.hq, p.batch);
+        gd_sdpa_decode_combine_kernel<D><<<cgrid, D, 0, stream>>>(ws, pos, (gd_half *)out, p);
+    }
+    return (int)hipGetLastError();
+}
+
+/* Returns hipErrorInvalidValue when (D, G) has no split-KV instantiation. */
+extern "C" int gd_hip_launch_sdpa_decode_split(hipStream_t stream, const void *q, const void *k, const void *v,
+                                               const int32_t *pos, void *out, float *ws,
+                                               const gd_hip_sdpa_decode_params *params)
+{
+    const gd_hip_sdpa_decode_params &p = *params;
+    const uint32_t g = p.hq / p.hkv;
+#define GD_CASE(DD, GG) if (p.dh == DD && g == GG) return launch_split<DD, GG>(stream, q, k, v, pos, out, ws, p)
+    GD_CASE(64, 1); GD_CASE(64, 2); GD_CASE(64, 4); GD_CASE(64, 8);
+    GD_CASE(128, 1); GD_CASE(128, 2); GD_CASE(128, 4); GD_CASE(128, 8);
+#undef GD_CASE
+    return (int)hipErrorInvalidValue;
+}
+
+extern "C" int gd_hip_launch_sdpa_decode_generic(hipStream_t stream, const void *q, const void *k, const void *v,
+                                                 const int32_t *pos, void *out,
+                                                 const gd_hip_sdpa_decode_params *params)
+{
+    const gd_hip_sdpa_decode_params &p = *params;
+    const unsigned blocks = p.batch * p.hq * p.tq;
+    if (p.dtype == 1u)
+        gd_sdpa_decode_generic_kernel<gd_half><<<blocks, 64, 0, stream>>>(
+            (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, pos, (gd_half *)out, p);
+    else
+        gd_sdpa_decode_generic_kernel<float><<<blocks, 64, 0, stream>>>(
+            (const float *)q, (const float *)k, (const float *)v, pos, (float *)out, p);
+    return (int)hipGetLastError();
+}

@@ -1,0 +1,48 @@
+/*
+ * Host dispatch of gd_backend_sdpa_varlen (reference src/core/backend.h:671-698; checks of
+ * src/ops/sdpa_varlen/core_sdpa_varlen.c:12-122 that concern the backend: shapes, dtype,
+ * head-size limit raised from 64 to 256, prefix needs causal).  The stats output of the
+ * training path is not produced: a non-NULL stats view is refused.
+ */
+#include <math.h>
+
+#include "../../../backends/hip/backend_hip_internal.h"
+
+int gd_hip_launch_sdpa_varlen(hipStream_t stream, const void *q, const void *k, const void *v, const int32_t *cu,
+                              void *out, uint32_t n_rows, uint32_t batch, uint32_t hq, uint32_t hkv, uint32_t dh,
+                              uint32_t causal, uint32_t window, uint32_t prefix_len, uint32_t max_seqlen, float scale,
+                              int is_f16);
+
+gd_status gd_backend_sdpa_varlen(gd_backend *backend, const gd_backend_tensor_view *q,
+                                 const gd_backend_tensor_view *k, const gd_backend_tensor_view *v,
+                                 const gd_backend_tensor_view *cu_seqlens, const gd_backend_tensor_view *out,
+                                 const gd_backend_tensor_view *stats, const gd_backend_sdpa_varlen_args *args)
+{
+    uint32_t i;
+    if (backend == NULL || args == NULL || !gd_hip_view_ok(q) || !gd_hip_view_ok(k) || !gd_hip_view_ok(v) ||
+        !gd_hip_view_ok(cu_seqlens) || !gd_hip_view_ok(out))
+        return GD_ERR_INVALID_ARGUMENT;
+    if (stats != NULL || args->use_forward_stats != 0u) return GD_ERR_UNSUPPORTED;
+    if ((q->dtype != GD_BACKEND_DTYPE_F16 && q->dtype != GD_BACKEND_DTYPE_F32) || k->dtype != q->dtype ||
+        v->dtype != q->dtype || out->dtype != q->dtype || cu_seqlens->dtype != GD_BACKEND_DTYPE_I32)
+        return GD_ERR_UNSUPPORTED;
+    if (q->rank != 3u || k->rank != 3u || v->rank != 3u || out->rank != 3u || cu_seqlens->rank != 1u ||
+        cu_seqlens->shape[0] < 2 || (cu_seqlens->offset & 3u) != 0u)
+        return GD_ERR_INVALID_ARGUMENT;
+    for (i = 0u; i < 3u; ++i) {
+        if (k->shape[i] != v->shape[i] || out->shape[i] != q->shape[i]) return GD_ERR_INVALID_ARGUMENT;
+    }
+    if (q->shape[0] != k->shape[0] || q->shape[2] != k->shape[2] || (q->shape[1] % k->shape[1]) != 0 ||
+        q->shape[2] > 256 || q->shape[1] > 65535 || (uint64_t)q->shape[0] * (uint64_t)q->shape[1] > 0x7fffffffu ||
+        cu_seqlens->shape[0] - 1 > (int64_t)INT32_MAX)
+        return GD_ERR_INVALID_ARGUMENT;
+    if (!(args->scale > 0.0f) || !isfinite(args->scale) || (args->prefix_len > 0u && args->causal == 0u) ||
+        (args->max_seqlen > 0u && args->prefix_len > args->max_seqlen))
+        return GD_ERR_INVALID_ARGUMENT;
+    return gd_hip_finish_op(backend, gd_hip_launch_sdpa_varlen(
+        backend->stream, gd_hip_view_ptr(q), gd_hip_view_ptr(k), gd_hip_view_ptr(v),
+        (const int32_t *)gd_hip_view_ptr(cu_seqlens), gd_hip_view_ptr(out), (uint32_t)q->shape[0],
+        (uint32_t)(cu_seqlens->shape[0] - 1), (uint32_t)q->shape[1], (uint32_t)k->shape[1], (uint32_t)q->shape[2],
+        args->causal, args->sliding_window, args->prefix_len, args->max_seqlen, args->scale,
+        q->dtype == GD_BACKEND_DTYPE_F16));
+}

@@ -347,6 +347,11 @@ void gd_backend_graph_destroy(gd_backend_graph *graph);
 gd_status gd_backend_device_info(const gd_backend *backend, char *name, size_t name_len,
                                  int32_t *compute_units, uint64_t *global_mem_bytes);
 
+/* Kernel tunables, normally left at 0 = automatic.  name "sdpa_chunk": keys per workgroup of
+ * the split-KV decode kernel (also read once from the environment variable
+ * GD_HIP_SDPA_CHUNK).  Unknown name -> GD_ERR_INVALID_ARGUMENT. */
+gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t value);
+
 /* Raw device address of a buffer (base of the allocation). */
 void *gd_backend_buffer_device_ptr(gd_backend_buffer *buffer);
 

@@ -1,0 +1,540 @@
+"""Parity of every HIP operator against the CPU oracle, through the C-ABI.
+
+Bars (BASELINE.json north_star): cache append, gathers, argmax ids and index maps are
+bit-exact; sdpa_decode, projections and rms_norm are within rtol 2e-3 / atol 1e-3 of the
+oracle in F16.  Inputs come from the oracle's splitmix64 + Box-Muller generator, seeded.
+"""
+import ctypes as C
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+RTOL, ATOL = 2e-3, 1e-3
+
+
+def _golden(name):
+    with open(os.path.join(GOLDEN, name)) as f:
+        return json.load(f)
+
+
+def _close(got, want, rtol=RTOL, atol=ATOL):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    err = np.abs(got - want)
+    bound = atol + rtol * np.abs(want)
+    assert np.all(err <= bound), f"max err {err.max():.3e}, worst excess {(err - bound).max():.3e}"
+
+
+def _bits(a):
+    return np.ascontiguousarray(a).view(np.uint16 if a.dtype == np.float16 else np.uint32)
+
+
+@pytest.fixture()
+def arena(backend):
+    buf = backend.buffer(512 << 20)
+    yield buf
+    backend.free(buf)
+
+
+# ---- lifecycle -------------------------------------------------------------------------
+
+def test_backend_identity_and_scope_rules(backend, gda):
+    assert backend.name.startswith("hip:")
+    assert gda.lib().gd_backend_kind_query(backend.handle) == 2
+    backend.scope_begin()
+    assert backend.call("gd_backend_scope_begin") == gda.BAD_STATE  # nested scope
+    f = backend.record_fence()
+    backend.fence_wait(f)
+    name, cus, mem = backend.device_info()
+    assert cus > 0 and mem > (1 << 30)
+
+
+def test_upload_download_fill(backend, arena, gda):
+    rng = np.random.default_rng(0)
+    a = rng.integers(0, 255, 100003, dtype=np.uint8)
+    t = arena.from_numpy(a)
+    assert np.array_equal(t.read(), a)
+    h = arena.alloc((1001,), gda.F16)
+    backend.fill(h, 0x3c00)
+    assert np.all(h.read() == np.float16(1.0))
+    w = arena.alloc((77,), gda.I32)
+    backend.fill(w, 0xdeadbeef)
+    assert np.all(w.read().view(np.uint32) == 0xdeadbeef)
+    b = arena.alloc((13,), gda.U8)
+    backend.fill(b, 0x5a)
+    assert np.all(b.read() == 0x5a)
+    # queued work is visible to a download inside a scope (program order)
+    backend.scope_begin()
+    backend.fill(h, 0x4000)
+    assert np.all(h.read() == np.float16(2.0))
+    backend.fence_wait(backend.record_fence())
+
+
+# ---- A1 kv_cache_append -------------------------------------------------------------------
+
+@pytest.mark.parametrize("np_dtype", [np.float32, np.float16])
+def test_append_reference_golden_vectors(backend, arena, gda, np_dtype):
+    g = _golden("kv_cache_append_vectors.json")
+    c = g["at"]
+    k = arena.from_numpy(np.zeros(c["cache_shape"], np_dtype))
+    v = arena.from_numpy(np.zeros(c["cache_shape"], np_dtype))
+    kn = arena.from_numpy(np.array(c["k_new"], np_dtype).reshape(c["new_shape"]))
+    vn = arena.from_numpy(np.array(c["v_new"], np_dtype).reshape(c["new_shape"]))
+    backend.kv_cache_append_at(k, v, c["cache_pos"], kn, vn)
+    assert np.array_equal(k.read().ravel(), np.array(c["expect_k"], np_dtype))
+    assert np.array_equal(v.read().ravel(), np.array(c["expect_v"], np_dtype))
+    c = g["positions"]
+    k = arena.from_numpy(np.zeros(c["cache_shape"], np_dtype))
+    v = arena.from_numpy(np.zeros(c["cache_shape"], np_dtype))
+    kn = arena.from_numpy(np.array(c["k_new"], np_dtype).reshape(c["new_shape"]))
+    vn = arena.from_numpy(np.array(c["v_new"], np_dtype).reshape(c["new_shape"]))
+    pos = arena.from_numpy(np.array(c["cache_pos"], np.int32))
+    backend.kv_cache_append_positions(k, v, pos, kn, vn)
+    assert np.array_equal(k.read().ravel(), np.array(c["expect_k"], np_dtype))
+    assert np.array_equal(v.read().ravel(), np.array(c["expect_v"], np_dtype))
+    c = g["packed"]
+    k = arena.from_numpy(np.zeros(c["cache_shape"], np_dtype))
+    v = arena.from_numpy(np.zeros(c["cache_shape"], np_dtype))
+    kn = arena.from_numpy(np.array(c["k_new"], np_dtype).reshape(c["new_shape"]))
+    vn = arena.from_numpy(np.array(c["v_new"], np_dtype).reshape(c["new_shape"]))
+    pos = arena.from_numpy(np.array(c["cache_pos"], np.int32))
+    cu = arena.from_numpy(np.array(c["cu_seqlens"], np.int32))
+    backend.kv_cache_append_packed(k, v, pos, cu, kn, vn)
+    assert np.array_equal(k.read().ravel(), np.array(c["expect_k"], np_dtype))
+    assert np.array_equal(v.read().ravel(), np.array(c["expect_v"], np_dtype))
+
+
+def test_append_positions_bit_exact_with_skips(backend, arena, oracle):
+    B, Tmax, H, D = 32, 300, 8, 64
+    k0, v0 = oracle.normal_f16((B, Tmax, H, D), 11), oracle.normal_f16((B, Tmax, H, D), 12)
+    kn, vn = oracle.normal_f16((B, 1, H, D), 13), oracle.normal_f16((B, 1, H, D), 14)
+    pos = oracle.uniform_i32(B, 15, 0, Tmax - 1)
+    pos[3], pos[7], pos[9] = -1, Tmax, Tmax - 1  # skipped, skipped, last valid slot
+    k, v = arena.from_numpy(k0), arena.from_numpy(v0)
+    backend.kv_cache_append_positions(k, v, arena.from_numpy(pos), arena.from_numpy(kn), arena.from_numpy(vn))
+    wk, wv = k0.copy(), v0.copy()
+    oracle.kv_cache_append(wk, wv, kn, vn, pos)
+    assert np.array_equal(_bits(k.read()), _bits(wk)) and np.array_equal(_bits(v.read()), _bits(wv))
+
+
+@pytest.mark.parametrize("D,tnew", [(64, 3), (6, 2), (5, 1)])  # 16-, 4- and 1-byte copy units
+def test_append_copy_units_and_multi_token(backend, arena, oracle, D, tnew):
+    B, Tmax, H = 3, 9, 2
+    k0, v0 = oracle.normal_f16((B, Tmax, H, D), 21), oracle.normal_f16((B, Tmax, H, D), 22)
+    kn, vn = oracle.normal_f16((B, tnew, H, D), 23), oracle.normal_f16((B, tnew, H, D), 24)
+    pos = np.array([0, 4, Tmax - tnew], np.int32)
+    k, v = arena.from_numpy(k0), arena.from_numpy(v0)
+    backend.kv_cache_append_positions(k, v, arena.from_numpy(pos), arena.from_numpy(kn), arena.from_numpy(vn))
+    wk, wv = k0.copy(), v0.copy()
+    oracle.kv_cache_append(wk, wv, kn, vn, pos)
+    assert np.array_equal(_bits(k.read()), _bits(wk)) and np.array_equal(_bits(v.read()), _bits(wv))
+
+
+def test_append_packed_bit_exact_with_skips(backend, arena, oracle):
+    B, Tmax, H, D = 6, 40, 4, 32
+    lens = np.array([7, 0, 40, 13, 5, 9], np.int32)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    pos = np.array([0, 3, 0, 30, -2, 31], np.int32)  # seq 3 overflows (30+13), seq 4 negative, seq 5 fits exactly
+    N = int(cu[-1]) + 3
+    k0, v0 = oracle.normal_f16((B, Tmax, H, D), 31), oracle.normal_f16((B, Tmax, H, D), 32)
+    kn, vn = oracle.normal_f16((N, H, D), 33), oracle.normal_f16((N, H, D), 34)
+    k, v = arena.from_numpy(k0), arena.from_numpy(v0)
+    backend.kv_cache_append_packed(k, v, arena.from_numpy(pos), arena.from_numpy(cu), arena.from_numpy(kn),
+                                   arena.from_numpy(vn))
+    wk, wv = k0.copy(), v0.copy()
+    oracle.kv_cache_append_packed(wk, wv, kn, vn, pos, cu)
+    assert np.array_equal(_bits(k.read()), _bits(wk)) and np.array_equal(_bits(v.read()), _bits(wv))
+
+
+def test_append_rejects_bad_arguments(backend, arena, gda):
+    k = arena.alloc((2, 5, 1, 8), gda.F16)
+    v = arena.alloc((2, 5, 1, 8), gda.F16)
+    kn = arena.alloc((2, 2, 1, 8), gda.F16)
+    vn = arena.alloc((2, 2, 1, 8), gda.F16)
+    bad_d = arena.alloc((2, 2, 1, 4), gda.F16)
+    for cache_pos in (-1, 4, 6):  # negative, span passes Tmax, beyond Tmax
+        a = gda.KvAppendArgs(cache_pos)
+        st = backend.call("gd_backend_kv_cache_append_at", k.view(), v.view(), kn.view(), vn.view(), C.byref(a))
+        assert st == gda.INVALID_ARGUMENT
+    a = gda.KvAppendArgs(0)
+    assert backend.call("gd_backend_kv_cache_append_at", k.view(), v.view(), bad_d.view(), bad_d.view(),
+                        C.byref(a)) == gda.INVALID_ARGUMENT
+    pos3 = arena.alloc((3,), gda.I32)
+    assert backend.call("gd_backend_kv_cache_append_positions", k.view(), v.view(), pos3.view(), kn.view(),
+                        vn.view(), C.byref(a)) == gda.INVALID_ARGUMENT
+
+
+# ---- A2 sdpa_decode -------------------------------------------------------------------------
+
+def test_decode_reference_test_case(backend, arena, oracle):
+    """tests/test_sdpa_varlen.c:679-719 of the reference: Tq=2, GQA 2:1, Dh=4, rank-0 position tensor."""
+    c = _golden("reference_test_cases.json")["sdpa_decode_test_decode"]
+    B, Tq, Tmax, Hq, Hkv, D = (c[x] for x in ("B", "Tq", "Tmax", "Hq", "Hkv", "Dh"))
+    q = oracle.fill_tokens(B * Tq * Hq * D, c["q_base"]).reshape(B, Tq, Hq, D)
+    k = oracle.fill_tokens(B * Tmax * Hkv * D, c["k_base"]).reshape(B, Tmax, Hkv, D)
+    v = oracle.fill_tokens(B * Tmax * Hkv * D, c["v_base"]).reshape(B, Tmax, Hkv, D)
+    tq, tk, tv = arena.from_numpy(q), arena.from_numpy(k), arena.from_numpy(v)
+    pos = arena.from_numpy(np.array([c["cache_pos"]], np.int32))
+    out = arena.from_numpy(np.zeros(q.shape, np.float16))
+    backend.sdpa_decode(tq, tk, tv, pos, out, c["scale"])
+    want = oracle.sdpa_decode(q, k, v, [c["cache_pos"]], c["scale"])
+    assert np.abs(out.read().astype(np.float32) - want).max() < c["tol_abs"]
+
+
+def test_decode_positions_equals_scalar_f32(backend, arena, oracle, gda):
+    """tests/test_kv_cache_decode.c:181-303 of the reference: three position forms agree (F32 tensors)."""
+    c = _golden("reference_test_cases.json")["sdpa_decode_positions_vs_scalar"]
+    qs, ks = c["q_shape"], c["kv_shape"]
+    i = np.arange(int(np.prod(qs)), dtype=np.float32)
+    q = ((i - 7.0) * 0.03).astype(np.float32).reshape(qs)
+    j = np.arange(int(np.prod(ks)), dtype=np.float32)
+    k = ((j - 11.0) * 0.02).astype(np.float32).reshape(ks)
+    v = ((j + 3.0) * -0.015).astype(np.float32).reshape(ks)
+    tq, tk, tv = arena.from_numpy(q), arena.from_numpy(k), arena.from_numpy(v)
+    pos = arena.from_numpy(np.array(c["cache_pos"], np.int32))
+    out = arena.from_numpy(np.zeros(qs, np.float32))
+    backend.sdpa_decode_positions(tq, tk, tv, pos, out, c["scale"])
+    got = out.read()
+    for b in range(qs[0]):
+        ob = arena.from_numpy(np.zeros([1] + qs[1:], np.float32))
+        backend.sdpa_decode_at(tq.rows(b, 1), tk.rows(b, 1), tv.rows(b, 1), c["cache_pos"][b], ob, c["scale"])
+        assert np.abs(ob.read()[0] - got[b]).max() < c["tol_abs"]
+        p0 = arena.from_numpy(np.array([c["cache_pos"][b]], np.int32))
+        ot = arena.from_numpy(np.zeros([1] + qs[1:], np.float32))
+        backend.sdpa_decode(tq.rows(b, 1), tk.rows(b, 1), tv.rows(b, 1), p0, ot, c["scale"])
+        assert np.abs(ot.read()[0] - got[b]).max() < c["tol_abs"]
+    _close(got, oracle.sdpa_decode(q, k, v, c["cache_pos"], c["scale"]), 1e-5, 1e-6)
+
+
+def _decode_case(backend, arena, oracle, B, H, Hkv, D, Tmax, pos, scale, window=0, seed=100, chunk=0):
+    q = oracle.normal_f16((B, 1, H, D), seed)
+    k = oracle.normal_f16((B, Tmax, Hkv, D), seed + 1)
+    v = oracle.normal_f16((B, Tmax, Hkv, D), seed + 2)
+    sentinel = np.full(q.shape, 7.0, np.float16)
+    tq, tk, tv = arena.from_numpy(q), arena.from_numpy(k), arena.from_numpy(v)
+    tp, out = arena.from_numpy(np.asarray(pos, np.int32)), arena.from_numpy(sentinel)
+    backend.set_tunable("sdpa_chunk", chunk)
+    try:
+        backend.sdpa_decode_positions(tq, tk, tv, tp, out, scale, window)
+    finally:
+        backend.set_tunable("sdpa_chunk", 0)
+    want = oracle.sdpa_decode(q, k, v, pos, scale, window, out_init=sentinel.astype(np.float32))
+    _close(out.read(), want)
+    return out.read()
+
+
+@pytest.mark.parametrize("chunk", [0, 64, 1024])
+def test_decode_isolated_config_shape(backend, arena, oracle, chunk):
+    """BASELINE config 1 at a length the oracle finishes in seconds: B=32, H=8, DH=64, ragged lengths,
+    append one token then decode over L+1 keys, scale 1/8."""
+    B, H, D, Tmax = 32, 8, 64, 1025
+    L = oracle.uniform_i32(B, 1001, 1, Tmax - 1)
+    k0, v0 = oracle.normal_f16((B, Tmax, H, D), 1002), oracle.normal_f16((B, Tmax, H, D), 1003)
+    q, kn, vn = (oracle.normal_f16((B, 1, H, D), s) for s in (1004, 1005, 1006))
+    tk, tv, tp = arena.from_numpy(k0), arena.from_numpy(v0), arena.from_numpy(L)
+    backend.kv_cache_append_positions(tk, tv, tp, arena.from_numpy(kn), arena.from_numpy(vn))
+    wk, wv = k0.copy(), v0.copy()
+    oracle.kv_cache_append(wk, wv, kn, vn, L)
+    assert np.array_equal(_bits(tk.read()), _bits(wk)) and np.array_equal(_bits(tv.read()), _bits(wv))
+    out = arena.alloc(q.shape, 1)
+    backend.set_tunable("sdpa_chunk", chunk)
+    try:
+        backend.sdpa_decode_positions(arena.from_numpy(q), tk, tv, tp, out, 0.125)
+    finally:
+        backend.set_tunable("sdpa_chunk", 0)
+    _close(out.read(), oracle.sdpa_decode(q, wk, wv, L, 0.125))
+
+
+@pytest.mark.parametrize("H,Hkv,D", [(8, 8, 64), (16, 16, 128), (8, 2, 64), (8, 1, 128), (6, 3, 64), (6, 2, 64)])
+def test_decode_head_layouts(backend, arena, oracle, H, Hkv, D):
+    pos = np.array([0, 1, 63, 64, 200, 299, -1, 31], np.int32)
+    _decode_case(backend, arena, oracle, 8, H, Hkv, D, 300, pos, 1.0 / np.sqrt(D), seed=200 + H + D, chunk=96)
+
+
+@pytest.mark.parametrize("window", [1, 7, 256, 1000])
+def test_decode_sliding_window(backend, arena, oracle, window):
+    pos = np.array([0, 5, 255, 256, 257, 511, 400, 100], np.int32)
+    _decode_case(backend, arena, oracle, 8, 8, 8, 64, 512, pos, 0.125, window, seed=300 + window, chunk=64)
+
+
+def test_decode_position_past_cache_end_clamps(backend, arena, oracle):
+    _decode_case(backend, arena, oracle, 2, 4, 4, 64, 40, np.array([40, 100], np.int32), 0.125, seed=400)
+
+
+def test_decode_generic_paths(backend, arena, oracle):
+    """prefix masks, Tq > 1 and odd head sizes take the generic kernel."""
+    rng_seed = 500
+    for (Tq, D, window, prefix) in [(1, 64, 0, 3), (1, 64, 4, 2), (3, 64, 0, 0), (2, 40, 5, 0), (1, 72, 0, 0)]:
+        B, H, Hkv, Tmax = 3, 4, 2, 70
+        q = oracle.normal_f16((B, Tq, H, D), rng_seed)
+        k = oracle.normal_f16((B, Tmax, Hkv, D), rng_seed + 1)
+        v = oracle.normal_f16((B, Tmax, Hkv, D), rng_seed + 2)
+        pos = np.array([0, 33, 66], np.int32)
+        out = arena.from_numpy(np.zeros(q.shape, np.float16))
+        backend.sdpa_decode_positions(arena.from_numpy(q), arena.from_numpy(k), arena.from_numpy(v),
+                                      arena.from_numpy(pos), out, 0.2, window, prefix)
+        _close(out.read(), oracle.sdpa_decode(q, k, v, pos, 0.2, window, prefix))
+        rng_seed += 10
+
+
+def test_decode_closed_forms(backend, arena, oracle):
+    B, H, D, Tmax = 4, 8, 64, 130
+    q = oracle.normal_f16((B, 1, H, D), 600)
+    v = oracle.normal_f16((B, Tmax, H, D), 601)
+    k = np.broadcast_to(oracle.normal_f16((1, 1, H, D), 602), (B, Tmax, H, D)).copy()
+    pos = np.array([129, 64, 0, 17], np.int32)
+    out = arena.alloc(q.shape, 1)
+    backend.sdpa_decode_positions(arena.from_numpy(q), arena.from_numpy(k), arena.from_numpy(v),
+                                  arena.from_numpy(pos), out, 0.125)
+    got = out.read().astype(np.float64)
+    for b in range(B):  # equal keys -> mean of the visible values; one key -> that value
+        _close(got[b, 0], v[b, : pos[b] + 1].astype(np.float64).mean(0))
+    assert np.array_equal(_bits(out.read()[2, 0]), _bits(v[2, 0]))
+
+
+def test_decode_rejects_bad_arguments(backend, arena, gda):
+    q = arena.alloc((2, 1, 4, 64), gda.F16)
+    k = arena.alloc((2, 16, 2, 64), gda.F16)
+    out = arena.alloc((2, 1, 4, 64), gda.F16)
+    pos = arena.alloc((2,), gda.I32)
+    a = gda.SdpaDecodeArgs(0.125, 0, 0, 0)
+    ok = backend.call("gd_backend_sdpa_decode_positions", q.view(), k.view(), k.view(), pos.view(), out.view(), C.byref(a))
+    assert ok == gda.GD_OK
+    bad_scale = gda.SdpaDecodeArgs(0.0, 0, 0, 0)
+    assert backend.call("gd_backend_sdpa_decode_positions", q.view(), k.view(), k.view(), pos.view(), out.view(),
+                        C.byref(bad_scale)) == gda.INVALID_ARGUMENT
+    bad_prefix = gda.SdpaDecodeArgs(0.125, 0, 17, 0)
+    assert backend.call("gd_backend_sdpa_decode_positions", q.view(), k.view(), k.view(), pos.view(), out.view(),
+                        C.byref(bad_prefix)) == gda.INVALID_ARGUMENT
+    k3 = arena.alloc((2, 16, 3, 64), gda.F16)  # 4 query heads over 3 kv heads
+    assert backend.call("gd_backend_sdpa_decode_positions", q.view(), k3.view(), k3.view(), pos.view(), out.view(),
+                        C.byref(a)) == gda.INVALID_ARGUMENT
+    at = gda.SdpaDecodeArgs(0.125, 0, 0, 16)  # Tq does not fit after position 16
+    assert backend.call("gd_backend_sdpa_decode_at", q.view(), k.view(), k.view(), out.view(), C.byref(at)) == gda.INVALID_ARGUMENT
+
+
+# ---- A11 sdpa_varlen ----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("H,Hkv,D,window,prefix", [(4, 4, 64, 0, 0), (4, 2, 128, 0, 0), (4, 4, 64, 5, 0), (2, 1, 32, 3, 4)])
+def test_varlen_matches_oracle(backend, arena, oracle, H, Hkv, D, window, prefix):
+    lens = np.array([70, 1, 0, 129, 33], np.int32)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    N = int(cu[-1])
+    q, k, v = oracle.normal_f16((N, H, D), 700), oracle.normal_f16((N, Hkv, D), 701), oracle.normal_f16((N, Hkv, D), 702)
+    out = arena.from_numpy(np.zeros(q.shape, np.float16))
+    backend.sdpa_varlen(arena.from_numpy(q), arena.from_numpy(k), arena.from_numpy(v), arena.from_numpy(cu), out,
+                        0.15, True, window, prefix, 256)
+    _close(out.read(), oracle.sdpa_varlen(q, k, v, cu, 0.15, True, window, prefix, 256))
+
+
+def test_varlen_max_seqlen_truncates(backend, arena, oracle):
+    cu = np.array([0, 50, 60], np.int32)
+    q, k, v = (oracle.normal_f16((60, 2, 64), s) for s in (710, 711, 712))
+    out = arena.from_numpy(np.full(q.shape, 3.0, np.float16))
+    backend.sdpa_varlen(arena.from_numpy(q), arena.from_numpy(k), arena.from_numpy(v), arena.from_numpy(cu), out,
+                        0.125, True, 0, 0, 32)
+    got = out.read()
+    _close(got, oracle.sdpa_varlen(q, k, v, cu, 0.125, True, 0, 0, 32))
+    assert np.all(got[32:50] == 0)
+
+
+# ---- A3 rms_norm ---------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("rows,cols", [(64, 512), (16, 2048), (3, 100), (1, 8200), (5, 7)])
+def test_rms_norm_f16(backend, arena, oracle, rows, cols):
+    x = oracle.normal_f16((rows, cols), 800 + cols, 1.5)
+    w = (1.0 + 0.1 * oracle.normal_f16((cols,), 801).astype(np.float32)).astype(np.float16)
+    out = arena.alloc((rows, cols), 1)
+    backend.rms_norm_forward(arena.from_numpy(x), arena.from_numpy(w), out, 1e-5)
+    _close(out.read(), oracle.rms_norm(x, w, 1e-5))
+
+
+def test_rms_norm_f32_reference_case(backend, arena, oracle, gda):
+    c = _golden("reference_test_cases.json")["rms_norm_f32_2x4"]
+    x = np.array(c["x"], np.float32).reshape(2, 4)
+    w = np.array(c["w"], np.float32)
+    out = arena.alloc((2, 4), gda.F32)
+    backend.rms_norm_forward(arena.from_numpy(x), arena.from_numpy(w), out, c["eps"])
+    assert np.abs(out.read() - oracle.rms_norm(x, w, c["eps"])).max() < c["tol_abs"]
+    a = gda.RmsNormArgs(rows=2, cols=4, eps=0.0)
+    assert backend.call("gd_backend_rms_norm_forward", out.view(), arena.from_numpy(w).view(), out.view(),
+                        C.byref(a)) == gda.INVALID_ARGUMENT
+
+
+# ---- A4 qkv_split_rope -------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("N,H,D,interleaved", [(64, 8, 64, False), (16, 16, 128, False), (5, 3, 24, False),
+                                               (7, 2, 64, True), (4, 2, 6, True)])
+def test_qkv_split_rope(backend, arena, oracle, N, H, D, interleaved):
+    qkv = oracle.normal_f16((N, 3 * H * D), 900 + D)
+    pos = oracle.uniform_i32(N, 901, 0, 4095)
+    pos[0] = 0
+    q, k, v = (arena.alloc((N, H, D), 1) for _ in range(3))
+    backend.qkv_split_rope_forward(arena.from_numpy(qkv), arena.from_numpy(pos), q, k, v, H, D, 10000.0, interleaved)
+    wq, wk, wv = oracle.qkv_split_rope(qkv, pos, H, D, 10000.0, interleaved)
+    assert np.array_equal(_bits(v.read()), _bits(wv))  # v and the index map: bit-exact
+    _close(q.read(), wq)
+    _close(k.read(), wk)
+    # position 0 is the identity, bit for bit
+    src = qkv.reshape(N, 3, H, D)
+    assert np.array_equal(_bits(q.read()[0]), _bits(src[0, 0])) and np.array_equal(_bits(k.read()[0]), _bits(src[0, 1]))
+
+
+def test_qkv_split_rope_rejects_partial_rotation(backend, arena, gda):
+    qkv = arena.alloc((2, 3 * 2 * 8), gda.F16)
+    pos = arena.alloc((2,), gda.I32)
+    o = arena.alloc((2, 2, 8), gda.F16)
+    a = gda.RopeArgs(10000.0, 4, 0)  # n_dims != head_dim
+    assert backend.call("gd_backend_qkv_split_rope_forward", qkv.view(), pos.view(), o.view(), o.view(), o.view(),
+                        2, 8, C.byref(a)) == gda.INVALID_ARGUMENT
+
+
+# ---- A5/A6/A7 projections ------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("M,K,N", [(64, 512, 1536), (1, 512, 2048), (16, 2048, 96), (33, 136, 50), (64, 1536, 512),
+                                   (130, 64, 48), (3, 20, 7)])
+def test_linear_nt_and_bias_roundings(backend, arena, oracle, M, K, N):
+    x = oracle.normal_f16((M, K), 1000 + K, 1.0)
+    w = oracle.normal_f16((N, K), 1001 + N, 0.05)
+    bias = oracle.normal_f16((N,), 1002, 0.5)
+    tx, tw, tb = arena.from_numpy(x), arena.from_numpy(w), arena.from_numpy(bias)
+    y = arena.alloc((M, N), 1)
+    backend.matmul_nt(tx, tw, y)
+    _close(y.read(), oracle.linear_nt(x, w))
+    backend.linear_nt(tx, tw, tb, y)
+    _close(y.read(), oracle.linear_nt(x, w, bias))
+
+
+@pytest.mark.parametrize("M,K,N", [(64, 1536, 512), (16, 352, 2048), (1, 64, 40), (70, 24, 33), (2, 9, 5)])
+def test_linear_kn_and_swiglu_fusion(backend, arena, oracle, M, K, N):
+    x = oracle.normal_f16((M, K), 1100 + K, 1.0)
+    w = oracle.normal_f16((K, N), 1101 + N, 0.05)
+    bias = oracle.normal_f16((N,), 1102, 0.5)
+    tx, tw, tb = arena.from_numpy(x), arena.from_numpy(w), arena.from_numpy(bias)
+    y = arena.alloc((M, N), 1)
+    backend.matmul(tx, tw, y)
+    _close(y.read(), oracle.linear(x, w))
+    backend.linear(tx, tw, tb, y)
+    _close(y.read(), oracle.linear(x, w, bias))
+    x12 = oracle.normal_f16((M, 2 * K), 1103, 1.0)
+    backend.swiglu_split_linear(arena.from_numpy(x12), tw, tb, y)
+    _close(y.read(), oracle.swiglu_split_linear(x12, w, bias))
+    backend.swiglu_split_linear(arena.from_numpy(x12), tw, None, y)
+    _close(y.read(), oracle.swiglu_split_linear(x12, w))
+
+
+def test_linear_reference_fill_values_and_strided_rows(backend, arena, oracle):
+    """Inputs of the reference's tests/test_linear.c (fill_values) and a row-strided x view."""
+    c = _golden("reference_test_cases.json")["linear_f16"]
+    M, K, N = 4, 16, 8
+    x = oracle.fill_values(M * K, 0.01, -0.1).astype(np.float16).reshape(M, K)
+    w = oracle.fill_values(K * N, 0.02, -0.3).astype(np.float16).reshape(K, N)
+    b = oracle.fill_values(N, 0.05, -0.5).astype(np.float16)
+    y = arena.alloc((M, N), 1)
+    backend.linear(arena.from_numpy(x), arena.from_numpy(w), arena.from_numpy(b), y)
+    want = x.astype(np.float64) @ w.astype(np.float64) + b.astype(np.float64)
+    assert np.abs(y.read().astype(np.float64) - want).max() < c["tol_abs"]
+    wide = oracle.normal_f16((M, 2 * K), 1200)
+    tw = arena.from_numpy(wide)
+    import ctypes
+    xm = tw.matrix(rows=M, cols=K, row_elems=2 * K)  # left half of every row
+    st = backend.call("gd_backend_matmul", ctypes.byref(xm), arena.from_numpy(w).matrix(), y.matrix())
+    assert st == 0
+    _close(y.read(), oracle.linear(wide[:, :K], w))
+
+
+def test_linear_rejects_bad_arguments(backend, arena, gda):
+    x = arena.alloc((4, 16), gda.F16)
+    w = arena.alloc((16, 8), gda.F16)
+    y = arena.alloc((4, 8), gda.F16)
+    bad_w = arena.alloc((15, 8), gda.F16)
+    f32 = arena.alloc((4, 16), gda.F32)
+    assert backend.call("gd_backend_matmul", x.matrix(), bad_w.matrix(), y.matrix()) == gda.INVALID_ARGUMENT
+    assert backend.call("gd_backend_matmul", f32.matrix(), w.matrix(), y.matrix()) == gda.UNSUPPORTED
+    assert backend.call("gd_backend_matmul_nt", x.matrix(), w.matrix(), y.matrix()) == gda.INVALID_ARGUMENT
+
+
+# ---- A8 add, swiglu_split, A9 embedding, A10 argmax, gather ----------------------------------------------------
+
+def test_add_residual_bias_and_broadcast(backend, arena, oracle):
+    a = oracle.normal_f16((64, 512), 1300, 30.0)
+    b = oracle.normal_f16((64, 512), 1301, 0.3)
+    out = arena.alloc((64, 512), 1)
+    backend.add(arena.from_numpy(a), arena.from_numpy(b), out)
+    assert np.array_equal(_bits(out.read()), _bits(a + b))
+    bias = oracle.normal_f16((512,), 1302)
+    backend.add(arena.from_numpy(a), arena.from_numpy(bias), out)
+    assert np.array_equal(_bits(out.read()), _bits(a + bias))
+    backend.add(arena.from_numpy(bias), arena.from_numpy(a), out)
+    assert np.array_equal(_bits(out.read()), _bits(a + bias))
+    x = oracle.normal_f16((3, 1, 5), 1303)
+    y = oracle.normal_f16((4, 1), 1304)
+    o = arena.alloc((3, 4, 5), 1)
+    backend.add(arena.from_numpy(x), arena.from_numpy(y), o)
+    assert np.array_equal(_bits(o.read()), _bits(x + y))
+    odd = oracle.normal_f16((7, 3), 1305)
+    o2 = arena.alloc((7, 3), 1)
+    backend.add(arena.from_numpy(odd), arena.from_numpy(odd), o2)
+    assert np.array_equal(_bits(o2.read()), _bits(odd + odd))
+
+
+def test_add_rejects_incompatible_shapes(backend, arena, gda):
+    x, y, o = arena.alloc((4, 6), gda.F16), arena.alloc((5,), gda.F16), arena.alloc((4, 6), gda.F16)
+    assert backend.call("gd_backend_add", x.view(), y.view(), o.view()) == gda.INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("rows,H", [(64, 1536), (3, 4), (2, 8), (5, 13)])
+def test_swiglu_split(backend, arena, oracle, rows, H):
+    x12 = oracle.normal_f16((rows, 2 * H), 1400 + H, 2.0)
+    out = arena.alloc((rows, H), 1)
+    backend.swiglu_split_forward(arena.from_numpy(x12), out)
+    _close(out.read(), oracle.swiglu_split(x12))
+
+
+def test_embedding_bit_exact_and_nan_rows(backend, arena, oracle, gda):
+    table = oracle.normal_f16((2048, 512), 1500, 0.02)
+    ids = oracle.uniform_i32(64, 1501, 0, 2047)
+    ids[5], ids[9] = -1, 2048
+    out = arena.alloc((64, 512), 1)
+    backend.embedding_forward(arena.from_numpy(table), arena.from_numpy(ids), out)
+    assert np.array_equal(_bits(out.read()), _bits(oracle.embedding(table, ids)))
+    t32 = oracle.fill_normal(10 * 3, 1502, 1.0).reshape(10, 3)
+    ids = np.array([9, 0, 11], np.int32)
+    o32 = arena.alloc((3, 3), gda.F32)
+    backend.embedding_forward(arena.from_numpy(t32), arena.from_numpy(ids), o32)
+    got = o32.read()
+    assert np.array_equal(got[:2], t32[[9, 0]]) and np.all(np.isnan(got[2]))
+
+
+def test_argmax_rows(backend, arena, oracle, gda):
+    logits = oracle.normal_f16((64, 2048), 1600, 3.0)
+    logits[1, 100] = logits[1, 1900] = np.float16(60.0)  # tie -> lowest index
+    logits[2, :] = np.nan
+    logits[3, 7] = np.inf
+    logits[4, :] = -np.inf
+    logits[4, 2047] = np.float16(-5.0)
+    ids, gap = arena.alloc((64,), gda.I32), arena.alloc((64,), gda.F32)
+    backend.argmax_rows(arena.from_numpy(logits), ids, gap)
+    want_ids, want_gap = oracle.argmax_rows(logits)
+    assert np.array_equal(ids.read(), want_ids)
+    assert np.array_equal(gap.read(), want_gap)
+    wide = oracle.normal_f16((16, 32768), 1601, 3.0)
+    ids2 = arena.alloc((16,), gda.I32)
+    backend.argmax_rows(arena.from_numpy(wide), ids2)
+    assert np.array_equal(ids2.read(), oracle.argmax_rows(wide)[0])
+
+
+def test_gather_rows_and_position_increment(backend, arena, oracle, gda):
+    src = oracle.normal_f16((100, 512), 1700)
+    rows = np.array([99, 0, 42, 42, 100], np.int32)  # last one is out of range: row untouched
+    out = arena.from_numpy(np.full((5, 512), 9.0, np.float16))
+    backend.gather_rows(arena.from_numpy(src), arena.from_numpy(rows), out)
+    got = out.read()
+    assert np.array_equal(_bits(got[:4]), _bits(src[[99, 0, 42, 42]])) and np.all(got[4] == 9.0)
+    p = arena.from_numpy(np.arange(64, dtype=np.int32))
+    backend.add_scalar_i32(p, p, 1)
+    assert np.array_equal(p.read(), np.arange(1, 65))
