@@ -124,6 +124,7 @@ _SIGNATURES = {
     "gd_backend_linear_nt": [_vp, _MV, _MV, _VV, _MV],
     "gd_backend_gather_rows": [_vp, _TV, _TV, _TV],
     "gd_backend_add_scalar_i32": [_vp, _TV, _TV, C.c_int32],
+    "gd_backend_decode_advance": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, _TV],
     "gd_backend_copy": [_vp, _vp, C.c_size_t, _vp, C.c_size_t, C.c_size_t],
     "gd_backend_timer_create": [_vp, C.POINTER(_vp)],
     "gd_backend_timer_start": [_vp],

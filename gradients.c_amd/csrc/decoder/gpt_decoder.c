@@ -1,0 +1,487 @@
+/*
+ * Decoder-only language model of the reference's example, inference part, with run-time
+ * dimensions.  The operator order, residual wiring and cache bookkeeping restate
+ * examples/gpt_lm/gpt_lm_shared.c of the reference: gpt_block_decode_cached (:961-1071),
+ * gpt_lm_decode_logits (:1204-1246), gpt_block_prefill_cached (:825-959),
+ * gpt_lm_prefill_last_logits (:1174-1202), gpt_kv_cache_init (:480-538) and the weight
+ * initialisation (:196-218, 290-402).  Everything goes through the public gd_* operators.
+ */
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "gd_gpt_decoder.h"
+
+#define TRY(expr)                       \
+    do {                                \
+        gd_status st__ = (expr);        \
+        if (st__ != GD_OK) return st__; \
+    } while (0)
+
+typedef struct gpt_linear {
+    gd_tensor weight, bias;
+    bool transposed; /* weight stored [out, in] */
+} gpt_linear;
+
+typedef struct gpt_block {
+    gd_tensor attn_norm_w, mlp_norm_w;
+    gpt_linear qkv_proj, attn_proj, up_gate, down_proj;
+} gpt_block;
+
+struct gd_gpt_decoder {
+    gd_context *ctx;
+    gd_gpt_config cfg;
+    gd_tensor token_embedding, lm_head, lm_head_bias, final_norm_w;
+    gpt_block *blocks;
+    gd_tensor *k_cache, *v_cache;
+    int32_t *pos; /* host copy of the live lengths */
+    /* device-resident decode state (state arena) */
+    gd_tensor ids_dev, pos_dev, step_dev;
+};
+
+/* ---- deterministic initialisation (reference :32-48, 196-218) ----------------------- */
+
+static uint64_t mix64(uint64_t x)
+{
+    x = (x ^ (x >> 30)) * UINT64_C(0xbf58476d1ce4e5b9);
+    x = (x ^ (x >> 27)) * UINT64_C(0x94d049bb133111eb);
+    return x ^ (x >> 31);
+}
+
+static uint64_t splitmix64(uint64_t x) { return mix64(x + UINT64_C(0x9e3779b97f4a7c15)); }
+
+static double uniform_open_closed(uint64_t *state)
+{
+    *state += UINT64_C(0x9e3779b97f4a7c15);
+    return ((double)(mix64(*state) >> 11) + 1.0) * (1.0 / 9007199254740992.0);
+}
+
+static gd_status init_normal(gd_context *ctx, gd_tensor *t, uint64_t seed, float stddev)
+{
+    int64_t n;
+    float *values;
+    uint64_t state = seed;
+    size_t i = 0U;
+    gd_status st;
+    TRY(gd_tensor_numel(t, &n));
+    values = (float *)malloc((size_t)n * sizeof(float));
+    if (values == NULL) return GD_ERR_OUT_OF_MEMORY;
+    while (i < (size_t)n) {
+        const double u1 = uniform_open_closed(&state), u2 = uniform_open_closed(&state);
+        const double radius = sqrt(-2.0 * log(u1)), angle = 6.283185307179586476925286766559 * u2;
+        values[i++] = (float)(radius * cos(angle) * (double)stddev);
+        if (i < (size_t)n) values[i++] = (float)(radius * sin(angle) * (double)stddev);
+    }
+    st = gd_tensor_write_f32(ctx, t, values, (size_t)n);
+    free(values);
+    return st;
+}
+
+static gd_status param(gd_context *ctx, gd_dtype dtype, uint32_t rank, int64_t d0, int64_t d1, gd_tensor *out)
+{
+    int64_t dims[2] = {d0, d1};
+    return gd_tensor_empty(ctx, GD_ARENA_PARAMS, dtype, gd_shape_make(rank, dims), 256U, out);
+}
+
+static gd_status linear_init(gd_context *ctx, gpt_linear *l, int64_t in, int64_t out, bool transposed, uint64_t seed,
+                             float stddev)
+{
+    l->transposed = transposed;
+    TRY(param(ctx, GD_DTYPE_F16, 2U, transposed ? out : in, transposed ? in : out, &l->weight));
+    TRY(init_normal(ctx, &l->weight, seed, stddev));
+    TRY(param(ctx, GD_DTYPE_F16, 1U, out, 0, &l->bias));
+    return gd_tensor_zero_(ctx, &l->bias);
+}
+
+static gd_status ones_param(gd_context *ctx, int64_t n, gd_tensor *out)
+{
+    int64_t dims[1] = {n};
+    return gd_tensor_ones(ctx, GD_ARENA_PARAMS, GD_DTYPE_F16, gd_shape_make(1U, dims), 256U, out);
+}
+
+static size_t pad256(size_t n) { return (n + 255U) & ~(size_t)255U; }
+
+size_t gd_gpt_params_bytes(const gd_gpt_config *c)
+{
+    const size_t Dm = (size_t)c->d_model, Hm = (size_t)c->mlp_hidden, V = (size_t)c->vocab;
+    size_t per_layer = 2U * pad256(Dm * 2U) + pad256(3U * Dm * Dm * 2U) + pad256(3U * Dm * 2U) + pad256(Dm * Dm * 2U) +
+                       pad256(Dm * 2U) + pad256(2U * Hm * Dm * 2U) + pad256(2U * Hm * 2U) + pad256(Hm * Dm * 2U) +
+                       pad256(Dm * 2U);
+    size_t total = pad256(V * Dm * 2U) * (c->tie_lm_head ? 1U : 2U) + pad256(V * 2U) + pad256(Dm * 2U);
+    return total + per_layer * (size_t)c->n_layers + 4096U;
+}
+
+size_t gd_gpt_state_bytes(const gd_gpt_config *c)
+{
+    const size_t cache = pad256((size_t)c->batch * (size_t)c->max_seq * (size_t)c->n_heads * (size_t)c->head_dim * 2U);
+    return cache * 2U * (size_t)c->n_layers + 3U * pad256((size_t)c->batch * 4U) + 4096U;
+}
+
+gd_status gd_gpt_decoder_create(gd_context *ctx, const gd_gpt_config *cfg, gd_gpt_decoder **out)
+{
+    gd_gpt_decoder *d;
+    const float std = 0.02f;
+    float resid;
+    int32_t l;
+    int64_t cache_dims[4], bdim[1], one[1] = {1};
+    gd_status st = GD_OK;
+    if (out != NULL) *out = NULL;
+    if (ctx == NULL || cfg == NULL || out == NULL || cfg->vocab <= 0 || cfg->d_model <= 0 || cfg->n_layers <= 0 ||
+        cfg->n_heads <= 0 || cfg->head_dim <= 0 || cfg->mlp_hidden <= 0 || cfg->max_seq <= 0 || cfg->batch <= 0 ||
+        cfg->n_heads * cfg->head_dim != cfg->d_model || cfg->sdpa_window < 0)
+        return GD_ERR_INVALID_ARGUMENT;
+    d = (gd_gpt_decoder *)calloc(1, sizeof(*d));
+    if (d == NULL) return GD_ERR_OUT_OF_MEMORY;
+    d->ctx = ctx;
+    d->cfg = *cfg;
+    if (!(d->cfg.rms_eps > 0.0f)) d->cfg.rms_eps = 1.0e-5f;
+    if (!(d->cfg.rope_theta > 0.0f)) d->cfg.rope_theta = 10000.0f;
+    d->blocks = (gpt_block *)calloc((size_t)cfg->n_layers, sizeof(gpt_block));
+    d->k_cache = (gd_tensor *)calloc((size_t)cfg->n_layers, sizeof(gd_tensor));
+    d->v_cache = (gd_tensor *)calloc((size_t)cfg->n_layers, sizeof(gd_tensor));
+    d->pos = (int32_t *)calloc((size_t)cfg->batch, sizeof(int32_t));
+    if (d->blocks == NULL || d->k_cache == NULL || d->v_cache == NULL || d->pos == NULL) {
+        gd_gpt_decoder_destroy(d);
+        return GD_ERR_OUT_OF_MEMORY;
+    }
+    resid = std / sqrtf(2.0f * (float)cfg->n_layers);
+#define STEP(expr) do { if (st == GD_OK) st = (expr); } while (0)
+    STEP(param(ctx, GD_DTYPE_F16, 2U, cfg->vocab, cfg->d_model, &d->token_embedding));
+    STEP(init_normal(ctx, &d->token_embedding, splitmix64(cfg->seed ^ UINT64_C(0xabc001)), std));
+    if (cfg->tie_lm_head) {
+        d->lm_head = d->token_embedding;
+    } else {
+        STEP(param(ctx, GD_DTYPE_F16, 2U, cfg->vocab, cfg->d_model, &d->lm_head));
+        STEP(init_normal(ctx, &d->lm_head, splitmix64(cfg->seed ^ UINT64_C(0xabc002)), std));
+    }
+    STEP(param(ctx, GD_DTYPE_F16, 1U, cfg->vocab, 0, &d->lm_head_bias));
+    STEP(gd_tensor_zero_(ctx, &d->lm_head_bias));
+    STEP(ones_param(ctx, cfg->d_model, &d->final_norm_w));
+    cache_dims[0] = cfg->batch;
+    cache_dims[1] = cfg->max_seq;
+    cache_dims[2] = cfg->n_heads;
+    cache_dims[3] = cfg->head_dim;
+    for (l = 0; l < cfg->n_layers && st == GD_OK; ++l) {
+        gpt_block *b = &d->blocks[l];
+        const uint64_t bs = cfg->seed ^ ((uint64_t)l << 8);
+        STEP(ones_param(ctx, cfg->d_model, &b->attn_norm_w));
+        STEP(ones_param(ctx, cfg->d_model, &b->mlp_norm_w));
+        STEP(linear_init(ctx, &b->qkv_proj, cfg->d_model, 3 * (int64_t)cfg->d_model, true, splitmix64(bs ^ 1U), std));
+        STEP(linear_init(ctx, &b->attn_proj, cfg->d_model, cfg->d_model, true, splitmix64(bs ^ 2U), resid));
+        STEP(linear_init(ctx, &b->up_gate, cfg->d_model, 2 * (int64_t)cfg->mlp_hidden, true, splitmix64(bs ^ 3U), std));
+        STEP(linear_init(ctx, &b->down_proj, cfg->mlp_hidden, cfg->d_model, false, splitmix64(bs ^ 4U), resid));
+        STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_F16, gd_shape_make(4U, cache_dims), 256U, &d->k_cache[l]));
+        STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_F16, gd_shape_make(4U, cache_dims), 256U, &d->v_cache[l]));
+    }
+    bdim[0] = cfg->batch;
+    STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_I32, gd_shape_make(1U, bdim), 256U, &d->ids_dev));
+    STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_I32, gd_shape_make(1U, bdim), 256U, &d->pos_dev));
+    STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_I32, gd_shape_make(1U, one), 256U, &d->step_dev));
+#undef STEP
+    if (st != GD_OK) {
+        gd_gpt_decoder_destroy(d);
+        return st;
+    }
+    *out = d;
+    return GD_OK;
+}
+
+void gd_gpt_decoder_destroy(gd_gpt_decoder *d)
+{
+    if (d == NULL) return;
+    free(d->blocks);
+    free(d->k_cache);
+    free(d->v_cache);
+    free(d->pos);
+    free(d);
+}
+
+gd_tensor *gd_gpt_decoder_tensor(gd_gpt_decoder *d, const char *name, int32_t layer)
+{
+    gpt_block *b;
+    if (d == NULL || name == NULL) return NULL;
+    if (!strcmp(name, "embed")) return &d->token_embedding;
+    if (!strcmp(name, "lm_head")) return &d->lm_head;
+    if (!strcmp(name, "lm_bias")) return &d->lm_head_bias;
+    if (!strcmp(name, "final_norm")) return &d->final_norm_w;
+    if (layer < 0 || layer >= d->cfg.n_layers) return NULL;
+    b = &d->blocks[layer];
+    if (!strcmp(name, "attn_norm")) return &b->attn_norm_w;
+    if (!strcmp(name, "mlp_norm")) return &b->mlp_norm_w;
+    if (!strcmp(name, "w_qkv")) return &b->qkv_proj.weight;
+    if (!strcmp(name, "b_qkv")) return &b->qkv_proj.bias;
+    if (!strcmp(name, "w_attn")) return &b->attn_proj.weight;
+    if (!strcmp(name, "b_attn")) return &b->attn_proj.bias;
+    if (!strcmp(name, "w_upgate")) return &b->up_gate.weight;
+    if (!strcmp(name, "b_upgate")) return &b->up_gate.bias;
+    if (!strcmp(name, "w_down")) return &b->down_proj.weight;
+    if (!strcmp(name, "b_down")) return &b->down_proj.bias;
+    if (!strcmp(name, "k_cache")) return &d->k_cache[layer];
+    if (!strcmp(name, "v_cache")) return &d->v_cache[layer];
+    return NULL;
+}
+
+int32_t *gd_gpt_decoder_positions(gd_gpt_decoder *d) { return d != NULL ? d->pos : NULL; }
+
+/* ---- forward pieces -------------------------------------------------------------------- */
+
+/* reference src/nn/module.c:1012-1028 */
+static gd_status linear_forward(gd_context *ctx, const gpt_linear *l, const gd_tensor *x, gd_tensor *out)
+{
+    if (l->transposed) return gd_linear_transposed_weight(ctx, x, &l->weight, &l->bias, out);
+    return gd_linear(ctx, x, &l->weight, &l->bias, out);
+}
+
+/* attention input -> block output, shared by decode and prefill (reference :1052-1070, 941-958) */
+static gd_status block_tail(gd_gpt_decoder *d, const gpt_block *b, const gd_tensor *residual, const gd_tensor *attn_flat,
+                            gd_tensor *out)
+{
+    gd_context *ctx = d->ctx;
+    gd_tensor attn_proj, attn_resid, mlp_normed, up_gate, mlp_proj;
+    TRY(linear_forward(ctx, &b->attn_proj, attn_flat, &attn_proj));
+    TRY(gd_add(ctx, residual, &attn_proj, &attn_resid));
+    TRY(gd_rms_norm(ctx, &attn_resid, &b->mlp_norm_w, d->cfg.rms_eps, &mlp_normed));
+    TRY(linear_forward(ctx, &b->up_gate, &mlp_normed, &up_gate));
+    TRY(gd_swiglu_split_linear(ctx, &up_gate, &b->down_proj.weight, &b->down_proj.bias, &mlp_proj));
+    return gd_add(ctx, &attn_resid, &mlp_proj, out);
+}
+
+static gd_status block_decode(gd_gpt_decoder *d, int32_t l, const gd_tensor *x, const gd_tensor *positions,
+                              const gd_tensor *cache_positions, gd_tensor *out)
+{
+    gd_context *ctx = d->ctx;
+    const gpt_block *b = &d->blocks[l];
+    const gd_gpt_config *c = &d->cfg;
+    const gd_rope_config rope = {c->rope_theta, c->head_dim, false};
+    const gd_sdpa_decode_config sdpa = {0.0f, c->sdpa_window, 0};
+    gd_tensor normed, qkv, q3, k3, v3, q, k, v, attn, attn_flat;
+    int64_t q_shape[4] = {x->shape[0], 1, c->n_heads, c->head_dim};
+    int64_t flat_shape[2] = {x->shape[0], c->d_model};
+    TRY(gd_rms_norm(ctx, x, &b->attn_norm_w, c->rms_eps, &normed));
+    TRY(linear_forward(ctx, &b->qkv_proj, &normed, &qkv));
+    TRY(gd_qkv_split_rope(ctx, &qkv, positions, c->n_heads, c->head_dim, &rope, &q3, &k3, &v3));
+    TRY(gd_reshape(ctx, &q3, gd_shape_make(4U, q_shape), &q));
+    TRY(gd_reshape(ctx, &k3, gd_shape_make(4U, q_shape), &k));
+    TRY(gd_reshape(ctx, &v3, gd_shape_make(4U, q_shape), &v));
+    TRY(gd_kv_cache_append_positions(ctx, &d->k_cache[l], &d->v_cache[l], cache_positions, &k, &v));
+    TRY(gd_sdpa_decode_positions(ctx, &q, &d->k_cache[l], &d->v_cache[l], cache_positions, &sdpa, &attn));
+    TRY(gd_reshape(ctx, &attn, gd_shape_make(2U, flat_shape), &attn_flat));
+    return block_tail(d, b, x, &attn_flat, out);
+}
+
+static gd_status block_prefill(gd_gpt_decoder *d, int32_t l, const gd_tensor *x, const gd_tensor *positions,
+                               const gd_tensor *cu, const gd_tensor *cache_positions, gd_tensor *out)
+{
+    gd_context *ctx = d->ctx;
+    const gpt_block *b = &d->blocks[l];
+    const gd_gpt_config *c = &d->cfg;
+    const gd_rope_config rope = {c->rope_theta, c->head_dim, false};
+    const gd_sdpa_varlen_config sdpa = {0.0f, true, c->sdpa_window, 0, c->max_seq};
+    gd_tensor normed, qkv, q, k, v, attn, attn_flat;
+    int64_t flat_shape[2] = {x->shape[0], c->d_model};
+    TRY(gd_rms_norm(ctx, x, &b->attn_norm_w, c->rms_eps, &normed));
+    TRY(linear_forward(ctx, &b->qkv_proj, &normed, &qkv));
+    TRY(gd_qkv_split_rope(ctx, &qkv, positions, c->n_heads, c->head_dim, &rope, &q, &k, &v));
+    TRY(gd_kv_cache_append_packed(ctx, &d->k_cache[l], &d->v_cache[l], cache_positions, cu, &k, &v));
+    TRY(gd_sdpa_varlen(ctx, &q, &k, &v, cu, &sdpa, &attn));
+    TRY(gd_reshape(ctx, &attn, gd_shape_make(2U, flat_shape), &attn_flat));
+    return block_tail(d, b, x, &attn_flat, out);
+}
+
+static gd_status data_i32(gd_context *ctx, const int32_t *values, int64_t n, gd_tensor *out)
+{
+    int64_t dims[1] = {n};
+    TRY(gd_tensor_empty(ctx, GD_ARENA_DATA, GD_DTYPE_I32, gd_shape_make(1U, dims), 256U, out));
+    return gd_tensor_write(ctx, out, values, (size_t)n * sizeof(int32_t));
+}
+
+static gd_status head(gd_gpt_decoder *d, const gd_tensor *x, gd_tensor *logits, gd_tensor *ids, gd_tensor *gaps)
+{
+    gd_tensor normed;
+    TRY(gd_rms_norm(d->ctx, x, &d->final_norm_w, d->cfg.rms_eps, &normed));
+    TRY(gd_linear_transposed_weight(d->ctx, &normed, &d->lm_head, &d->lm_head_bias, logits));
+    return gd_argmax_rows(d->ctx, logits, ids, gaps);
+}
+
+static gd_status fetch(gd_gpt_decoder *d, const gd_tensor *logits, const gd_tensor *ids, const gd_tensor *gaps,
+                       int32_t *next_ids, float *out_gaps, uint16_t *out_logits)
+{
+    const size_t B = (size_t)d->cfg.batch;
+    if (next_ids != NULL) TRY(gd_tensor_read(d->ctx, ids, next_ids, B * sizeof(int32_t)));
+    if (out_gaps != NULL) TRY(gd_tensor_read(d->ctx, gaps, out_gaps, B * sizeof(float)));
+    if (out_logits != NULL) TRY(gd_tensor_read(d->ctx, logits, out_logits, B * (size_t)d->cfg.vocab * 2U));
+    return GD_OK;
+}
+
+gd_status gd_gpt_decoder_step(gd_gpt_decoder *d, const int32_t *ids, int32_t *next_ids, float *gaps, uint16_t *logits)
+{
+    gd_context *ctx;
+    gd_tensor t_ids, t_pos, t_cache_pos, x, y, t_logits, t_next, t_gaps;
+    gd_status st;
+    int32_t l, b;
+    if (d == NULL || ids == NULL) return GD_ERR_INVALID_ARGUMENT;
+    ctx = d->ctx;
+    TRY(gd_begin_step(ctx, GD_SCOPE_INFER, gd_batch_empty()));
+    st = data_i32(ctx, ids, d->cfg.batch, &t_ids);
+    if (st == GD_OK) st = data_i32(ctx, d->pos, d->cfg.batch, &t_pos);
+    if (st == GD_OK) st = data_i32(ctx, d->pos, d->cfg.batch, &t_cache_pos);
+    if (st == GD_OK) st = gd_embedding(ctx, &d->token_embedding, &t_ids, &x);
+    for (l = 0; l < d->cfg.n_layers && st == GD_OK; ++l) {
+        st = block_decode(d, l, &x, &t_pos, &t_cache_pos, &y);
+        x = y;
+    }
+    if (st == GD_OK) st = head(d, &x, &t_logits, &t_next, &t_gaps);
+    if (st != GD_OK) {
+        (void)gd_end_step(ctx);
+        return st;
+    }
+    for (b = 0; b < d->cfg.batch; ++b) d->pos[b] += 1;
+    TRY(gd_end_step(ctx));
+    return fetch(d, &t_logits, &t_next, &t_gaps, next_ids, gaps, logits);
+}
+
+gd_status gd_gpt_decoder_prefill(gd_gpt_decoder *d, const int32_t *ids, const int32_t *cu, int32_t *next_ids,
+                                 float *gaps, uint16_t *logits)
+{
+    gd_context *ctx;
+    gd_tensor t_ids, t_pos, t_cu, t_cache_pos, t_last, x, y, last_hidden, t_logits, t_next, t_gaps;
+    gd_status st = GD_OK;
+    int32_t *positions, *zero, *last_rows;
+    int32_t B, N, b, r, l;
+    if (d == NULL || ids == NULL || cu == NULL) return GD_ERR_INVALID_ARGUMENT;
+    ctx = d->ctx;
+    B = d->cfg.batch;
+    N = cu[B];
+    if (cu[0] != 0 || N <= 0) return GD_ERR_INVALID_ARGUMENT;
+    for (b = 0; b < B; ++b) {
+        if (cu[b + 1] <= cu[b] || cu[b + 1] - cu[b] > d->cfg.max_seq) return GD_ERR_INVALID_ARGUMENT;
+    }
+    positions = (int32_t *)malloc((size_t)N * sizeof(int32_t));
+    zero = (int32_t *)calloc((size_t)B, sizeof(int32_t));
+    last_rows = (int32_t *)malloc((size_t)B * sizeof(int32_t));
+    if (positions == NULL || zero == NULL || last_rows == NULL) {
+        free(positions); free(zero); free(last_rows);
+        return GD_ERR_OUT_OF_MEMORY;
+    }
+    for (b = 0; b < B; ++b) {
+        for (r = cu[b]; r < cu[b + 1]; ++r) positions[r] = r - cu[b];
+        last_rows[b] = cu[b + 1] - 1;
+    }
+    st = gd_begin_step(ctx, GD_SCOPE_INFER, gd_batch_empty());
+    if (st == GD_OK) {
+        st = data_i32(ctx, ids, N, &t_ids);
+        if (st == GD_OK) st = data_i32(ctx, positions, N, &t_pos);
+        if (st == GD_OK) st = data_i32(ctx, cu, (int64_t)B + 1, &t_cu);
+        if (st == GD_OK) st = data_i32(ctx, zero, B, &t_cache_pos);
+        if (st == GD_OK) st = data_i32(ctx, last_rows, B, &t_last);
+        if (st == GD_OK) st = gd_embedding(ctx, &d->token_embedding, &t_ids, &x);
+        for (l = 0; l < d->cfg.n_layers && st == GD_OK; ++l) {
+            st = block_prefill(d, l, &x, &t_pos, &t_cu, &t_cache_pos, &y);
+            x = y;
+        }
+        if (st == GD_OK) st = gd_gather_rows(ctx, &x, &t_last, &last_hidden);
+        if (st == GD_OK) st = head(d, &last_hidden, &t_logits, &t_next, &t_gaps);
+        if (st == GD_OK) {
+            for (b = 0; b < B; ++b) d->pos[b] = cu[b + 1] - cu[b];
+            st = gd_end_step(ctx);
+        } else {
+            (void)gd_end_step(ctx);
+        }
+    }
+    free(positions); free(zero); free(last_rows);
+    if (st != GD_OK) return st;
+    return fetch(d, &t_logits, &t_next, &t_gaps, next_ids, gaps, logits);
+}
+
+/* ---- device-resident decode -------------------------------------------------------------- */
+
+/* One step with ids / positions read from device tensors; enqueues only (no host transfer). */
+static gd_status enqueue_resident_step(gd_gpt_decoder *d, const gd_tensor *out_ids, const gd_tensor *out_gaps)
+{
+    gd_context *ctx = d->ctx;
+    gd_tensor x, y, logits, next, gaps;
+    gd_backend_tensor_view vn, vg, vi, vp, vs, vo, vog;
+    int32_t l;
+    TRY(gd_embedding(ctx, &d->token_embedding, &d->ids_dev, &x));
+    for (l = 0; l < d->cfg.n_layers; ++l) {
+        TRY(block_decode(d, l, &x, &d->pos_dev, &d->pos_dev, &y));
+        x = y;
+    }
+    TRY(head(d, &x, &logits, &next, &gaps));
+    memset(&vn, 0, sizeof(vn));
+#define VIEW1(t, v)                                                                 \
+    do {                                                                            \
+        memset(&(v), 0, sizeof(v));                                                 \
+        (v).buffer = (gd_backend_buffer *)(t)->storage.buffer;                      \
+        (v).offset = (t)->storage.offset + (t)->view_offset;                        \
+        (v).count = (size_t)(t)->shape[0];                                          \
+        (v).dtype = (uint32_t)(t)->dtype;                                           \
+        (v).rank = 1U;                                                              \
+        (v).shape[0] = (t)->shape[0];                                               \
+        (v).strides[0] = 1;                                                         \
+    } while (0)
+    VIEW1(&next, vn); VIEW1(&gaps, vg); VIEW1(&d->ids_dev, vi); VIEW1(&d->pos_dev, vp); VIEW1(&d->step_dev, vs);
+    VIEW1(out_ids, vo); VIEW1(out_gaps, vog);
+#undef VIEW1
+    return gd_backend_decode_advance(gd_context_backend(ctx), &vn, &vg, &vi, &vp, &vs, &vo, &vog);
+}
+
+gd_status gd_gpt_decoder_run_resident(gd_gpt_decoder *d, const int32_t *first_ids, int32_t n_steps, int32_t *out_ids,
+                                      float *out_gaps, float *step_ms)
+{
+    gd_context *ctx;
+    gd_backend *be;
+    gd_backend_graph *graph = NULL;
+    gd_backend_timer *timer = NULL;
+    gd_tensor t_out_ids, t_out_gaps;
+    gd_status st;
+    int64_t dims[1];
+    int32_t b, s, zero = 0;
+    if (d == NULL || first_ids == NULL || n_steps <= 0 || out_ids == NULL) return GD_ERR_INVALID_ARGUMENT;
+    ctx = d->ctx;
+    be = gd_context_backend(ctx);
+    for (b = 0; b < d->cfg.batch; ++b) {
+        if (d->pos[b] + n_steps > d->cfg.max_seq) return GD_ERR_INVALID_ARGUMENT;
+    }
+    TRY(gd_tensor_write(ctx, &d->ids_dev, first_ids, (size_t)d->cfg.batch * sizeof(int32_t)));
+    TRY(gd_tensor_write(ctx, &d->pos_dev, d->pos, (size_t)d->cfg.batch * sizeof(int32_t)));
+    TRY(gd_tensor_write(ctx, &d->step_dev, &zero, sizeof(zero)));
+    TRY(gd_begin_step(ctx, GD_SCOPE_INFER, gd_batch_empty()));
+    dims[0] = (int64_t)n_steps * d->cfg.batch;
+    st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_I32, gd_shape_make(1U, dims), 256U, &t_out_ids);
+    if (st == GD_OK) st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F32, gd_shape_make(1U, dims), 256U, &t_out_gaps);
+    /* step 0 runs eagerly (it also sizes the attention workspace); steps 1.. replay a captured graph */
+    if (st == GD_OK) st = enqueue_resident_step(d, &t_out_ids, &t_out_gaps);
+    if (st == GD_OK && n_steps > 1) {
+        st = gd_backend_graph_begin_capture(be);
+        if (st == GD_OK) {
+            st = enqueue_resident_step(d, &t_out_ids, &t_out_gaps);
+            if (st == GD_OK) st = gd_backend_graph_end_capture(be, &graph);
+            else (void)gd_backend_graph_end_capture(be, &graph);
+        }
+        if (st == GD_OK && step_ms != NULL) st = gd_backend_timer_create(be, &timer);
+        if (st == GD_OK && timer != NULL) st = gd_backend_timer_start(timer);
+        for (s = 1; s < n_steps && st == GD_OK; ++s) st = gd_backend_graph_launch(be, graph);
+        if (st == GD_OK && timer != NULL) st = gd_backend_timer_stop(timer);
+    }
+    if (st != GD_OK) {
+        (void)gd_end_step(ctx);
+        if (graph != NULL) gd_backend_graph_destroy(graph);
+        if (timer != NULL) gd_backend_timer_destroy(timer);
+        return st;
+    }
+    st = gd_end_step(ctx);
+    if (st == GD_OK) st = gd_tensor_read(ctx, &t_out_ids, out_ids, (size_t)dims[0] * sizeof(int32_t));
+    if (st == GD_OK && out_gaps != NULL) st = gd_tensor_read(ctx, &t_out_gaps, out_gaps, (size_t)dims[0] * sizeof(float));
+    if (st == GD_OK && step_ms != NULL) {
+        float ms = 0.0f;
+        if (timer != NULL) st = gd_backend_timer_elapsed_ms(timer, &ms);
+        *step_ms = n_steps > 1 ? ms / (float)(n_steps - 1) : 0.0f;
+    }
+    if (graph != NULL) gd_backend_graph_destroy(graph);
+    if (timer != NULL) gd_backend_timer_destroy(timer);
+    if (st == GD_OK) {
+        for (b = 0; b < d->cfg.batch; ++b) d->pos[b] += n_steps;
+    }
+    return st;
+}

@@ -1,0 +1,76 @@
+/*
+ * gd_gpt_decoder.h - the decoder-only language model of the reference's example
+ * (examples/gpt_lm/gpt_lm_shared.c), inference part, with run-time dimensions: weights, K/V
+ * caches, packed prefill and the batched cached decode step, written against the public gd_*
+ * operators of gradients_infer.h in the reference's call order
+ * (gpt_block_decode_cached :961-1071, gpt_lm_decode_logits :1204-1246,
+ * gpt_block_prefill_cached :825-959, gpt_lm_prefill_last_logits :1174-1202).
+ *
+ * Two ways to run a decode step:
+ *   gd_gpt_decoder_step          one gd_begin_step .. gd_end_step scope per token, every operator
+ *                                issued through the public API, ids uploaded and results
+ *                                downloaded each step (the reference generator's loop);
+ *   gd_gpt_decoder_run_resident  token ids and cache positions stay on the device, the greedy
+ *                                token of step t feeds step t+1 without a host round trip, and the
+ *                                step is replayed from a captured graph.
+ * Both produce the same tokens.
+ */
+#ifndef GD_GPT_DECODER_H
+#define GD_GPT_DECODER_H
+
+#include "gradients_infer.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct gd_gpt_config {
+    int32_t vocab, d_model, n_layers, n_heads, head_dim, mlp_hidden;
+    int32_t max_seq;     /* cache rows per sequence (Tmax) */
+    int32_t batch;       /* sequences decoded together */
+    int32_t sdpa_window; /* 0 = attend to the whole cache; the reference example uses 256 */
+    int32_t tie_lm_head; /* 1: LM head shares the embedding table (reference :393-402); 0: own [V,Dm] weight */
+    float rms_eps;       /* reference 1e-5 (gpt_lm_shared.h:58) */
+    float rope_theta;    /* reference 10000 */
+    uint64_t seed;
+} gd_gpt_config;
+
+typedef struct gd_gpt_decoder gd_gpt_decoder;
+
+/* Bytes the params and state arenas need for this configuration (for gd_memory_config). */
+size_t gd_gpt_params_bytes(const gd_gpt_config *cfg);
+size_t gd_gpt_state_bytes(const gd_gpt_config *cfg);
+
+/* Allocates weights in the params arena and caches in the state arena and initialises the weights
+ * the way the reference example does (N(0,0.02) from a splitmix64 + Box-Muller stream seeded per
+ * tensor, residual projections scaled by 1/sqrt(2L), biases 0, norm weights 1; :196-218,290-402). */
+gd_status gd_gpt_decoder_create(gd_context *ctx, const gd_gpt_config *cfg, gd_gpt_decoder **out);
+void gd_gpt_decoder_destroy(gd_gpt_decoder *dec);
+
+/* Weight / cache tensors by name (embed, lm_head, lm_bias, final_norm, attn_norm, mlp_norm, w_qkv,
+ * b_qkv, w_attn, b_attn, w_upgate, b_upgate, w_down, b_down, k_cache, v_cache); NULL if unknown. */
+gd_tensor *gd_gpt_decoder_tensor(gd_gpt_decoder *dec, const char *name, int32_t layer);
+
+/* Host copy of the live length of every sequence ([batch]); writable (e.g. after filling caches). */
+int32_t *gd_gpt_decoder_positions(gd_gpt_decoder *dec);
+
+/* Packed prefill from position 0: ids [cu[batch]], cu [batch+1] on the host.  Outputs (each may be
+ * NULL): greedy next ids [batch], top-2 gaps [batch], logits [batch, vocab] as F16 bits. */
+gd_status gd_gpt_decoder_prefill(gd_gpt_decoder *dec, const int32_t *ids, const int32_t *cu, int32_t *next_ids,
+                                 float *gaps, uint16_t *logits);
+
+/* One batched decode step through the public operator API.  ids [batch] on the host. */
+gd_status gd_gpt_decoder_step(gd_gpt_decoder *dec, const int32_t *ids, int32_t *next_ids, float *gaps,
+                              uint16_t *logits);
+
+/* n_steps greedy steps with device-resident ids and positions, starting from first_ids [batch].
+ * out_ids receives [n_steps, batch] token ids, out_gaps (may be NULL) the top-2 gaps.
+ * step_ms (may be NULL) receives the mean device time per step measured with stream events. */
+gd_status gd_gpt_decoder_run_resident(gd_gpt_decoder *dec, const int32_t *first_ids, int32_t n_steps,
+                                      int32_t *out_ids, float *out_gaps, float *step_ms);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* GD_GPT_DECODER_H */

@@ -632,7 +632,8 @@ typedef struct gdo_decoder {
     int64_t vocab, d_model, n_layers, n_heads, head_dim, mlp_hidden, max_seq, batch;
     float rms_eps, rope_theta;
     int window;
-    uint16_t *embed;      /* [V,Dm] (tied LM head) */
+    uint16_t *embed;      /* [V,Dm] */
+    uint16_t *lm_head;    /* [V,Dm]; == embed while the head is tied (reference :393-402) */
     uint16_t *lm_bias;    /* [V] */
     uint16_t *final_norm; /* [Dm] */
     uint16_t **attn_norm, **mlp_norm;    /* [Dm] */
@@ -675,6 +676,7 @@ GDO_API gdo_decoder *gdo_decoder_create(int64_t vocab, int64_t d_model, int64_t 
     d->head_dim = head_dim; d->mlp_hidden = mlp_hidden; d->max_seq = max_seq; d->batch = batch;
     d->rms_eps = 1.0e-5f; d->rope_theta = 10000.0f; d->window = window;
     d->embed = normal_h((size_t)(vocab * d_model), gdo_splitmix64(seed ^ UINT64_C(0xabc001)), std);
+    d->lm_head = d->embed;
     d->lm_bias = alloc_h((size_t)vocab);
     d->final_norm = ones_h((size_t)d_model);
 #define ARR(name) d->name = (uint16_t **)calloc(L, sizeof(uint16_t *))
@@ -710,6 +712,7 @@ GDO_API void gdo_decoder_destroy(gdo_decoder *d)
     }
     free(d->attn_norm); free(d->mlp_norm); free(d->w_qkv); free(d->b_qkv); free(d->w_attn);
     free(d->b_attn); free(d->w_upgate); free(d->b_upgate); free(d->w_down); free(d->b_down);
+    if (d->lm_head != d->embed) free(d->lm_head);
     free(d->k_cache); free(d->v_cache); free(d->embed); free(d->lm_bias); free(d->final_norm);
     free(d->pos); free(d);
 }
@@ -720,7 +723,7 @@ GDO_API uint16_t *gdo_decoder_tensor(gdo_decoder *d, const char *name, int64_t l
 {
 #define ONE(n) if (!strcmp(name, #n)) return d->n
 #define PER(n) if (!strcmp(name, #n)) return d->n[layer]
-    ONE(embed); ONE(lm_bias); ONE(final_norm);
+    ONE(embed); ONE(lm_head); ONE(lm_bias); ONE(final_norm);
     PER(attn_norm); PER(mlp_norm); PER(w_qkv); PER(b_qkv); PER(w_attn); PER(b_attn);
     PER(w_upgate); PER(b_upgate); PER(w_down); PER(b_down); PER(k_cache); PER(v_cache);
 #undef ONE
@@ -729,6 +732,13 @@ GDO_API uint16_t *gdo_decoder_tensor(gdo_decoder *d, const char *name, int64_t l
 }
 
 GDO_API int32_t *gdo_decoder_positions(gdo_decoder *d) { return d->pos; }
+
+/* Gives the LM head its own [V,Dm] weight, N(0,0.02) from splitmix64(seed ^ 0xabc002). */
+GDO_API void gdo_decoder_untie_lm_head(gdo_decoder *d, uint64_t seed)
+{
+    if (d->lm_head == d->embed) d->lm_head = alloc_h((size_t)(d->vocab * d->d_model));
+    gdo_fill_normal_f16(d->lm_head, (size_t)(d->vocab * d->d_model), gdo_splitmix64(seed ^ UINT64_C(0xabc002)), 0.02f);
+}
 
 /* One transformer block over `rows` token rows; `attend` runs the attention for
  * this block.  Order of operators: reference examples/gpt_lm/gpt_lm_shared.c:
@@ -794,7 +804,7 @@ static void head_forward(gdo_decoder *d, int64_t rows, const uint16_t *x, uint16
 {
     uint16_t *normed = alloc_h((size_t)(rows * d->d_model));
     gdo_rms_norm_f16(x, d->final_norm, rows, d->d_model, d->rms_eps, normed);
-    gdo_linear_nt_f16(normed, d->embed, d->lm_bias, rows, d->d_model, d->vocab, logits);
+    gdo_linear_nt_f16(normed, d->lm_head, d->lm_bias, rows, d->d_model, d->vocab, logits);
     free(normed);
 }
 

@@ -74,6 +74,7 @@ def _declare(l):
         "gdo_embedding_f16": [_vp, _vp, _i64, _i64, _i64, _vp],
         "gdo_argmax_rows_f16": [_vp, _i64, _i64, _vp, _vp],
         "gdo_decoder_destroy": [_vp],
+        "gdo_decoder_untie_lm_head": [_vp, _u64],
         "gdo_decoder_step": [_vp, _vp, _vp, _vp, _vp],
         "gdo_decoder_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _vp],
     }
@@ -293,7 +294,7 @@ class Decoder:
     """CPU decoder following the reference example's call sequence."""
 
     _SHAPES = {
-        "embed": lambda d: (d.vocab, d.d_model), "lm_bias": lambda d: (d.vocab,),
+        "embed": lambda d: (d.vocab, d.d_model), "lm_head": lambda d: (d.vocab, d.d_model), "lm_bias": lambda d: (d.vocab,),
         "final_norm": lambda d: (d.d_model,), "attn_norm": lambda d: (d.d_model,),
         "mlp_norm": lambda d: (d.d_model,), "w_qkv": lambda d: (3 * d.d_model, d.d_model),
         "b_qkv": lambda d: (3 * d.d_model,), "w_attn": lambda d: (d.d_model, d.d_model),
@@ -305,12 +306,14 @@ class Decoder:
     }
 
     def __init__(self, vocab, d_model, n_layers, n_heads, head_dim, mlp_hidden, max_seq, batch,
-                 window=0, seed=1000):
+                 window=0, seed=1000, tie_lm_head=True):
         self.vocab, self.d_model, self.n_layers = vocab, d_model, n_layers
         self.n_heads, self.head_dim, self.mlp_hidden = n_heads, head_dim, mlp_hidden
         self.max_seq, self.batch, self.window, self.seed = max_seq, batch, window, seed
         self._h = lib().gdo_decoder_create(vocab, d_model, n_layers, n_heads, head_dim, mlp_hidden,
                                            max_seq, batch, window, seed)
+        if not tie_lm_head:
+            lib().gdo_decoder_untie_lm_head(self._h, seed)
 
     def close(self):
         if self._h:
