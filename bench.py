@@ -1,0 +1,152 @@
+#!/usr/bin/env python3
+"""Benchmark of the decode hot path on one MI355X.
+
+Workload (BASELINE.json configs[2]): gpt_lm default architecture (vocab 2048, d_model 512,
+3 layers, 8 heads x 64, SwiGLU hidden 1536, untied LM head), random-init F16 weights, batch 64,
+every sequence's K/V cache pre-filled to 511 tokens by a real packed prefill of uniform random
+token ids.  One step = the full layer stack for 64 new tokens at cache position 511 (512 keys per
+sequence): embedding, rms_norm, qkv projection, qkv_split_rope, K/V append, sdpa_decode, output
+projection, swiglu_split_linear, LM head, greedy argmax; the token of one step feeds the next on
+the device.  The cache position is held at 511 so that every timed step has exactly this shape.
+
+Prints ONE JSON line: whole-job tokens/s, plus
+  roofline      sdpa_decode (the dominant HBM consumer) timed alone with stream events at the same
+                shape on the decoder's own caches: algorithmic bytes / mean launch time vs 8 TB/s;
+  cpu_baseline  the CPU oracle's decoder running the same step shape on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def _package():
+    import __graft_entry__ as entry
+    return entry._package(), entry._oracle()
+
+
+def sdpa_roofline(dec, D, pkg, iters=200):
+    """Mean duration of one sdpa_decode launch at the step's shape, with events on the backend stream."""
+    import ctypes as C
+    cfg = dec.cfg
+    be = dec.ctx.backend()
+    buf = be.buffer(8 << 20)
+    B, H, Dh, T = cfg.batch, cfg.n_heads, cfg.head_dim, cfg.max_seq
+    rng = np.random.default_rng(1)
+    q = buf.from_numpy((rng.standard_normal((B, 1, H, Dh))).astype(np.float16))
+    out = buf.alloc((B, 1, H, Dh), pkg.F16)
+    pos = buf.from_numpy(np.full(B, T - 1, np.int32))
+    kv, vv = D.view_of(dec.tensor("k_cache", 0)), D.view_of(dec.tensor("v_cache", 0))
+    args = pkg.SdpaDecodeArgs(1.0 / np.sqrt(Dh), cfg.sdpa_window, 0, 0)
+
+    def launch():
+        st = be.call("gd_backend_sdpa_decode_positions", q.view(), kv, vv, pos.view(), out.view(), C.byref(args))
+        assert st == 0, st
+
+    timer = pkg.Timer(be)
+    be.scope_begin()  # inside a scope operators are enqueued without waiting
+    for _ in range(20):
+        launch()
+    timer.start()
+    for _ in range(iters):
+        launch()
+    timer.stop()
+    ms = timer.elapsed_ms()
+    be.fence_wait(be.record_fence())
+    timer.close()
+    be.free(buf)
+    keys = min(T, cfg.sdpa_window) if cfg.sdpa_window > 0 else T
+    algo_bytes = B * keys * H * Dh * 2 * 2 + 2 * B * H * Dh * 2 + 4 * B
+    sec = ms / 1e3 / iters
+    gbs = algo_bytes / sec / 1e9
+    return {"bound": "hbm", "kernel": "gd_sdpa_decode_split_kernel<64,1>", "achieved": round(gbs, 1),
+            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+            "algorithmic_bytes_per_launch": algo_bytes, "us_per_launch": round(sec * 1e6, 3), "launches": iters}
+
+
+def cpu_baseline(oracle, cfg_tuple, budget_s=12.0, max_steps=64):
+    """The CPU oracle's decoder on the same step shape: caches filled to 511 rows with random F16 rows
+    (a CPU prefill of 32k tokens would take minutes), then whole decode steps until the budget is used."""
+    vocab, d_model, layers, heads, head_dim, hidden, max_seq, batch = cfg_tuple
+    ref = oracle.Decoder(vocab, d_model, layers, heads, head_dim, hidden, max_seq, batch, 0, 1002, False)
+    for l in range(layers):
+        ref.tensor("k_cache", l)[:] = oracle.normal_f16((batch, max_seq, heads, head_dim), 7000 + l, 0.5)
+        ref.tensor("v_cache", l)[:] = oracle.normal_f16((batch, max_seq, heads, head_dim), 7100 + l, 0.5)
+    ids = oracle.uniform_i32(batch, 7200, 0, vocab - 1)
+    steps, t0 = 0, time.perf_counter()
+    while steps < max_steps and (steps == 0 or time.perf_counter() - t0 < budget_s):
+        ref.positions[:] = max_seq - 1
+        _, ids, _ = ref.step(ids)
+        steps += 1
+    dt = time.perf_counter() - t0
+    ref.close()
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return {"value": round(batch * steps / dt, 2), "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"{steps} whole decode steps of the same shape (B={batch}, 511-row caches filled with random "
+                      f"F16 rows instead of a CPU prefill), {dt:.1f} s, oracle/gd_oracle.c with OpenMP"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py measures one GPU: the decode path holds every sequence, its K/V cache and a full "
+                 "weight replica on a single device (sequences are independent, so more GPUs would only add "
+                 "replicas); run with --gpus 1")
+    pkg, oracle = _package()
+    pkg.lib()
+    from gradients_c_amd import decoder as D
+
+    B, T = 64, 512
+    shape = (2048, 512, 3, 8, 64, 1536, T, B)
+    cfg = D.gpt_config(*shape, window=0, tie_lm_head=False, seed=1002)
+    dec = D.GptDecoder(cfg, max_prefill_tokens=B * (T - 1))
+    prompt = oracle.uniform_i32(B * (T - 1), 1002, 0, 2047)
+    cu = (np.arange(B + 1) * (T - 1)).astype(np.int32)
+    t0 = time.perf_counter()
+    _, first, _ = dec.prefill(prompt, cu, want_logits=False)
+    prefill_s = time.perf_counter() - t0
+
+    total = a.warmup + a.steps
+    dec.resident_begin(first, total + 1, hold_positions=True)  # step 0 runs eagerly inside begin
+    dec.resident_run(a.warmup)
+    dec.resident_sync()
+    t0 = time.perf_counter()
+    dec.resident_run(a.steps)
+    dec.resident_sync()
+    elapsed = time.perf_counter() - t0
+    ids, gaps = dec.resident_end()
+    assert ids.shape == (total + 1, B) and ids.min() >= 0 and ids.max() < 2048
+
+    roof = sdpa_roofline(dec, D, pkg)
+    dec.close()
+    cpu = None if a.no_cpu_baseline else cpu_baseline(oracle, shape)
+
+    ms_per_step = elapsed * 1e3 / a.steps
+    line = {
+        "metric": "decode tokens/sec at B=64", "value": round(B * a.steps / elapsed, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "configs[2]: gpt_lm default decoder (V2048 Dm512 L3 H8 Dh64 Hm1536, untied head), "
+                               "batched decode step B=64, caches pre-filled to 511 tokens by packed prefill of "
+                               "uniform random ids, full stack incl. greedy argmax, device-resident token feedback",
+                   "batch": B, "cache_tokens": T, "sdpa_window": 0, "prefill_seconds": round(prefill_s, 3)},
+        "roofline": roof, "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

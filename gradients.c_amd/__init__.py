@@ -124,7 +124,7 @@ _SIGNATURES = {
     "gd_backend_linear_nt": [_vp, _MV, _MV, _VV, _MV],
     "gd_backend_gather_rows": [_vp, _TV, _TV, _TV],
     "gd_backend_add_scalar_i32": [_vp, _TV, _TV, C.c_int32],
-    "gd_backend_decode_advance": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, _TV],
+    "gd_backend_decode_advance": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, _TV, C.c_int32],
     "gd_backend_copy": [_vp, _vp, C.c_size_t, _vp, C.c_size_t, C.c_size_t],
     "gd_backend_timer_create": [_vp, C.POINTER(_vp)],
     "gd_backend_timer_start": [_vp],
@@ -297,21 +297,26 @@ class Timer:
 class Backend:
     """gd_backend: one HIP device, one stream.  Methods mirror the gd_backend_* operators."""
 
-    def __init__(self):
-        h = _vp()
-        st = lib().gd_backend_create_default(C.byref(h))
-        if st != GD_OK:
-            raise GdError(st, "gd_backend_create_default (no HIP device? there is no CPU fallback)")
-        self.handle = h.value
+    def __init__(self, borrowed_handle=None):
+        """Creates the default backend, or wraps the backend owned by a gd_context (borrowed)."""
+        self._owned = borrowed_handle is None
+        if self._owned:
+            h = _vp()
+            st = lib().gd_backend_create_default(C.byref(h))
+            if st != GD_OK:
+                raise GdError(st, "gd_backend_create_default (no HIP device? there is no CPU fallback)")
+            self.handle = h.value
+        else:
+            self.handle = borrowed_handle
         self._buffers = []
 
     def close(self):
         for b in self._buffers:
             b.close()
         self._buffers = []
-        if self.handle:
+        if self.handle and self._owned:
             lib().gd_backend_destroy(self.handle)
-            self.handle = None
+        self.handle = None
 
     @property
     def name(self):

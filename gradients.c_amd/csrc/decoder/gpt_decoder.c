@@ -37,6 +37,11 @@ struct gd_gpt_decoder {
     int32_t *pos; /* host copy of the live lengths */
     /* device-resident decode state (state arena) */
     gd_tensor ids_dev, pos_dev, step_dev;
+    /* open resident session */
+    bool resident_open;
+    int32_t resident_max_steps, resident_steps, resident_hold;
+    gd_backend_graph *resident_graph;
+    gd_tensor resident_out_ids, resident_out_gaps;
 };
 
 /* ---- deterministic initialisation (reference :32-48, 196-218) ----------------------- */
@@ -396,7 +401,19 @@ gd_status gd_gpt_decoder_prefill(gd_gpt_decoder *d, const int32_t *ids, const in
 /* ---- device-resident decode -------------------------------------------------------------- */
 
 /* One step with ids / positions read from device tensors; enqueues only (no host transfer). */
-static gd_status enqueue_resident_step(gd_gpt_decoder *d, const gd_tensor *out_ids, const gd_tensor *out_gaps)
+static void view1(const gd_tensor *t, gd_backend_tensor_view *v)
+{
+    memset(v, 0, sizeof(*v));
+    v->buffer = (gd_backend_buffer *)t->storage.buffer;
+    v->offset = t->storage.offset + t->view_offset;
+    v->count = (size_t)t->shape[0];
+    v->dtype = (uint32_t)t->dtype;
+    v->rank = 1U;
+    v->shape[0] = t->shape[0];
+    v->strides[0] = 1;
+}
+
+static gd_status enqueue_resident_step(gd_gpt_decoder *d)
 {
     gd_context *ctx = d->ctx;
     gd_tensor x, y, logits, next, gaps;
@@ -408,80 +425,136 @@ static gd_status enqueue_resident_step(gd_gpt_decoder *d, const gd_tensor *out_i
         x = y;
     }
     TRY(head(d, &x, &logits, &next, &gaps));
-    memset(&vn, 0, sizeof(vn));
-#define VIEW1(t, v)                                                                 \
-    do {                                                                            \
-        memset(&(v), 0, sizeof(v));                                                 \
-        (v).buffer = (gd_backend_buffer *)(t)->storage.buffer;                      \
-        (v).offset = (t)->storage.offset + (t)->view_offset;                        \
-        (v).count = (size_t)(t)->shape[0];                                          \
-        (v).dtype = (uint32_t)(t)->dtype;                                           \
-        (v).rank = 1U;                                                              \
-        (v).shape[0] = (t)->shape[0];                                               \
-        (v).strides[0] = 1;                                                         \
-    } while (0)
-    VIEW1(&next, vn); VIEW1(&gaps, vg); VIEW1(&d->ids_dev, vi); VIEW1(&d->pos_dev, vp); VIEW1(&d->step_dev, vs);
-    VIEW1(out_ids, vo); VIEW1(out_gaps, vog);
-#undef VIEW1
-    return gd_backend_decode_advance(gd_context_backend(ctx), &vn, &vg, &vi, &vp, &vs, &vo, &vog);
+    view1(&next, &vn);
+    view1(&gaps, &vg);
+    view1(&d->ids_dev, &vi);
+    view1(&d->pos_dev, &vp);
+    view1(&d->step_dev, &vs);
+    view1(&d->resident_out_ids, &vo);
+    view1(&d->resident_out_gaps, &vog);
+    return gd_backend_decode_advance(gd_context_backend(ctx), &vn, &vg, &vi, &vp, &vs, &vo, &vog,
+                                     d->resident_hold ? 0 : 1);
 }
 
-gd_status gd_gpt_decoder_run_resident(gd_gpt_decoder *d, const int32_t *first_ids, int32_t n_steps, int32_t *out_ids,
-                                      float *out_gaps, float *step_ms)
+static void resident_abort(gd_gpt_decoder *d)
+{
+    (void)gd_end_step(d->ctx);
+    if (d->resident_graph != NULL) gd_backend_graph_destroy(d->resident_graph);
+    d->resident_graph = NULL;
+    d->resident_open = false;
+}
+
+gd_status gd_gpt_decoder_resident_begin(gd_gpt_decoder *d, const int32_t *first_ids, int32_t max_steps,
+                                        int32_t hold_positions)
 {
     gd_context *ctx;
     gd_backend *be;
-    gd_backend_graph *graph = NULL;
-    gd_backend_timer *timer = NULL;
-    gd_tensor t_out_ids, t_out_gaps;
     gd_status st;
     int64_t dims[1];
-    int32_t b, s, zero = 0;
-    if (d == NULL || first_ids == NULL || n_steps <= 0 || out_ids == NULL) return GD_ERR_INVALID_ARGUMENT;
+    int32_t b, zero = 0;
+    if (d == NULL || first_ids == NULL || max_steps <= 0) return GD_ERR_INVALID_ARGUMENT;
+    if (d->resident_open) return GD_ERR_BAD_STATE;
     ctx = d->ctx;
     be = gd_context_backend(ctx);
     for (b = 0; b < d->cfg.batch; ++b) {
-        if (d->pos[b] + n_steps > d->cfg.max_seq) return GD_ERR_INVALID_ARGUMENT;
+        if (d->pos[b] < 0 || d->pos[b] + (hold_positions ? 1 : max_steps) > d->cfg.max_seq) return GD_ERR_INVALID_ARGUMENT;
     }
     TRY(gd_tensor_write(ctx, &d->ids_dev, first_ids, (size_t)d->cfg.batch * sizeof(int32_t)));
     TRY(gd_tensor_write(ctx, &d->pos_dev, d->pos, (size_t)d->cfg.batch * sizeof(int32_t)));
     TRY(gd_tensor_write(ctx, &d->step_dev, &zero, sizeof(zero)));
     TRY(gd_begin_step(ctx, GD_SCOPE_INFER, gd_batch_empty()));
-    dims[0] = (int64_t)n_steps * d->cfg.batch;
-    st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_I32, gd_shape_make(1U, dims), 256U, &t_out_ids);
-    if (st == GD_OK) st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F32, gd_shape_make(1U, dims), 256U, &t_out_gaps);
-    /* step 0 runs eagerly (it also sizes the attention workspace); steps 1.. replay a captured graph */
-    if (st == GD_OK) st = enqueue_resident_step(d, &t_out_ids, &t_out_gaps);
-    if (st == GD_OK && n_steps > 1) {
+    d->resident_open = true;
+    d->resident_graph = NULL;
+    d->resident_max_steps = max_steps;
+    d->resident_steps = 0;
+    d->resident_hold = hold_positions != 0;
+    dims[0] = (int64_t)max_steps * d->cfg.batch;
+    st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_I32, gd_shape_make(1U, dims), 256U, &d->resident_out_ids);
+    if (st == GD_OK) st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F32, gd_shape_make(1U, dims), 256U, &d->resident_out_gaps);
+    /* the first step runs eagerly (it also sizes the attention workspace); later steps replay a graph */
+    if (st == GD_OK) st = enqueue_resident_step(d);
+    if (st == GD_OK) d->resident_steps = 1;
+    if (st == GD_OK && max_steps > 1) {
         st = gd_backend_graph_begin_capture(be);
         if (st == GD_OK) {
-            st = enqueue_resident_step(d, &t_out_ids, &t_out_gaps);
-            if (st == GD_OK) st = gd_backend_graph_end_capture(be, &graph);
-            else (void)gd_backend_graph_end_capture(be, &graph);
+            st = enqueue_resident_step(d);
+            if (st == GD_OK) st = gd_backend_graph_end_capture(be, &d->resident_graph);
+            else (void)gd_backend_graph_end_capture(be, &d->resident_graph);
         }
-        if (st == GD_OK && step_ms != NULL) st = gd_backend_timer_create(be, &timer);
-        if (st == GD_OK && timer != NULL) st = gd_backend_timer_start(timer);
-        for (s = 1; s < n_steps && st == GD_OK; ++s) st = gd_backend_graph_launch(be, graph);
-        if (st == GD_OK && timer != NULL) st = gd_backend_timer_stop(timer);
     }
-    if (st != GD_OK) {
-        (void)gd_end_step(ctx);
-        if (graph != NULL) gd_backend_graph_destroy(graph);
-        if (timer != NULL) gd_backend_timer_destroy(timer);
-        return st;
+    if (st != GD_OK) resident_abort(d);
+    return st;
+}
+
+gd_status gd_gpt_decoder_resident_run(gd_gpt_decoder *d, int32_t n_steps)
+{
+    gd_backend *be;
+    int32_t s;
+    if (d == NULL || n_steps < 0) return GD_ERR_INVALID_ARGUMENT;
+    if (!d->resident_open) return GD_ERR_BAD_STATE;
+    if (d->resident_steps + n_steps > d->resident_max_steps) return GD_ERR_INVALID_ARGUMENT;
+    be = gd_context_backend(d->ctx);
+    for (s = 0; s < n_steps; ++s) {
+        TRY(gd_backend_graph_launch(be, d->resident_graph));
+        d->resident_steps += 1;
     }
+    return GD_OK;
+}
+
+gd_status gd_gpt_decoder_resident_sync(gd_gpt_decoder *d)
+{
+    if (d == NULL) return GD_ERR_INVALID_ARGUMENT;
+    return gd_synchronize(d->ctx);
+}
+
+gd_status gd_gpt_decoder_resident_end(gd_gpt_decoder *d, int32_t *out_ids, float *out_gaps, int32_t *steps_done)
+{
+    gd_context *ctx;
+    gd_status st;
+    gd_tensor ids_view, gaps_view;
+    int32_t b;
+    if (d == NULL) return GD_ERR_INVALID_ARGUMENT;
+    if (!d->resident_open) return GD_ERR_BAD_STATE;
+    ctx = d->ctx;
     st = gd_end_step(ctx);
-    if (st == GD_OK) st = gd_tensor_read(ctx, &t_out_ids, out_ids, (size_t)dims[0] * sizeof(int32_t));
-    if (st == GD_OK && out_gaps != NULL) st = gd_tensor_read(ctx, &t_out_gaps, out_gaps, (size_t)dims[0] * sizeof(float));
-    if (st == GD_OK && step_ms != NULL) {
-        float ms = 0.0f;
-        if (timer != NULL) st = gd_backend_timer_elapsed_ms(timer, &ms);
-        *step_ms = n_steps > 1 ? ms / (float)(n_steps - 1) : 0.0f;
+    if (st == GD_OK && out_ids != NULL) {
+        st = gd_tensor_slice(ctx, &d->resident_out_ids, 0U, 0, (int64_t)d->resident_steps * d->cfg.batch, &ids_view);
+        if (st == GD_OK) st = gd_tensor_read(ctx, &ids_view, out_ids, (size_t)d->resident_steps * (size_t)d->cfg.batch * sizeof(int32_t));
     }
-    if (graph != NULL) gd_backend_graph_destroy(graph);
+    if (st == GD_OK && out_gaps != NULL) {
+        st = gd_tensor_slice(ctx, &d->resident_out_gaps, 0U, 0, (int64_t)d->resident_steps * d->cfg.batch, &gaps_view);
+        if (st == GD_OK) st = gd_tensor_read(ctx, &gaps_view, out_gaps, (size_t)d->resident_steps * (size_t)d->cfg.batch * sizeof(float));
+    }
+    if (d->resident_graph != NULL) gd_backend_graph_destroy(d->resident_graph);
+    d->resident_graph = NULL;
+    d->resident_open = false;
+    if (steps_done != NULL) *steps_done = d->resident_steps;
+    if (st == GD_OK && !d->resident_hold) {
+        for (b = 0; b < d->cfg.batch; ++b) d->pos[b] += d->resident_steps;
+    }
+    return st;
+}
+
+gd_status gd_gpt_decoder_run_resident(gd_gpt_decoder *d, const int32_t *first_ids, int32_t n_steps, int32_t *out_ids,
+                                      float *out_gaps, float *step_ms)
+{
+    gd_backend_timer *timer = NULL;
+    gd_status st;
+    float ms = 0.0f;
+    if (d == NULL || n_steps <= 0 || out_ids == NULL) return GD_ERR_INVALID_ARGUMENT;
+    TRY(gd_gpt_decoder_resident_begin(d, first_ids, n_steps, 0));
+    st = GD_OK;
+    if (step_ms != NULL) st = gd_backend_timer_create(gd_context_backend(d->ctx), &timer);
+    if (st == GD_OK && timer != NULL) st = gd_backend_timer_start(timer);
+    if (st == GD_OK) st = gd_gpt_decoder_resident_run(d, n_steps - 1);
+    if (st == GD_OK && timer != NULL) st = gd_backend_timer_stop(timer);
+    if (st != GD_OK) {
+        resident_abort(d);
+    } else {
+        st = gd_gpt_decoder_resident_end(d, out_ids, out_gaps, NULL);
+        if (st == GD_OK && timer != NULL) st = gd_backend_timer_elapsed_ms(timer, &ms);
+    }
     if (timer != NULL) gd_backend_timer_destroy(timer);
-    if (st == GD_OK) {
-        for (b = 0; b < d->cfg.batch; ++b) d->pos[b] += n_steps;
-    }
+    if (step_ms != NULL) *step_ms = n_steps > 1 ? ms / (float)(n_steps - 1) : 0.0f;
     return st;
 }

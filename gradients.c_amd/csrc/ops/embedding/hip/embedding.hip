@@ -65,7 +65,8 @@ extern "C" int gd_hip_launch_add_scalar_i32(hipStream_t stream, const int32_t *s
 __global__ void __launch_bounds__(256)
 gd_decode_advance_kernel(const int32_t *__restrict__ next_ids, const float *__restrict__ gaps, int32_t *__restrict__ ids,
                          int32_t *__restrict__ positions, int32_t *__restrict__ step_counter,
-                         int32_t *__restrict__ out_ids, float *__restrict__ out_gaps, uint32_t batch, uint32_t max_steps)
+                         int32_t *__restrict__ out_ids, float *__restrict__ out_gaps, uint32_t batch, uint32_t max_steps,
+                         int32_t pos_delta)
 {
     /* one workgroup: every thread reads the counter before thread 0 advances it */
     const int32_t s = *step_counter;
@@ -73,7 +74,7 @@ gd_decode_advance_kernel(const int32_t *__restrict__ next_ids, const float *__re
     for (uint32_t b = threadIdx.x; b < batch; b += blockDim.x) {
         const int32_t t = next_ids[b];
         ids[b] = t;
-        positions[b] += 1;
+        positions[b] += pos_delta;
         if (s >= 0 && (uint32_t)s < max_steps) {
             out_ids[(size_t)s * batch + b] = t;
             if (out_gaps != nullptr) out_gaps[(size_t)s * batch + b] = gaps[b];
@@ -84,9 +85,9 @@ gd_decode_advance_kernel(const int32_t *__restrict__ next_ids, const float *__re
 
 extern "C" int gd_hip_launch_decode_advance(hipStream_t stream, const int32_t *next_ids, const float *gaps, int32_t *ids,
                                             int32_t *positions, int32_t *step_counter, int32_t *out_ids,
-                                            float *out_gaps, uint32_t batch, uint32_t max_steps)
+                                            float *out_gaps, uint32_t batch, uint32_t max_steps, int32_t pos_delta)
 {
     gd_decode_advance_kernel<<<1, 256, 0, stream>>>(next_ids, gaps, ids, positions, step_counter, out_ids, out_gaps,
-                                                     batch, max_steps);
+                                                     batch, max_steps, pos_delta);
     return (int)hipGetLastError();
 }

@@ -10,7 +10,7 @@ int gd_hip_launch_gather_rows(hipStream_t stream, const void *table, const int32
 int gd_hip_launch_add_scalar_i32(hipStream_t stream, const int32_t *src, int32_t *dst, uint64_t n, int32_t delta);
 int gd_hip_launch_decode_advance(hipStream_t stream, const int32_t *next_ids, const float *gaps, int32_t *ids,
                                  int32_t *positions, int32_t *step_counter, int32_t *out_ids, float *out_gaps,
-                                 uint32_t batch, uint32_t max_steps);
+                                 uint32_t batch, uint32_t max_steps, int32_t pos_delta);
 
 static gd_status gather(gd_backend *backend, const gd_backend_tensor_view *table, const gd_backend_tensor_view *ids,
                         const gd_backend_tensor_view *out, uint64_t n_ids, uint64_t vocab, uint64_t dim, int nan)
@@ -66,7 +66,8 @@ static bool i32_ok(const gd_backend_tensor_view *v)
 gd_status gd_backend_decode_advance(gd_backend *backend, const gd_backend_tensor_view *next_ids,
                                     const gd_backend_tensor_view *gaps, const gd_backend_tensor_view *ids,
                                     const gd_backend_tensor_view *positions, const gd_backend_tensor_view *step_counter,
-                                    const gd_backend_tensor_view *out_ids, const gd_backend_tensor_view *out_gaps)
+                                    const gd_backend_tensor_view *out_ids, const gd_backend_tensor_view *out_gaps,
+                                    int32_t pos_delta)
 {
     size_t batch;
     if (backend == NULL || !i32_ok(next_ids) || !i32_ok(ids) || !i32_ok(positions) || !i32_ok(step_counter) ||
@@ -84,5 +85,5 @@ gd_status gd_backend_decode_advance(gd_backend *backend, const gd_backend_tensor
         backend->stream, (const int32_t *)gd_hip_view_ptr(next_ids), gaps != NULL ? (const float *)gd_hip_view_ptr(gaps) : NULL,
         (int32_t *)gd_hip_view_ptr(ids), (int32_t *)gd_hip_view_ptr(positions), (int32_t *)gd_hip_view_ptr(step_counter),
         (int32_t *)gd_hip_view_ptr(out_ids), out_gaps != NULL ? (float *)gd_hip_view_ptr(out_gaps) : NULL,
-        (uint32_t)batch, (uint32_t)(out_ids->count / batch)));
+        (uint32_t)batch, (uint32_t)(out_ids->count / batch), pos_delta));
 }

@@ -118,6 +118,10 @@ def lib():
         l.gd_gpt_decoder_prefill.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp]
         l.gd_gpt_decoder_step.argtypes = [_vp, _vp, _vp, _vp, _vp]
         l.gd_gpt_decoder_run_resident.argtypes = [_vp, _vp, C.c_int32, _vp, _vp, C.POINTER(C.c_float)]
+        l.gd_gpt_decoder_resident_begin.argtypes = [_vp, _vp, C.c_int32, C.c_int32]
+        l.gd_gpt_decoder_resident_run.argtypes = [_vp, C.c_int32]
+        l.gd_gpt_decoder_resident_sync.argtypes = [_vp]
+        l.gd_gpt_decoder_resident_end.argtypes = [_vp, _vp, _vp, C.POINTER(C.c_int32)]
         _declared = True
     return l
 
@@ -142,6 +146,11 @@ class Context:
         if self.handle:
             lib().gd_context_destroy(self.handle)
             self.handle = None
+
+    def backend(self):
+        """Borrowed Backend wrapper around gd_context_backend (for timers and raw operator calls)."""
+        from . import Backend
+        return Backend(lib().gd_context_backend(self.handle))
 
     def check(self, st, what):
         if st != GD_OK:
@@ -188,8 +197,11 @@ class GptDecoder:
         l = lib()
         rows = max(cfg.batch, max_prefill_tokens)
         if scratch_slot_bytes is None:
-            per_row = 2 * (3 * cfg.d_model * 3 + 2 * cfg.mlp_hidden + 10 * cfg.d_model) + 64
-            scratch_slot_bytes = 2 * (rows * per_row + cfg.batch * cfg.vocab * 2) + (64 << 20)
+            # every operator output of every layer lives until the step ends (bump allocation):
+            # 13 d_model-wide and one 2*hidden-wide F16 tensor per layer and row, 256-byte padded
+            per_row = 2 * (13 * cfg.d_model + 2 * cfg.mlp_hidden) + 14 * 256
+            scratch_slot_bytes = (rows * per_row * cfg.n_layers * 2 + rows * cfg.d_model * 4
+                                  + cfg.batch * cfg.vocab * 4 + (64 << 20))
         self.ctx = Context(l.gd_gpt_params_bytes(C.byref(cfg)), l.gd_gpt_state_bytes(C.byref(cfg)),
                            scratch_slot_bytes, data_slot_bytes=max(1 << 20, 16 * rows + (1 << 16)))
         h = _vp()
@@ -259,3 +271,36 @@ class GptDecoder:
                                                ids.ctypes.data_as(_vp), gaps.ctypes.data_as(_vp), C.byref(ms))
         self.ctx.check(st, "gd_gpt_decoder_run_resident")
         return ids, gaps, ms.value
+
+    def resident_begin(self, first_ids, max_steps, hold_positions=False):
+        first = np.ascontiguousarray(first_ids, np.int32)
+        self._resident_max = max_steps
+        self.ctx.check(lib().gd_gpt_decoder_resident_begin(self.handle, first.ctypes.data_as(_vp), max_steps,
+                                                           int(hold_positions)), "gd_gpt_decoder_resident_begin")
+
+    def resident_run(self, n_steps):
+        self.ctx.check(lib().gd_gpt_decoder_resident_run(self.handle, n_steps), "gd_gpt_decoder_resident_run")
+
+    def resident_sync(self):
+        self.ctx.check(lib().gd_gpt_decoder_resident_sync(self.handle), "gd_gpt_decoder_resident_sync")
+
+    def resident_end(self):
+        ids = np.empty((self._resident_max, self.cfg.batch), np.int32)
+        gaps = np.empty((self._resident_max, self.cfg.batch), np.float32)
+        done = C.c_int32()
+        self.ctx.check(lib().gd_gpt_decoder_resident_end(self.handle, ids.ctypes.data_as(_vp), gaps.ctypes.data_as(_vp),
+                                                         C.byref(done)), "gd_gpt_decoder_resident_end")
+        return ids[:done.value], gaps[:done.value]
+
+
+def view_of(t):
+    """gd_backend_tensor_view of a contiguous gd_tensor (what the operator front ends build)."""
+    from . import TensorView
+    v = TensorView()
+    v.buffer, v.offset, v.dtype, v.rank = t.storage.buffer, t.storage.offset + t.view_offset, t.dtype, t.rank
+    n, st = 1, 1
+    for d in range(t.rank - 1, -1, -1):
+        v.shape[d], v.strides[d] = t.shape[d], st
+        st *= t.shape[d]
+    v.count = st
+    return v

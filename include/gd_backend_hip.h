@@ -323,7 +323,7 @@ gd_status gd_backend_add_scalar_i32(gd_backend *backend, const gd_backend_tensor
                                     const gd_backend_tensor_view *dst, int32_t delta);
 
 /* End of a device-resident greedy decode step, one launch: ids[b] = next_ids[b];
- * positions[b] += 1; s = *step_counter; when s < max_steps, out_ids[s*B + b] = next_ids[b] and
+ * positions[b] += pos_delta; s = *step_counter; when s < max_steps, out_ids[s*B + b] = next_ids[b] and
  * (out_gaps != NULL) out_gaps[s*B + b] = gaps[b]; then *step_counter = s + 1.  All tensors
  * contiguous; next_ids/ids/positions I32 [B], step_counter I32 [1], out_ids I32 [max_steps*B],
  * gaps / out_gaps F32 (both NULL or both given). */
@@ -332,7 +332,7 @@ gd_status gd_backend_decode_advance(gd_backend *backend, const gd_backend_tensor
                                     const gd_backend_tensor_view *positions,
                                     const gd_backend_tensor_view *step_counter,
                                     const gd_backend_tensor_view *out_ids,
-                                    const gd_backend_tensor_view *out_gaps);
+                                    const gd_backend_tensor_view *out_gaps, int32_t pos_delta);
 
 /* Device copy between buffers, enqueued like an operator. */
 gd_status gd_backend_copy(gd_backend *backend, gd_backend_buffer *dst, size_t dst_offset,

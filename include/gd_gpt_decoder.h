@@ -63,9 +63,24 @@ gd_status gd_gpt_decoder_prefill(gd_gpt_decoder *dec, const int32_t *ids, const 
 gd_status gd_gpt_decoder_step(gd_gpt_decoder *dec, const int32_t *ids, int32_t *next_ids, float *gaps,
                               uint16_t *logits);
 
-/* n_steps greedy steps with device-resident ids and positions, starting from first_ids [batch].
- * out_ids receives [n_steps, batch] token ids, out_gaps (may be NULL) the top-2 gaps.
- * step_ms (may be NULL) receives the mean device time per step measured with stream events. */
+/* Device-resident greedy decoding.  A session keeps token ids and cache positions on the device:
+ *   begin  uploads first_ids [batch] and the positions, opens one inference step scope, runs the
+ *          first step eagerly and captures the step into a graph;
+ *   run    enqueues n more steps (graph replays) without waiting;
+ *   sync   waits for everything enqueued;
+ *   end    closes the scope and downloads the tokens of all steps run so far: out_ids
+ *          [steps, batch] and (may be NULL) out_gaps; steps_done (may be NULL) = rows written.
+ * At most max_steps steps can run in a session.  With hold_positions != 0 the cache positions do
+ * not advance: every step appends at the same row and attends over the same number of keys (used
+ * to time one fixed-shape step repeatedly). */
+gd_status gd_gpt_decoder_resident_begin(gd_gpt_decoder *dec, const int32_t *first_ids, int32_t max_steps,
+                                        int32_t hold_positions);
+gd_status gd_gpt_decoder_resident_run(gd_gpt_decoder *dec, int32_t n_steps);
+gd_status gd_gpt_decoder_resident_sync(gd_gpt_decoder *dec);
+gd_status gd_gpt_decoder_resident_end(gd_gpt_decoder *dec, int32_t *out_ids, float *out_gaps, int32_t *steps_done);
+
+/* begin + run(n_steps - 1) + end in one call.  step_ms (may be NULL) receives the mean device time
+ * per replayed step measured with stream events. */
 gd_status gd_gpt_decoder_run_resident(gd_gpt_decoder *dec, const int32_t *first_ids, int32_t n_steps,
                                       int32_t *out_ids, float *out_gaps, float *step_ms);
 
