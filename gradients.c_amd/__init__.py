@@ -74,6 +74,10 @@ class SdpaDecodeArgs(C.Structure):
                 ("cache_pos", C.c_int32)]
 
 
+class FusedLinearArgs(C.Structure):
+    _fields_ = [("w_is_nk", C.c_uint32), ("bias_mode", C.c_uint32), ("prologue", C.c_uint32), ("eps", C.c_float)]
+
+
 class KvAppendArgs(C.Structure):
     _fields_ = [("cache_pos", C.c_int32)]
 
@@ -122,6 +126,8 @@ _SIGNATURES = {
     "gd_backend_argmax_rows": [_vp, _TV, _TV, _TV],
     "gd_backend_swiglu_split_linear": [_vp, _MV, _MV, _VV, _MV],
     "gd_backend_linear_nt": [_vp, _MV, _MV, _VV, _MV],
+    "gd_backend_fused_linear": [_vp, _MV, _MV, _VV, _MV, _VV, _MV, C.POINTER(FusedLinearArgs)],
+    "gd_backend_qkv_rope_append": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, C.c_uint32, C.c_uint32, C.POINTER(RopeArgs)],
     "gd_backend_gather_rows": [_vp, _TV, _TV, _TV],
     "gd_backend_add_scalar_i32": [_vp, _TV, _TV, C.c_int32],
     "gd_backend_decode_advance": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, _TV, C.c_int32],
@@ -393,6 +399,12 @@ class Backend:
         _check(self.call("gd_backend_swiglu_split_linear", x12.matrix(), w.matrix(),
                          bias.vector() if bias else None, y.matrix()), "gd_backend_swiglu_split_linear")
 
+    def fused_linear(self, x, w, bias, residual, norm_weight, y, w_is_nk, bias_mode, prologue, eps=0.0):
+        a = FusedLinearArgs(int(w_is_nk), bias_mode, prologue, eps)
+        _check(self.call("gd_backend_fused_linear", x.matrix(), w.matrix(), bias.vector() if bias else None,
+                         residual.matrix() if residual else None, norm_weight.vector() if norm_weight else None,
+                         y.matrix(), C.byref(a)), "gd_backend_fused_linear")
+
     def add(self, x, y, out):
         _check(self.call("gd_backend_add", x.view(), y.view(), out.view()), "gd_backend_add")
 
@@ -400,6 +412,11 @@ class Backend:
         a = RopeArgs(theta, head_dim, int(interleaved))
         _check(self.call("gd_backend_qkv_split_rope_forward", qkv.view(), pos.view(), q.view(), k.view(), v.view(),
                          n_heads, head_dim, C.byref(a)), "gd_backend_qkv_split_rope_forward")
+
+    def qkv_rope_append(self, qkv, pos, cache_pos, q, k_cache, v_cache, n_heads, head_dim, theta=10000.0):
+        a = RopeArgs(theta, head_dim, 0)
+        _check(self.call("gd_backend_qkv_rope_append", qkv.view(), pos.view(), cache_pos.view(), q.view(),
+                         k_cache.view(), v_cache.view(), n_heads, head_dim, C.byref(a)), "gd_backend_qkv_rope_append")
 
     def swiglu_split_forward(self, x12, out):
         _check(self.call("gd_backend_swiglu_split_forward", x12.view(), out.view()), "gd_backend_swiglu_split_forward")

@@ -91,6 +91,8 @@ gd_status gd_backend_create_default(gd_backend **out_backend)
     hv = getenv("GD_HIP_HOST_VISIBLE");
     b->host_visible_buffers = hv != NULL && hv[0] == '1' && hv[1] == '\0';
     b->sdpa_chunk = env_int("GD_HIP_SDPA_CHUNK", 0, 32, 1 << 20);
+    b->sdpa_waves = env_int("GD_HIP_SDPA_WAVES", 0, 4, 8);
+    b->sdpa_unroll = env_int("GD_HIP_SDPA_UNROLL", 0, 4, 8);
     *out_backend = b;
     return GD_OK;
 }
@@ -131,6 +133,12 @@ gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t 
     if (strcmp(name, "sdpa_chunk") == 0) {
         if (value < 0 || value > (1 << 20)) return GD_ERR_INVALID_ARGUMENT;
         backend->sdpa_chunk = (int)value;
+        return GD_OK;
+    }
+    if (strcmp(name, "sdpa_waves") == 0 || strcmp(name, "sdpa_unroll") == 0) {
+        if (value != 0 && value != 4 && value != 8) return GD_ERR_INVALID_ARGUMENT;
+        if (name[5] == 'w') backend->sdpa_waves = (int)value;
+        else backend->sdpa_unroll = (int)value;
         return GD_OK;
     }
     return GD_ERR_INVALID_ARGUMENT;

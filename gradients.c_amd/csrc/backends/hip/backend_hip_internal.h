@@ -31,7 +31,9 @@ struct gd_backend {
     void *attn_ws;
     size_t attn_ws_bytes;
     /* tunables read from the environment once at creation */
-    int sdpa_chunk;      /* keys per workgroup in the split-KV decode kernel */
+    int sdpa_chunk;      /* keys per workgroup in the split-KV decode kernel (0 = automatic) */
+    int sdpa_waves;      /* 4 or 8 wavefronts per workgroup (0 = default 8) */
+    int sdpa_unroll;     /* 4 or 8 key-row loads in flight per lane (0 = default 8) */
 };
 
 struct gd_backend_buffer {

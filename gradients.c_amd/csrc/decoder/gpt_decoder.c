@@ -39,7 +39,7 @@ struct gd_gpt_decoder {
     gd_tensor ids_dev, pos_dev, step_dev;
     /* open resident session */
     bool resident_open;
-    int32_t resident_max_steps, resident_steps, resident_hold;
+    int32_t resident_max_steps, resident_steps, resident_hold, resident_unfused;
     gd_backend_graph *resident_graph;
     gd_tensor resident_out_ids, resident_out_gaps;
 };
@@ -413,18 +413,142 @@ static void view1(const gd_tensor *t, gd_backend_tensor_view *v)
     v->strides[0] = 1;
 }
 
+static bool mview(const gd_tensor *t, int64_t rows, int64_t cols, gd_backend_matrix_view *m)
+{
+    m->buffer = (gd_backend_buffer *)t->storage.buffer;
+    m->offset = t->storage.offset + t->view_offset;
+    m->rows = (uint32_t)rows;
+    m->cols = (uint32_t)cols;
+    m->row_bytes = (size_t)cols * 2U;
+    m->dtype = (uint32_t)t->dtype;
+    return m->buffer != NULL;
+}
+
+static void vview(const gd_tensor *t, gd_backend_vector_view *v)
+{
+    v->buffer = (gd_backend_buffer *)t->storage.buffer;
+    v->offset = t->storage.offset + t->view_offset;
+    v->length = (uint32_t)t->shape[0];
+    v->dtype = (uint32_t)t->dtype;
+}
+
+static void tview(const gd_tensor *t, gd_backend_tensor_view *v)
+{
+    int64_t stride = 1;
+    uint32_t i;
+    memset(v, 0, sizeof(*v));
+    v->buffer = (gd_backend_buffer *)t->storage.buffer;
+    v->offset = t->storage.offset + t->view_offset;
+    v->dtype = (uint32_t)t->dtype;
+    v->rank = t->rank;
+    for (i = t->rank; i > 0U; --i) {
+        v->shape[i - 1U] = t->shape[i - 1U];
+        v->strides[i - 1U] = stride;
+        stride *= t->shape[i - 1U];
+    }
+    v->count = (size_t)stride;
+}
+
+static gd_status scratch_f16(gd_context *ctx, int64_t rows, int64_t cols, gd_tensor *out)
+{
+    int64_t dims[2] = {rows, cols};
+    return gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F16, gd_shape_make(2U, dims), 256U, out);
+}
+
+/* y = [residual +] bias_mode(prologue(x) @ w) through gd_backend_fused_linear */
+static gd_status fused_project(gd_gpt_decoder *d, const gd_tensor *x, int64_t x_cols, const gpt_linear *lin,
+                               const gd_tensor *w_override, const gd_tensor *bias, const gd_tensor *residual,
+                               const gd_tensor *norm_w, uint32_t prologue, int64_t n_out, gd_tensor *y)
+{
+    gd_backend_matrix_view xm, wm, rm, ym;
+    gd_backend_vector_view bv, nv;
+    gd_backend_fused_linear_args a;
+    const gd_tensor *w = w_override != NULL ? w_override : &lin->weight;
+    const int64_t B = d->cfg.batch;
+    gd_status st;
+    TRY(scratch_f16(d->ctx, B, n_out, y));
+    mview(x, B, x_cols, &xm);
+    mview(w, w->shape[0], w->shape[1], &wm);
+    mview(y, B, n_out, &ym);
+    if (residual != NULL) mview(residual, B, n_out, &rm);
+    if (norm_w != NULL) vview(norm_w, &nv);
+    vview(bias, &bv);
+    a.w_is_nk = lin->transposed ? 1U : 0U;
+    a.bias_mode = lin->transposed ? 2U : 1U; /* [N,K]: matmul_nt + add (two roundings); [K,N]: fused F32 bias */
+    a.prologue = prologue;
+    a.eps = d->cfg.rms_eps;
+    st = gd_backend_fused_linear(gd_context_backend(d->ctx), &xm, &wm, &bv, residual != NULL ? &rm : NULL,
+                                 norm_w != NULL ? &nv : NULL, &ym, &a);
+    return st;
+}
+
+/* The decode step with the fused backend entry points: same operators, same rounding points as
+ * block_decode, 6 launches per layer. */
+static gd_status enqueue_fused_step(gd_gpt_decoder *d, gd_tensor *logits)
+{
+    gd_context *ctx = d->ctx;
+    gd_backend *be = gd_context_backend(ctx);
+    const gd_gpt_config *c = &d->cfg;
+    const gd_backend_rope_args rope = {c->rope_theta, (uint32_t)c->head_dim, 0U};
+    const gd_sdpa_decode_config sdpa = {0.0f, c->sdpa_window, 0};
+    const int64_t B = c->batch, Dm = c->d_model, Hm = c->mlp_hidden;
+    gd_tensor x, qkv, q, q4, attn, x1, ug, x2;
+    gd_backend_tensor_view vqkv, vpos, vq, vk, vv;
+    int64_t q_shape[4] = {B, 1, c->n_heads, c->head_dim};
+    int32_t l;
+    TRY(gd_embedding(ctx, &d->token_embedding, &d->ids_dev, &x));
+    for (l = 0; l < c->n_layers; ++l) {
+        const gpt_block *b = &d->blocks[l];
+        TRY(fused_project(d, &x, Dm, &b->qkv_proj, NULL, &b->qkv_proj.bias, NULL, &b->attn_norm_w, 2U, 3 * Dm, &qkv));
+        TRY(scratch_f16(ctx, B, Dm, &q));
+        tview(&qkv, &vqkv);
+        tview(&d->pos_dev, &vpos);
+        tview(&d->k_cache[l], &vk);
+        tview(&d->v_cache[l], &vv);
+        memset(&vq, 0, sizeof(vq));
+        vq.buffer = (gd_backend_buffer *)q.storage.buffer;
+        vq.offset = q.storage.offset;
+        vq.count = (size_t)(B * Dm);
+        vq.dtype = (uint32_t)GD_DTYPE_F16;
+        vq.rank = 3U;
+        vq.shape[0] = B; vq.shape[1] = c->n_heads; vq.shape[2] = c->head_dim;
+        vq.strides[0] = Dm; vq.strides[1] = c->head_dim; vq.strides[2] = 1;
+        TRY(gd_backend_qkv_rope_append(be, &vqkv, &vpos, &vpos, &vq, &vk, &vv, (uint32_t)c->n_heads,
+                                       (uint32_t)c->head_dim, &rope));
+        TRY(gd_reshape(ctx, &q, gd_shape_make(4U, q_shape), &q4));
+        TRY(gd_sdpa_decode_positions(ctx, &q4, &d->k_cache[l], &d->v_cache[l], &d->pos_dev, &sdpa, &attn));
+        TRY(fused_project(d, &attn, Dm, &b->attn_proj, NULL, &b->attn_proj.bias, &x, NULL, 0U, Dm, &x1));
+        TRY(fused_project(d, &x1, Dm, &b->up_gate, NULL, &b->up_gate.bias, NULL, &b->mlp_norm_w, 2U, 2 * Hm, &ug));
+        TRY(fused_project(d, &ug, 2 * Hm, &b->down_proj, NULL, &b->down_proj.bias, &x1, NULL, 1U, Dm, &x2));
+        x = x2;
+    }
+    {
+        gpt_linear head_lin;
+        head_lin.weight = d->lm_head;
+        head_lin.bias = d->lm_head_bias;
+        head_lin.transposed = true;
+        TRY(fused_project(d, &x, Dm, &head_lin, NULL, &d->lm_head_bias, NULL, &d->final_norm_w, 2U, c->vocab, logits));
+    }
+    return GD_OK;
+}
+
 static gd_status enqueue_resident_step(gd_gpt_decoder *d)
 {
     gd_context *ctx = d->ctx;
     gd_tensor x, y, logits, next, gaps;
     gd_backend_tensor_view vn, vg, vi, vp, vs, vo, vog;
     int32_t l;
-    TRY(gd_embedding(ctx, &d->token_embedding, &d->ids_dev, &x));
-    for (l = 0; l < d->cfg.n_layers; ++l) {
-        TRY(block_decode(d, l, &x, &d->pos_dev, &d->pos_dev, &y));
-        x = y;
+    if (d->resident_unfused) {
+        TRY(gd_embedding(ctx, &d->token_embedding, &d->ids_dev, &x));
+        for (l = 0; l < d->cfg.n_layers; ++l) {
+            TRY(block_decode(d, l, &x, &d->pos_dev, &d->pos_dev, &y));
+            x = y;
+        }
+        TRY(head(d, &x, &logits, &next, &gaps));
+    } else {
+        TRY(enqueue_fused_step(d, &logits));
+        TRY(gd_argmax_rows(ctx, &logits, &next, &gaps));
     }
-    TRY(head(d, &x, &logits, &next, &gaps));
     view1(&next, &vn);
     view1(&gaps, &vg);
     view1(&d->ids_dev, &vi);
@@ -445,8 +569,9 @@ static void resident_abort(gd_gpt_decoder *d)
 }
 
 gd_status gd_gpt_decoder_resident_begin(gd_gpt_decoder *d, const int32_t *first_ids, int32_t max_steps,
-                                        int32_t hold_positions)
+                                        int32_t flags)
 {
+    const int32_t hold_positions = flags & GD_GPT_RESIDENT_HOLD_POSITIONS;
     gd_context *ctx;
     gd_backend *be;
     gd_status st;
@@ -468,6 +593,8 @@ gd_status gd_gpt_decoder_resident_begin(gd_gpt_decoder *d, const int32_t *first_
     d->resident_max_steps = max_steps;
     d->resident_steps = 0;
     d->resident_hold = hold_positions != 0;
+    /* the fused rope + append kernel needs NeoX pairs of a head size that is a multiple of 16 */
+    d->resident_unfused = (flags & GD_GPT_RESIDENT_UNFUSED) != 0 || (d->cfg.head_dim % 16) != 0;
     dims[0] = (int64_t)max_steps * d->cfg.batch;
     st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_I32, gd_shape_make(1U, dims), 256U, &d->resident_out_ids);
     if (st == GD_OK) st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F32, gd_shape_make(1U, dims), 256U, &d->resident_out_gaps);

@@ -7,22 +7,27 @@
 #include "hip_linear_types.h"
 
 int gd_hip_launch_linear(hipStream_t stream, const void *x, const void *w, const void *bias, const void *residual,
-                         void *y, const gd_hip_linear_params *params, int vector_ok);
+                         const void *norm_w, void *y, const gd_hip_linear_params *params, int vector_ok,
+                         int min_workgroups);
 
-static gd_status project(gd_backend *backend, const gd_backend_matrix_view *x, const gd_backend_matrix_view *w,
-                         const gd_backend_vector_view *bias, const gd_backend_matrix_view *y, uint32_t w_is_nk,
-                         uint32_t epilogue, uint32_t swiglu)
+static gd_status project_full(gd_backend *backend, const gd_backend_matrix_view *x, const gd_backend_matrix_view *w,
+                              const gd_backend_vector_view *bias, const gd_backend_matrix_view *residual,
+                              const gd_backend_vector_view *norm_w, float eps, const gd_backend_matrix_view *y,
+                              uint32_t w_is_nk, uint32_t epilogue, uint32_t prologue)
 {
     gd_hip_linear_params p;
     uint32_t K;
     int vec;
     if (backend == NULL || !gd_hip_matrix_ok(x) || !gd_hip_matrix_ok(w) || !gd_hip_matrix_ok(y) ||
-        (bias != NULL && !gd_hip_vector_ok(bias)))
+        (bias != NULL && !gd_hip_vector_ok(bias)) || (residual != NULL && !gd_hip_matrix_ok(residual)) ||
+        (norm_w != NULL && !gd_hip_vector_ok(norm_w)))
         return GD_ERR_INVALID_ARGUMENT;
     if (x->dtype != GD_BACKEND_DTYPE_F16 || w->dtype != GD_BACKEND_DTYPE_F16 || y->dtype != GD_BACKEND_DTYPE_F16 ||
-        (bias != NULL && bias->dtype != GD_BACKEND_DTYPE_F16))
+        (bias != NULL && bias->dtype != GD_BACKEND_DTYPE_F16) ||
+        (residual != NULL && residual->dtype != GD_BACKEND_DTYPE_F16) ||
+        (norm_w != NULL && norm_w->dtype != GD_BACKEND_DTYPE_F16))
         return GD_ERR_UNSUPPORTED;
-    if (swiglu) {
+    if (prologue == GD_HIP_PRO_SWIGLU) {
         if ((x->cols & 1u) != 0u) return GD_ERR_INVALID_ARGUMENT;
         K = x->cols / 2u;
     } else {
@@ -30,9 +35,12 @@ static gd_status project(gd_backend *backend, const gd_backend_matrix_view *x, c
     }
     if (w_is_nk ? (w->cols != K || w->rows != y->cols) : (w->rows != K || w->cols != y->cols))
         return GD_ERR_INVALID_ARGUMENT;
-    if (x->rows != y->rows || (bias != NULL && bias->length != y->cols)) return GD_ERR_INVALID_ARGUMENT;
+    if (x->rows != y->rows || (bias != NULL && bias->length != y->cols) ||
+        (residual != NULL && (residual->rows != y->rows || residual->cols != y->cols)) ||
+        ((prologue == GD_HIP_PRO_RMS_NORM) != (norm_w != NULL)) || (norm_w != NULL && (norm_w->length != K || !(eps > 0.0f))))
+        return GD_ERR_INVALID_ARGUMENT;
     if ((uint64_t)y->rows * y->cols > 0x7fffffffull * 256u || (y->cols + 15u) / 16u > 0x7fffffffu ||
-        (y->rows + 15u) / 16u > 65535u * 4u)
+        (y->rows + 15u) / 16u > 65535u)
         return GD_ERR_UNSUPPORTED;
     p.M = y->rows;
     p.N = y->cols;
@@ -42,15 +50,25 @@ static gd_status project(gd_backend *backend, const gd_backend_matrix_view *x, c
     p.ldy = (uint32_t)(y->row_bytes / 2u);
     p.epilogue = bias != NULL ? epilogue : GD_HIP_EPI_NONE;
     p.w_is_nk = w_is_nk;
-    p.swiglu = swiglu;
-    p.has_residual = 0u;
-    p.ldr = 0u;
-    /* 16-byte fragment loads: x rows always, w rows when K-contiguous */
+    p.prologue = prologue;
+    p.has_residual = residual != NULL ? 1u : 0u;
+    p.ldr = residual != NULL ? (uint32_t)(residual->row_bytes / 2u) : 0u;
+    p.eps = eps;
+    /* 16-byte fragment loads: x rows always, w rows when K-contiguous, the norm weight */
     vec = (K % 8u) == 0u && ((x->offset | x->row_bytes) & 15u) == 0u &&
-          (!w_is_nk || ((w->offset | w->row_bytes) & 15u) == 0u);
+          (!w_is_nk || ((w->offset | w->row_bytes) & 15u) == 0u) && (norm_w == NULL || (norm_w->offset & 15u) == 0u);
     return gd_hip_finish_op(backend, gd_hip_launch_linear(
         backend->stream, gd_hip_matrix_ptr(x), gd_hip_matrix_ptr(w), bias != NULL ? gd_hip_vector_ptr(bias) : NULL,
-        NULL, gd_hip_matrix_ptr(y), &p, vec));
+        residual != NULL ? gd_hip_matrix_ptr(residual) : NULL, norm_w != NULL ? gd_hip_vector_ptr(norm_w) : NULL,
+        gd_hip_matrix_ptr(y), &p, vec, 2 * backend->compute_units));
+}
+
+static gd_status project(gd_backend *backend, const gd_backend_matrix_view *x, const gd_backend_matrix_view *w,
+                         const gd_backend_vector_view *bias, const gd_backend_matrix_view *y, uint32_t w_is_nk,
+                         uint32_t epilogue, uint32_t swiglu)
+{
+    return project_full(backend, x, w, bias, NULL, NULL, 0.0f, y, w_is_nk, epilogue,
+                        swiglu ? GD_HIP_PRO_SWIGLU : GD_HIP_PRO_NONE);
 }
 
 gd_status gd_backend_matmul(gd_backend *backend, const gd_backend_matrix_view *x, const gd_backend_matrix_view *w,
@@ -84,4 +102,15 @@ gd_status gd_backend_swiglu_split_linear(gd_backend *backend, const gd_backend_m
                                          const gd_backend_matrix_view *y)
 {
     return project(backend, x12, w, bias, y, 0u, GD_HIP_EPI_BIAS_F32, 1u);
+}
+
+gd_status gd_backend_fused_linear(gd_backend *backend, const gd_backend_matrix_view *x,
+                                  const gd_backend_matrix_view *w, const gd_backend_vector_view *bias,
+                                  const gd_backend_matrix_view *residual, const gd_backend_vector_view *norm_weight,
+                                  const gd_backend_matrix_view *y, const gd_backend_fused_linear_args *args)
+{
+    if (args == NULL || args->bias_mode > 2u || args->prologue > 2u || (args->bias_mode != 0u) != (bias != NULL))
+        return GD_ERR_INVALID_ARGUMENT;
+    return project_full(backend, x, w, bias, residual, norm_weight, args->eps, y, args->w_is_nk != 0u, args->bias_mode,
+                        args->prologue);
 }

@@ -7,14 +7,20 @@
 #define GD_HIP_EPI_BIAS_F32 1u    /* y = half(acc + bias)            (gd_backend_linear) */
 #define GD_HIP_EPI_BIAS_F16 2u    /* y = half(half(acc) + bias)      (matmul_nt then add) */
 
+/* prologue applied to the activation operand before it enters the MFMA, rounded to F16 */
+#define GD_HIP_PRO_NONE 0u
+#define GD_HIP_PRO_SWIGLU 1u      /* a = half(x[:, k] * silu(x[:, K + k])), x has 2K columns */
+#define GD_HIP_PRO_RMS_NORM 2u    /* a = half(x[:, k] * norm_w[k] * rsqrt(mean(x^2) + eps)) */
+
 typedef struct gd_hip_linear_params {
     uint32_t M, N, K;
     uint32_t ldx, ldw, ldy; /* row pitch in elements */
     uint32_t epilogue;
     uint32_t w_is_nk;       /* 1: w stored [N,K] (x w^T); 0: w stored [K,N] */
-    uint32_t swiglu;        /* 1: A operand = half(x[:, :K] * silu(x[:, K:2K])) */
-    uint32_t has_residual;  /* 1: y = half(epilogue(acc) + residual) with residual [M,N] pitch ldr */
+    uint32_t prologue;
+    uint32_t has_residual;  /* 1: y = half(epilogue(acc)) + residual, residual [M,N] pitch ldr */
     uint32_t ldr;
+    float eps;              /* rms_norm prologue */
 } gd_hip_linear_params;
 
 #endif

@@ -11,10 +11,27 @@
  */
 #include "../../_shared/hip_device.h"
 
+/* Explicitly rounded steps so every kernel of this file produces the same bits for the same input. */
+__device__ __forceinline__ void gd_rope_cos_sin(float fpos, uint32_t pair, float freq_scale, float *c, float *s)
+{
+    sincosf(__fmul_rn(fpos, exp2f(__fmul_rn((float)pair, freq_scale))), s, c);
+}
+
+__device__ __forceinline__ void gd_rope_rotate(float x0, float x1, float c, float s, gd_half *o0, gd_half *o1)
+{
+    *o0 = (gd_half)__fmaf_rn(x0, c, -__fmul_rn(x1, s));
+    *o1 = (gd_half)__fmaf_rn(x0, s, __fmul_rn(x1, c));
+}
+
+/* cache_pos == nullptr: k and v go to row n of [N,H,D] tensors (split form).  Otherwise they go to
+ * row cache_pos[n] of sequence n in [N,Tmax,H,D] caches (decode form, one new token per sequence);
+ * a sequence whose position is negative or >= tmax keeps its caches untouched, like the append
+ * kernel.  One kernel serves both forms so that both produce the same bits. */
 __global__ void __launch_bounds__(256)
 gd_qkv_split_rope_neox_vec_kernel(const gd_half *__restrict__ qkv, const int32_t *__restrict__ pos,
-                                  gd_half *__restrict__ q, gd_half *__restrict__ k, gd_half *__restrict__ v,
-                                  uint64_t tokens, uint32_t heads, uint32_t head_dim, float freq_scale)
+                                  const int32_t *__restrict__ cache_pos, gd_half *__restrict__ q,
+                                  gd_half *__restrict__ k, gd_half *__restrict__ v, uint64_t tokens, uint32_t heads,
+                                  uint32_t head_dim, uint32_t tmax, float freq_scale)
 {
     const uint32_t half_d = head_dim / 2u, groups = half_d / 8u; /* 8-pair groups per head */
     const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -25,14 +42,19 @@ gd_qkv_split_rope_neox_vec_kernel(const gd_half *__restrict__ qkv, const int32_t
     const uint64_t n = gid / ((uint64_t)groups * heads);
     const uint64_t area = (uint64_t)heads * head_dim;
     const gd_half *src = qkv + n * 3u * area + (uint64_t)h * head_dim + grp * 8u;
-    const uint64_t dst = n * area + (uint64_t)h * head_dim + grp * 8u;
+    const uint64_t within = (uint64_t)h * head_dim + grp * 8u;
+    const uint64_t qdst = n * area + within;
+    bool store_kv = true;
+    uint64_t kvdst = qdst;
+    if (cache_pos != nullptr) {
+        const int32_t cp = cache_pos[n];
+        store_kv = cp >= 0 && (uint32_t)cp < tmax;
+        kvdst = (n * tmax + (uint64_t)(store_kv ? cp : 0)) * area + within;
+    }
     const float fpos = (float)pos[n];
     float c[8], s[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        const float angle = fpos * exp2f((float)(grp * 8u + e) * freq_scale);
-        sincosf(angle, &s[e], &c[e]);
-    }
+    for (int e = 0; e < 8; ++e) gd_rope_cos_sin(fpos, grp * 8u + e, freq_scale, &c[e], &s[e]);
 #pragma unroll
     for (int which = 0; which < 2; ++which) {
         const gd_half8 lo = *reinterpret_cast<const gd_half8 *>(src + which * area);
@@ -40,16 +62,23 @@ gd_qkv_split_rope_neox_vec_kernel(const gd_half *__restrict__ qkv, const int32_t
         gd_half8 olo, ohi;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            const float x0 = (float)lo[e], x1 = (float)hi[e];
-            olo[e] = (gd_half)(x0 * c[e] - x1 * s[e]);
-            ohi[e] = (gd_half)(x0 * s[e] + x1 * c[e]);
+            gd_half a, b;
+            gd_rope_rotate((float)lo[e], (float)hi[e], c[e], s[e], &a, &b);
+            olo[e] = a;
+            ohi[e] = b;
         }
-        gd_half *o = which == 0 ? q : k;
-        *reinterpret_cast<gd_half8 *>(o + dst) = olo;
-        *reinterpret_cast<gd_half8 *>(o + dst + half_d) = ohi;
+        if (which == 0) {
+            *reinterpret_cast<gd_half8 *>(q + qdst) = olo;
+            *reinterpret_cast<gd_half8 *>(q + qdst + half_d) = ohi;
+        } else if (store_kv) {
+            *reinterpret_cast<gd_half8 *>(k + kvdst) = olo;
+            *reinterpret_cast<gd_half8 *>(k + kvdst + half_d) = ohi;
+        }
     }
-    *reinterpret_cast<gd_u128 *>(v + dst) = *reinterpret_cast<const gd_u128 *>(src + 2u * area);
-    *reinterpret_cast<gd_u128 *>(v + dst + half_d) = *reinterpret_cast<const gd_u128 *>(src + 2u * area + half_d);
+    if (store_kv) {
+        *reinterpret_cast<gd_u128 *>(v + kvdst) = *reinterpret_cast<const gd_u128 *>(src + 2u * area);
+        *reinterpret_cast<gd_u128 *>(v + kvdst + half_d) = *reinterpret_cast<const gd_u128 *>(src + 2u * area + half_d);
+    }
 }
 
 /* any even head size, either pairing: one thread per (token, head, pair) */
@@ -71,15 +100,25 @@ gd_qkv_split_rope_scalar_kernel(const gd_half *__restrict__ qkv, const int32_t *
     const gd_half *src = qkv + n * 3u * area + (uint64_t)h * head_dim;
     const uint64_t dst = n * area + (uint64_t)h * head_dim;
     float s, c;
-    sincosf((float)pos[n] * exp2f((float)pair * freq_scale), &s, &c);
-    const float q0 = (float)src[a], q1 = (float)src[b];
-    const float k0 = (float)src[area + a], k1 = (float)src[area + b];
-    q[dst + a] = (gd_half)(q0 * c - q1 * s);
-    q[dst + b] = (gd_half)(q0 * s + q1 * c);
-    k[dst + a] = (gd_half)(k0 * c - k1 * s);
-    k[dst + b] = (gd_half)(k0 * s + k1 * c);
+    gd_rope_cos_sin((float)pos[n], pair, freq_scale, &c, &s);
+    gd_rope_rotate((float)src[a], (float)src[b], c, s, &q[dst + a], &q[dst + b]);
+    gd_rope_rotate((float)src[area + a], (float)src[area + b], c, s, &k[dst + a], &k[dst + b]);
     v[dst + a] = src[2u * area + a];
     v[dst + b] = src[2u * area + b];
+}
+
+extern "C" int gd_hip_launch_qkv_rope_append(hipStream_t stream, const void *qkv, const int32_t *rope_pos,
+                                             const int32_t *cache_pos, void *q, void *k_cache, void *v_cache,
+                                             uint64_t tokens, uint32_t heads, uint32_t head_dim, uint32_t tmax,
+                                             float theta)
+{
+    const float freq_scale = -2.0f * log2f(theta) / (float)head_dim;
+    const uint64_t total = tokens * heads * (head_dim / 16u);
+    if (total == 0) return (int)hipSuccess;
+    gd_qkv_split_rope_neox_vec_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(
+        (const gd_half *)qkv, rope_pos, cache_pos, (gd_half *)q, (gd_half *)k_cache, (gd_half *)v_cache, tokens, heads,
+        head_dim, tmax, freq_scale);
+    return (int)hipGetLastError();
 }
 
 extern "C" int gd_hip_launch_qkv_split_rope(hipStream_t stream, const void *qkv, const int32_t *pos, void *q,
@@ -91,7 +130,8 @@ extern "C" int gd_hip_launch_qkv_split_rope(hipStream_t stream, const void *qkv,
     if (!interleaved && aligned16 && (head_dim % 16u) == 0u) {
         const uint64_t total = tokens * heads * (head_dim / 16u);
         gd_qkv_split_rope_neox_vec_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(
-            (const gd_half *)qkv, pos, (gd_half *)q, (gd_half *)k, (gd_half *)v, tokens, heads, head_dim, freq_scale);
+            (const gd_half *)qkv, pos, nullptr, (gd_half *)q, (gd_half *)k, (gd_half *)v, tokens, heads, head_dim, 0u,
+            freq_scale);
     } else {
         const uint64_t total = tokens * heads * (head_dim / 2u);
         gd_qkv_split_rope_scalar_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(

@@ -62,6 +62,8 @@ static gd_status dispatch(gd_backend *backend, const gd_backend_tensor_view *q, 
     p.dtype = q->dtype;
     p.chunk = 0u;
     p.nsplit = 1u;
+    p.waves = backend->sdpa_waves == 4 ? 4u : 8u;
+    p.unroll = backend->sdpa_unroll == 4 ? 4u : 8u;
     group = p.hq / p.hkv;
     if (q->dtype == GD_BACKEND_DTYPE_F16 && p.tq == 1u && (p.dh == 64u || p.dh == 128u) && p.prefix_len == 0u &&
         (group == 1u || group == 2u || group == 4u || group == 8u) &&
@@ -71,11 +73,11 @@ static gd_status dispatch(gd_backend *backend, const gd_backend_tensor_view *q, 
         uint32_t chunk = (uint32_t)backend->sdpa_chunk;
         gd_status st;
         if (chunk == 0u) {
-            /* aim at >= 4 workgroups per compute unit, never less than 256 keys per workgroup */
+            /* aim at >= 2 workgroups per compute unit, never less than 512 keys per workgroup */
             const uint64_t pairs = (uint64_t)p.batch * p.hkv;
-            const uint64_t want = ((uint64_t)backend->compute_units * 4u + pairs - 1u) / pairs;
+            const uint64_t want = ((uint64_t)backend->compute_units * 2u + pairs - 1u) / pairs;
             chunk = (uint32_t)((span + want - 1u) / want);
-            if (chunk < 256u) chunk = 256u;
+            if (chunk < 512u) chunk = 512u;
         }
         chunk = (chunk + 31u) & ~31u;
         if (chunk > span) chunk = (span + 31u) & ~31u;

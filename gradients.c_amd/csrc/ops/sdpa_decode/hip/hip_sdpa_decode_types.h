@@ -15,6 +15,8 @@ typedef struct gd_hip_sdpa_decode_params {
     uint32_t chunk;  /* keys per workgroup (split-KV kernel) */
     uint32_t nsplit; /* workgroups per (batch, kv head) */
     uint32_t dtype;  /* GD_BACKEND_DTYPE_F16 or _F32 (generic kernel) */
+    uint32_t waves;  /* wavefronts per workgroup of the split-KV kernel: 4 or 8 */
+    uint32_t unroll; /* key-row loads in flight per lane: 4 or 8 */
 } gd_hip_sdpa_decode_params;
 
 #endif

@@ -57,18 +57,34 @@ __device__ __forceinline__ int gd_decode_pos(const int32_t *pos, const gd_hip_sd
 
 /* ---- split-KV kernel ----------------------------------------------------------- */
 
-#define GD_SDPA_WAVES 4
+/* Sum over aligned groups of N (8 or 16) consecutive lanes; every lane of a group receives the total.
+ * Data-parallel-primitive adds (lane swaps inside a row of 16 lanes) instead of LDS shuffles:
+ * swap neighbours, swap pairs, mirror the 8-lane half row, and for 16 lanes mirror the row. */
+template <int CTRL>
+__device__ __forceinline__ float gd_dpp_add(float x)
+{
+    return x + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));
+}
 
-template <int D, int G>
-__global__ void __launch_bounds__(GD_SDPA_WAVES * 64)
+template <int N>
+__device__ __forceinline__ float gd_row_group_sum(float x)
+{
+    x = gd_dpp_add<0xB1>(x);  /* quad_perm [1,0,3,2] */
+    x = gd_dpp_add<0x4E>(x);  /* quad_perm [2,3,0,1] */
+    x = gd_dpp_add<0x141>(x); /* row_half_mirror */
+    if (N == 16) x = gd_dpp_add<0x140>(x); /* row_mirror */
+    return x;
+}
+
+template <int D, int G, int WAVES, int UNROLL>
+__global__ void __launch_bounds__(WAVES * 64)
 gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__restrict__ kc,
                             const gd_half *__restrict__ vc, const int32_t *__restrict__ pos_ptr,
                             gd_half *__restrict__ out, float *__restrict__ ws, gd_hip_sdpa_decode_params p)
 {
     constexpr int LPK = D / 8;      /* lanes per key row */
     constexpr int KPW = 64 / LPK;   /* key rows per wavefront load */
-    constexpr int KPB = KPW * GD_SDPA_WAVES;
-    constexpr int UNROLL = 4;
+    constexpr int KPB = KPW * WAVES;
     const int split = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int slot = lane / LPK, sub = lane % LPK;
@@ -88,20 +104,22 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
                 w[1] = 0.f;
             }
         } else {
-            for (int idx = threadIdx.x; idx < G * D; idx += GD_SDPA_WAVES * 64)
+            for (int idx = threadIdx.x; idx < G * D; idx += WAVES * 64)
                 out[((size_t)b * p.hq + (size_t)hkv * G) * D + idx] = (gd_half)0.f;
         }
         return;
     }
 
-    /* query rows of the G heads that share this kv head, pre-scaled into the exp2 domain */
+    /* query rows of the G heads that share this kv head stay in F16: products of two halfs are
+     * exact in F32, so v_dot2_f32_f16 loses nothing; the softmax scale (exp2 domain) is applied
+     * to the reduced dot product */
     const float qscale = p.scale * 1.4426950408889634f;
-    float qf[G][8];
+    gd_half2 qh[G][4];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
         const gd_half8 qv = *reinterpret_cast<const gd_half8 *>(q + ((size_t)b * p.hq + (size_t)hkv * G + g) * D + sub * 8);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) qf[g][e] = (float)qv[e] * qscale;
+        for (int e = 0; e < 4; ++e) qh[g][e] = (gd_half2){qv[2 * e], qv[2 * e + 1]};
     }
 
     float m[G], l[G], acc[G][8];
@@ -117,7 +135,7 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
     const gd_half *kbase = kc + ((size_t)b * p.tmax * p.hkv + hkv) * D + sub * 8;
     const gd_half *vbase = vc + ((size_t)b * p.tmax * p.hkv + hkv) * D + sub * 8;
 
-    for (int j0 = r0 + wave * KPW + slot; j0 < r1 + 0; j0 += KPB * UNROLL) {
+    for (int j0 = r0 + wave * KPW + slot; j0 < r1; j0 += KPB * UNROLL) {
         gd_half8 kv[UNROLL], vv[UNROLL];
         bool ok[UNROLL];
 #pragma unroll
@@ -129,30 +147,34 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
             vv[u] = *reinterpret_cast<const gd_half8 *>(vbase + (size_t)jj * row_stride);
         }
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            float kf[8], vf[8];
+        for (int g = 0; g < G; ++g) {
+            /* scores of the UNROLL rows, then one rescale of the running state for all of them */
+            float sc[UNROLL];
+            float mt = GD_NEG_INF;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                kf[e] = (float)kv[u][e];
-                vf[e] = (float)vv[u][e];
+            for (int u = 0; u < UNROLL; ++u) {
+                float d = 0.f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    d = __builtin_amdgcn_fdot2(qh[g][e], (gd_half2){kv[u][2 * e], kv[u][2 * e + 1]}, d, false);
+                d = gd_row_group_sum<LPK>(d);
+                sc[u] = ok[u] ? d * qscale : GD_NEG_INF;
+                mt = fmaxf(mt, sc[u]);
             }
+            const float mn = fmaxf(m[g], mt); /* finite: the first row of a trip is always live */
+            const float corr = exp2f(m[g] - mn); /* exp2(-inf) = 0 on the first trip */
+            float lsum = l[g] * corr;
 #pragma unroll
-            for (int g = 0; g < G; ++g) {
-                float s = 0.f;
+            for (int e = 0; e < 8; ++e) acc[g][e] *= corr;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) s = fmaf(qf[g][e], kf[e], s);
+            for (int u = 0; u < UNROLL; ++u) {
+                const float pr = exp2f(sc[u] - mn); /* 0 for rows past the range */
+                lsum += pr;
 #pragma unroll
-                for (int off = 1; off < LPK; off <<= 1) s += __shfl_xor(s, off, 64);
-                if (ok[u]) {
-                    const float mn = fmaxf(m[g], s);
-                    const float corr = exp2f(m[g] - mn); /* exp2(-inf) = 0 on the first key */
-                    const float pr = exp2f(s - mn);
-                    l[g] = l[g] * corr + pr;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) acc[g][e] = acc[g][e] * corr + pr * vf[e];
-                    m[g] = mn;
-                }
+                for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(pr, (float)vv[u][e], acc[g][e]);
             }
+            l[g] = lsum;
+            m[g] = mn;
         }
     }
 
@@ -177,8 +199,8 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
     }
 
     /* merge the wavefronts through LDS */
-    __shared__ float sm_acc[GD_SDPA_WAVES][G][D];
-    __shared__ float sm_m[GD_SDPA_WAVES][G], sm_l[GD_SDPA_WAVES][G];
+    __shared__ float sm_acc[WAVES][G][D];
+    __shared__ float sm_m[WAVES][G], sm_l[WAVES][G];
     if (slot == 0) {
 #pragma unroll
         for (int g = 0; g < G; ++g) {
@@ -191,14 +213,14 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
         }
     }
     __syncthreads();
-    for (int idx = threadIdx.x; idx < G * D; idx += GD_SDPA_WAVES * 64) {
+    for (int idx = threadIdx.x; idx < G * D; idx += WAVES * 64) {
         const int g = idx / D, c = idx % D;
         float mm = GD_NEG_INF;
 #pragma unroll
-        for (int w = 0; w < GD_SDPA_WAVES; ++w) mm = fmaxf(mm, sm_m[w][g]);
+        for (int w = 0; w < WAVES; ++w) mm = fmaxf(mm, sm_m[w][g]);
         float ll = 0.f, aa = 0.f;
 #pragma unroll
-        for (int w = 0; w < GD_SDPA_WAVES; ++w) {
+        for (int w = 0; w < WAVES; ++w) {
             const float cw = (sm_m[w][g] == GD_NEG_INF) ? 0.f : exp2f(sm_m[w][g] - mm);
             ll += sm_l[w][g] * cw;
             aa += sm_acc[w][g][c] * cw;
@@ -313,8 +335,18 @@ static int launch_split(hipStream_t stream, const void *q, const void *k, const 
                         void *out, float *ws, const gd_hip_sdpa_decode_params &p)
 {
     dim3 grid(p.nsplit, p.hkv, p.batch);
-    gd_sdpa_decode_split_kernel<D, G><<<grid, GD_SDPA_WAVES * 64, 0, stream>>>(
-        (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, pos, (gd_half *)out, ws, p);
+#define GD_GO(W, U)                                                                                   \
+    gd_sdpa_decode_split_kernel<D, G, W, U><<<grid, W * 64, 0, stream>>>(                              \
+        (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, pos, (gd_half *)out, ws, p)
+    if constexpr (G == 1) {
+        if (p.waves == 8u && p.unroll == 8u) GD_GO(8, 8);
+        else if (p.waves == 8u) GD_GO(8, 4);
+        else if (p.unroll == 8u) GD_GO(4, 8);
+        else GD_GO(4, 4);
+    } else {
+        GD_GO(4, 4);
+    }
+#undef GD_GO
     if (p.nsplit > 1u) {
         dim3 cgrid(p.hq, p.batch);
         gd_sdpa_decode_combine_kernel<D><<<cgrid, D, 0, stream>>>(ws, pos, (gd_half *)out, p);

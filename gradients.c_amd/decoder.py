@@ -272,11 +272,12 @@ class GptDecoder:
         self.ctx.check(st, "gd_gpt_decoder_run_resident")
         return ids, gaps, ms.value
 
-    def resident_begin(self, first_ids, max_steps, hold_positions=False):
+    def resident_begin(self, first_ids, max_steps, hold_positions=False, unfused=False):
         first = np.ascontiguousarray(first_ids, np.int32)
         self._resident_max = max_steps
-        self.ctx.check(lib().gd_gpt_decoder_resident_begin(self.handle, first.ctypes.data_as(_vp), max_steps,
-                                                           int(hold_positions)), "gd_gpt_decoder_resident_begin")
+        flags = (1 if hold_positions else 0) | (2 if unfused else 0)
+        self.ctx.check(lib().gd_gpt_decoder_resident_begin(self.handle, first.ctypes.data_as(_vp), max_steps, flags),
+                       "gd_gpt_decoder_resident_begin")
 
     def resident_run(self, n_steps):
         self.ctx.check(lib().gd_gpt_decoder_resident_run(self.handle, n_steps), "gd_gpt_decoder_resident_run")

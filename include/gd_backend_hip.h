@@ -309,6 +309,41 @@ gd_status gd_backend_linear_nt(gd_backend *backend, const gd_backend_matrix_view
                                const gd_backend_matrix_view *w, const gd_backend_vector_view *bias,
                                const gd_backend_matrix_view *y);
 
+/* One launch for a projection together with the elementwise operators the reference issues
+ * around it in the decoder block (examples/gpt_lm/gpt_lm_shared.c:1017-1070), with the same
+ * rounding points as the separate operators:
+ *   a = x                                            prologue 0
+ *     | half(x[:, :K] * silu(x[:, K:2K]))            prologue 1 (gd_swiglu_split)
+ *     | half(x * norm_weight * rsqrt(mean(x^2)+eps)) prologue 2 (gd_rms_norm)
+ *   t = a @ w  (w [K,N])  or  a @ w^T  (w [N,K], w_is_nk = 1), F32 accumulate
+ *   u = half(t)                                      bias_mode 0 (bias must be NULL)
+ *     | half(t + bias)                               bias_mode 1 (gd_linear)
+ *     | half(half(t) + bias)                         bias_mode 2 (gd_linear_transposed_weight)
+ *   y = u, or half(residual + u) when residual != NULL (gd_add). */
+typedef struct gd_backend_fused_linear_args {
+    uint32_t w_is_nk;
+    uint32_t bias_mode;
+    uint32_t prologue;
+    float eps;
+} gd_backend_fused_linear_args;
+gd_status gd_backend_fused_linear(gd_backend *backend, const gd_backend_matrix_view *x,
+                                  const gd_backend_matrix_view *w, const gd_backend_vector_view *bias,
+                                  const gd_backend_matrix_view *residual,
+                                  const gd_backend_vector_view *norm_weight,
+                                  const gd_backend_matrix_view *y, const gd_backend_fused_linear_args *args);
+
+/* Decode-step form of qkv_split_rope + kv_cache_append_positions in one launch: qkv [B, 3*H*D]
+ * (one new token per sequence), q [B,H,D] receives the rotated queries, the rotated keys and the
+ * copied values are written to row cache_pos[b] of k_cache / v_cache [B,Tmax,H,D].  Same
+ * arithmetic and the same bytes as the two separate operators; a sequence whose cache position is
+ * negative or >= Tmax keeps its caches untouched.  NeoX pairing, head_dim % 16 == 0, F16 only
+ * (GD_ERR_UNSUPPORTED otherwise: use the separate operators). */
+gd_status gd_backend_qkv_rope_append(gd_backend *backend, const gd_backend_tensor_view *qkv,
+                                     const gd_backend_tensor_view *pos_ids,
+                                     const gd_backend_tensor_view *cache_pos, const gd_backend_tensor_view *q,
+                                     const gd_backend_tensor_view *k_cache, const gd_backend_tensor_view *v_cache,
+                                     uint32_t n_heads, uint32_t head_dim, const gd_backend_rope_args *args);
+
 /* out[i,:] = src[rows[i],:]; replaces the reference's per-sequence slice +
  * concat when the last prompt rows are selected
  * (examples/gpt_lm/gpt_lm_shared.c:1117-1169).  Row index out of range -> row
@@ -361,7 +396,8 @@ gd_status gd_backend_device_info(const gd_backend *backend, char *name, size_t n
 
 /* Kernel tunables, normally left at 0 = automatic.  name "sdpa_chunk": keys per workgroup of
  * the split-KV decode kernel (also read once from the environment variable
- * GD_HIP_SDPA_CHUNK).  Unknown name -> GD_ERR_INVALID_ARGUMENT. */
+ * GD_HIP_SDPA_CHUNK); "sdpa_waves" (4 or 8 wavefronts per workgroup) and "sdpa_unroll" (4 or 8
+ * key-row loads in flight per lane) of the same kernel.  Unknown name -> GD_ERR_INVALID_ARGUMENT. */
 gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t value);
 
 /* Raw device address of a buffer (base of the allocation). */

@@ -70,11 +70,20 @@ gd_status gd_gpt_decoder_step(gd_gpt_decoder *dec, const int32_t *ids, int32_t *
  *   sync   waits for everything enqueued;
  *   end    closes the scope and downloads the tokens of all steps run so far: out_ids
  *          [steps, batch] and (may be NULL) out_gaps; steps_done (may be NULL) = rows written.
- * At most max_steps steps can run in a session.  With hold_positions != 0 the cache positions do
- * not advance: every step appends at the same row and attends over the same number of keys (used
- * to time one fixed-shape step repeatedly). */
+ * At most max_steps steps can run in a session.  flags:
+ *   GD_GPT_RESIDENT_HOLD_POSITIONS  the cache positions do not advance: every step appends at the
+ *                                   same row and attends over the same number of keys (used to time
+ *                                   one fixed-shape step repeatedly);
+ *   GD_GPT_RESIDENT_UNFUSED         issue the step through the public operators exactly like
+ *                                   gd_gpt_decoder_step (about 40 launches for 3 layers).  Without
+ *                                   it the step uses the fused backend entry points
+ *                                   (gd_backend_fused_linear, gd_backend_qkv_rope_append: 6 launches
+ *                                   per layer), which keep every rounding point of the separate
+ *                                   operators. */
+#define GD_GPT_RESIDENT_HOLD_POSITIONS 1
+#define GD_GPT_RESIDENT_UNFUSED 2
 gd_status gd_gpt_decoder_resident_begin(gd_gpt_decoder *dec, const int32_t *first_ids, int32_t max_steps,
-                                        int32_t hold_positions);
+                                        int32_t flags);
 gd_status gd_gpt_decoder_resident_run(gd_gpt_decoder *dec, int32_t n_steps);
 gd_status gd_gpt_decoder_resident_sync(gd_gpt_decoder *dec);
 gd_status gd_gpt_decoder_resident_end(gd_gpt_decoder *dec, int32_t *out_ids, float *out_gaps, int32_t *steps_done);

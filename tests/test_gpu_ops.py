@@ -538,3 +538,77 @@ def test_gather_rows_and_position_increment(backend, arena, oracle, gda):
     p = arena.from_numpy(np.arange(64, dtype=np.int32))
     backend.add_scalar_i32(p, p, 1)
     assert np.array_equal(p.read(), np.arange(1, 65))
+
+
+# ---- fused operators (same rounding points as the separate ones) -----------------------------------------------
+
+@pytest.mark.parametrize("M,K,N", [(64, 512, 1536), (16, 2048, 96), (5, 136, 50), (70, 512, 64)])
+def test_fused_linear_rms_prologue_and_residual(backend, arena, oracle, M, K, N):
+    x = oracle.normal_f16((M, K), 2000 + K, 1.3)
+    nw = (1.0 + 0.1 * oracle.normal_f16((K,), 2001).astype(np.float32)).astype(np.float16)
+    w = oracle.normal_f16((N, K), 2002 + N, 0.05)
+    bias = oracle.normal_f16((N,), 2003, 0.5)
+    res = oracle.normal_f16((M, N), 2004, 1.0)
+    y = arena.alloc((M, N), 1)
+    tx, tw, tb, tr, tn = (arena.from_numpy(a) for a in (x, w, bias, res, nw))
+    backend.fused_linear(tx, tw, tb, None, tn, y, True, 2, 2, 1e-5)
+    want = oracle.linear_nt(oracle.rms_norm(x, nw, 1e-5), w, bias)
+    _close(y.read(), want)
+    backend.fused_linear(tx, tw, tb, tr, None, y, True, 2, 0)
+    want = oracle.add(res, oracle.linear_nt(x, w, bias))
+    _close(y.read(), want)
+    backend.fused_linear(tx, tw, None, tr, tn, y, True, 0, 2, 1e-5)
+    _close(y.read(), oracle.add(res, oracle.linear_nt(oracle.rms_norm(x, nw, 1e-5), w)))
+
+
+@pytest.mark.parametrize("M,K,N,nk", [(64, 1536, 512, True), (64, 1536, 512, False), (16, 352, 2048, True), (3, 24, 33, False)])
+def test_fused_linear_swiglu_prologue_both_layouts(backend, arena, oracle, M, K, N, nk):
+    x12 = oracle.normal_f16((M, 2 * K), 2100 + K, 1.0)
+    w_kn = oracle.normal_f16((K, N), 2101 + N, 0.05)
+    bias = oracle.normal_f16((N,), 2102, 0.5)
+    res = oracle.normal_f16((M, N), 2103, 1.0)
+    w = np.ascontiguousarray(w_kn.T) if nk else w_kn
+    y = arena.alloc((M, N), 1)
+    backend.fused_linear(arena.from_numpy(x12), arena.from_numpy(w), arena.from_numpy(bias), arena.from_numpy(res), None, y,
+                         nk, 1, 1)
+    _close(y.read(), oracle.add(res, oracle.swiglu_split_linear(x12, w_kn, bias)))
+
+
+def test_fused_linear_rejects_bad_arguments(backend, arena, gda):
+    x, w, y = arena.alloc((4, 16), gda.F16), arena.alloc((8, 16), gda.F16), arena.alloc((4, 8), gda.F16)
+    b = arena.alloc((8,), gda.F16)
+    a = gda.FusedLinearArgs(1, 0, 2, 1e-5)  # rms prologue without a norm weight
+    assert backend.call("gd_backend_fused_linear", x.matrix(), w.matrix(), None, None, None, y.matrix(), C.byref(a)) == gda.INVALID_ARGUMENT
+    a = gda.FusedLinearArgs(1, 1, 0, 0.0)  # bias mode without a bias
+    assert backend.call("gd_backend_fused_linear", x.matrix(), w.matrix(), None, None, None, y.matrix(), C.byref(a)) == gda.INVALID_ARGUMENT
+    a = gda.FusedLinearArgs(1, 0, 0, 0.0)  # bias without a bias mode
+    assert backend.call("gd_backend_fused_linear", x.matrix(), w.matrix(), b.vector(), None, None, y.matrix(), C.byref(a)) == gda.INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("B,H,D", [(64, 8, 64), (16, 16, 128), (3, 2, 32)])
+def test_qkv_rope_append_equals_separate_ops(backend, arena, oracle, B, H, D):
+    Tmax = 40
+    qkv = oracle.normal_f16((B, 3 * H * D), 2200 + D)
+    pos = oracle.uniform_i32(B, 2201, 0, Tmax - 1)
+    cpos = pos.copy()
+    cpos[0] = -1
+    if B > 2:
+        cpos[2] = Tmax
+    k0, v0 = oracle.normal_f16((B, Tmax, H, D), 2202), oracle.normal_f16((B, Tmax, H, D), 2203)
+    q = arena.alloc((B, H, D), 1)
+    kc, vc = arena.from_numpy(k0), arena.from_numpy(v0)
+    backend.qkv_rope_append(arena.from_numpy(qkv), arena.from_numpy(pos), arena.from_numpy(cpos), q, kc, vc, H, D)
+    # same arithmetic as the separate device operators: bit-identical results
+    q2, k2, v2 = (arena.alloc((B, H, D), 1) for _ in range(3))
+    backend.qkv_split_rope_forward(arena.from_numpy(qkv), arena.from_numpy(pos), q2, k2, v2, H, D)
+    kc2, vc2 = arena.from_numpy(k0), arena.from_numpy(v0)
+    backend.kv_cache_append_positions(kc2, vc2, arena.from_numpy(cpos), k2.reshape(B, 1, H, D), v2.reshape(B, 1, H, D))
+    assert np.array_equal(_bits(q.read()), _bits(q2.read()))
+    assert np.array_equal(_bits(kc.read()), _bits(kc2.read())) and np.array_equal(_bits(vc.read()), _bits(vc2.read()))
+    # and against the oracle
+    wq, wk, wv = oracle.qkv_split_rope(qkv, pos, H, D)
+    ok, ov = k0.copy(), v0.copy()
+    oracle.kv_cache_append(ok, ov, wk.reshape(B, 1, H, D), wv.reshape(B, 1, H, D), cpos)
+    _close(q.read(), wq)
+    _close(kc.read(), ok)
+    assert np.array_equal(_bits(vc.read()), _bits(ov))
