@@ -26,6 +26,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+# HBM bytes per sdpa_decode launch at this shape from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
+# profiles/sdpa_decode_config2_pmc.md (fetch scaled by the factor a 64 MiB device copy shows in the same run)
+SDPA_TRAFFIC_BYTES = 67316700
 
 
 def _package():
@@ -79,8 +82,40 @@ def sdpa_roofline(dec, D, pkg, iters=200):
     sec = ms / 1e3 / iters
     gbs = algo_bytes / sec / 1e9
     return {"bound": "hbm", "kernel": "gd_sdpa_decode_split_kernel<64,1,8,8>", "achieved": round(gbs, 1),
-            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": SDPA_TRAFFIC_BYTES,
             "algorithmic_bytes_per_launch": algo_bytes, "us_per_launch": round(sec * 1e6, 3), "launches": iters}
+
+
+def kernel_only(pkg, launches=20, copy_mib=64):
+    """For counter collection (rocprofv3 --pmc): the sdpa_decode launch of the benchmark shape on
+    pattern-filled caches, followed by device copies of a known size whose counters calibrate the
+    units of FETCH_SIZE / WRITE_SIZE."""
+    import ctypes as C
+    be = pkg.Backend()
+    B, H, Dh, T = 64, 8, 64, 512
+    buf = be.buffer(256 << 20)
+    k, v = buf.alloc((B, T, H, Dh), pkg.F16), buf.alloc((B, T, H, Dh), pkg.F16)
+    be.fill(k, 0x3400)
+    be.fill(v, 0x3800)
+    rng = np.random.default_rng(1)
+    q = buf.from_numpy(rng.standard_normal((B, 1, H, Dh)).astype(np.float16))
+    out = buf.alloc((B, 1, H, Dh), pkg.F16)
+    pos = buf.from_numpy(np.full(B, T - 1, np.int32))
+    args = pkg.SdpaDecodeArgs(0.125, 0, 0, 0)
+    src, dst = buf.alloc((copy_mib << 20,), pkg.U8), buf.alloc((copy_mib << 20,), pkg.U8)
+    be.fill(src, 0x11)
+    be.scope_begin()
+    for _ in range(launches):
+        assert be.call("gd_backend_sdpa_decode_positions", q.view(), k.view(), v.view(), pos.view(), out.view(),
+                       C.byref(args)) == 0
+    for _ in range(5):
+        assert pkg.lib().gd_backend_copy(be.handle, dst.buffer.handle, dst.offset, src.buffer.handle, src.offset,
+                                         src.nbytes) == 0
+    be.fence_wait(be.record_fence())
+    print(json.dumps({"kernel_only": "gd_sdpa_decode_split_kernel", "launches": launches,
+                      "algorithmic_bytes_per_launch": B * T * H * Dh * 4 + 2 * B * H * Dh * 2 + 4 * B,
+                      "calibration_copy_bytes": copy_mib << 20, "calibration_copies": 5}))
+    be.close()
 
 
 def cpu_baseline(oracle, cfg_tuple, budget_s=12.0, max_steps=64):
@@ -111,6 +146,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--kernel-only", action="store_true",
+                    help="only launch sdpa_decode at the benchmark shape plus calibration copies (for --pmc runs)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU: the decode path holds every sequence, its K/V cache and a full "
@@ -118,6 +155,9 @@ def main():
                  "replicas); run with --gpus 1")
     pkg, oracle = _package()
     pkg.lib()
+    if a.kernel_only:
+        kernel_only(pkg)
+        return
     from gradients_c_amd import decoder as D
 
     B, T = 64, 512
