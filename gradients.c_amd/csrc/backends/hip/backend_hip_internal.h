@@ -34,6 +34,7 @@ struct gd_backend {
     int sdpa_chunk;      /* keys per workgroup in the split-KV decode kernel (0 = automatic) */
     int sdpa_waves;      /* 4 or 8 wavefronts per workgroup (0 = default 8) */
     int sdpa_unroll;     /* 4 or 8 key-row loads in flight per lane (0 = default 8) */
+    int sdpa_nontemporal; /* 1: streaming hint on the K/V loads */
 };
 
 struct gd_backend_buffer {

@@ -17,6 +17,7 @@ typedef struct gd_hip_sdpa_decode_params {
     uint32_t dtype;  /* GD_BACKEND_DTYPE_F16 or _F32 (generic kernel) */
     uint32_t waves;  /* wavefronts per workgroup of the split-KV kernel: 4 or 8 */
     uint32_t unroll; /* key-row loads in flight per lane: 4 or 8 */
+    uint32_t nontemporal; /* 1: K/V loads carry the streaming hint */
 } gd_hip_sdpa_decode_params;
 
 #endif

@@ -76,7 +76,7 @@ __device__ __forceinline__ float gd_row_group_sum(float x)
     return x;
 }
 
-template <int D, int G, int WAVES, int UNROLL>
+template <int D, int G, int WAVES, int UNROLL, bool NT>
 __global__ void __launch_bounds__(WAVES * 64)
 gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__restrict__ kc,
                             const gd_half *__restrict__ vc, const int32_t *__restrict__ pos_ptr,
@@ -135,17 +135,22 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
     const gd_half *kbase = kc + ((size_t)b * p.tmax * p.hkv + hkv) * D + sub * 8;
     const gd_half *vbase = vc + ((size_t)b * p.tmax * p.hkv + hkv) * D + sub * 8;
 
-    for (int j0 = r0 + wave * KPW + slot; j0 < r1; j0 += KPB * UNROLL) {
-        gd_half8 kv[UNROLL], vv[UNROLL];
-        bool ok[UNROLL];
+    /* Row loads of trip t+1 are issued before the arithmetic of trip t (two register buffers), so
+     * the memory pipe stays busy while the wavefront computes. */
+    auto load_trip = [&](gd_half8 (&kv)[UNROLL], gd_half8 (&vv)[UNROLL], bool (&ok)[UNROLL], int j0) {
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int j = j0 + u * KPB;
             ok[u] = j < r1;
             const int jj = ok[u] ? j : (r1 - 1);
-            kv[u] = *reinterpret_cast<const gd_half8 *>(kbase + (size_t)jj * row_stride);
-            vv[u] = *reinterpret_cast<const gd_half8 *>(vbase + (size_t)jj * row_stride);
+            const gd_half8 *kp = reinterpret_cast<const gd_half8 *>(kbase + (size_t)jj * row_stride);
+            const gd_half8 *vp = reinterpret_cast<const gd_half8 *>(vbase + (size_t)jj * row_stride);
+            /* every cache row is read exactly once per launch: optionally mark the loads streaming */
+            kv[u] = NT ? __builtin_nontemporal_load(kp) : *kp;
+            vv[u] = NT ? __builtin_nontemporal_load(vp) : *vp;
         }
+    };
+    auto compute_trip = [&](const gd_half8 (&kv)[UNROLL], const gd_half8 (&vv)[UNROLL], const bool (&ok)[UNROLL]) {
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             /* scores of the UNROLL rows, then one rescale of the running state for all of them */
@@ -175,6 +180,26 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
             }
             l[g] = lsum;
             m[g] = mn;
+        }
+    };
+
+    constexpr int STEP = KPB * UNROLL;
+    int ja = r0 + wave * KPW + slot;
+    if (ja < r1) {
+        gd_half8 kA[UNROLL], vA[UNROLL], kB[UNROLL], vB[UNROLL];
+        bool okA[UNROLL], okB[UNROLL];
+        load_trip(kA, vA, okA, ja);
+        while (true) {
+            const int jb = ja + STEP;
+            const bool has_b = jb < r1;
+            if (has_b) load_trip(kB, vB, okB, jb);
+            compute_trip(kA, vA, okA);
+            if (!has_b) break;
+            ja = jb + STEP;
+            const bool has_a = ja < r1;
+            if (has_a) load_trip(kA, vA, okA, ja);
+            compute_trip(kB, vB, okB);
+            if (!has_a) break;
         }
     }
 
@@ -336,8 +361,14 @@ static int launch_split(hipStream_t stream, const void *q, const void *k, const 
 {
     dim3 grid(p.nsplit, p.hkv, p.batch);
 #define GD_GO(W, U)                                                                                   \
-    gd_sdpa_decode_split_kernel<D, G, W, U><<<grid, W * 64, 0, stream>>>(                              \
-        (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, pos, (gd_half *)out, ws, p)
+    do {                                                                                              \
+        if (p.nontemporal)                                                                            \
+            gd_sdpa_decode_split_kernel<D, G, W, U, true><<<grid, W * 64, 0, stream>>>(                \
+                (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, pos, (gd_half *)out, ws, p); \
+        else                                                                                          \
+            gd_sdpa_decode_split_kernel<D, G, W, U, false><<<grid, W * 64, 0, stream>>>(               \
+                (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, pos, (gd_half *)out, ws, p); \
+    } while (0)
     if constexpr (G == 1) {
         if (p.waves == 8u && p.unroll == 8u) GD_GO(8, 8);
         else if (p.waves == 8u) GD_GO(8, 4);
