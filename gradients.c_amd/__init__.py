@@ -78,6 +78,11 @@ class FusedLinearArgs(C.Structure):
     _fields_ = [("w_is_nk", C.c_uint32), ("bias_mode", C.c_uint32), ("prologue", C.c_uint32), ("eps", C.c_float)]
 
 
+class ConcatArgs(C.Structure):
+    _fields_ = [("count", C.c_uint64), ("inner", C.c_uint64), ("slice_axis", C.c_uint64), ("full_axis", C.c_uint64),
+                ("axis_offset", C.c_uint64)]
+
+
 class KvAppendArgs(C.Structure):
     _fields_ = [("cache_pos", C.c_int32)]
 
@@ -128,6 +133,8 @@ _SIGNATURES = {
     "gd_backend_linear_nt": [_vp, _MV, _MV, _VV, _MV],
     "gd_backend_fused_linear": [_vp, _MV, _MV, _VV, _MV, _VV, _MV, C.POINTER(FusedLinearArgs)],
     "gd_backend_qkv_rope_append": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, C.c_uint32, C.c_uint32, C.POINTER(RopeArgs)],
+    "gd_backend_rand_uniform": [_vp, _vp, C.c_size_t, C.c_size_t, C.c_uint32, C.c_uint64, C.c_float, C.c_float],
+    "gd_backend_concat_to_full": [_vp, _TV, _TV, C.POINTER(ConcatArgs)],
     "gd_backend_gather_rows": [_vp, _TV, _TV, _TV],
     "gd_backend_add_scalar_i32": [_vp, _TV, _TV, C.c_int32],
     "gd_backend_decode_advance": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, _TV, C.c_int32],
@@ -367,6 +374,10 @@ class Backend:
         _check(lib().gd_backend_fill(self.handle, tensor.buffer.handle, tensor.offset, tensor.count,
                                      tensor.itemsize, pattern), "gd_backend_fill")
 
+    def rand_uniform(self, tensor, seed, low, high):
+        _check(lib().gd_backend_rand_uniform(self.handle, tensor.buffer.handle, tensor.offset, tensor.count,
+                                             tensor.dtype, seed, low, high), "gd_backend_rand_uniform")
+
     def call(self, name, *args):
         """Raw status of a gd_backend_* call (for error-path tests)."""
         return getattr(lib(), name)(self.handle, *args)
@@ -462,6 +473,12 @@ class Backend:
 
     def gather_rows(self, src, rows, out):
         _check(self.call("gd_backend_gather_rows", src.view(), rows.view(), out.view()), "gd_backend_gather_rows")
+
+    def concat_to_full(self, src, dst, axis, axis_offset):
+        """Place the contiguous slice `src` at `axis_offset` along `axis` of the contiguous `dst`."""
+        inner = int(np.prod(src.shape[axis + 1:], dtype=np.int64))
+        a = ConcatArgs(src.count, inner, src.shape[axis], dst.shape[axis], axis_offset)
+        _check(self.call("gd_backend_concat_to_full", src.view(), dst.view(), C.byref(a)), "gd_backend_concat_to_full")
 
     def add_scalar_i32(self, src, dst, delta):
         _check(self.call("gd_backend_add_scalar_i32", src.view(), dst.view(), delta), "gd_backend_add_scalar_i32")

@@ -15,6 +15,8 @@
 #include "backend_hip_internal.h"
 
 int gd_hip_launch_fill(hipStream_t stream, void *dst, size_t count, size_t elem_size, uint32_t pattern);
+int gd_hip_launch_rand_uniform(hipStream_t stream, void *dst, uint64_t count, uint32_t dtype, uint64_t seed,
+                               float low, float high);
 
 static gd_status status_of(hipError_t e)
 {
@@ -287,6 +289,21 @@ gd_status gd_backend_fill(gd_backend *backend, gd_backend_buffer *buffer, size_t
     if (count == 0u) return GD_OK;
     return gd_hip_finish_op(backend, gd_hip_launch_fill(backend->stream, (char *)buffer->dptr + offset,
                                                         count, elem_size, pattern));
+}
+
+gd_status gd_backend_rand_uniform(gd_backend *backend, gd_backend_buffer *buffer, size_t offset, size_t count,
+                                  uint32_t dtype, uint64_t seed, float low, float high)
+{
+    size_t elem_size;
+    if (dtype == GD_BACKEND_DTYPE_F16 || dtype == GD_BACKEND_DTYPE_BF16) elem_size = 2u;
+    else if (dtype == GD_BACKEND_DTYPE_F32) elem_size = 4u;
+    else return GD_ERR_UNSUPPORTED;
+    if (backend == NULL || buffer == NULL || count > UINT32_MAX || !(low <= high) || (offset % elem_size) != 0u ||
+        !range_ok(buffer, offset, count * elem_size))
+        return GD_ERR_INVALID_ARGUMENT;
+    if (count == 0u) return GD_OK;
+    return gd_hip_finish_op(backend, gd_hip_launch_rand_uniform(backend->stream, (char *)buffer->dptr + offset, count,
+                                                                dtype, seed, low, high));
 }
 
 gd_status gd_backend_copy(gd_backend *backend, gd_backend_buffer *dst, size_t dst_offset,

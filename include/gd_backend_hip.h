@@ -32,6 +32,7 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+#pragma GCC visibility push(default) /* the library is built with hidden visibility: only these are exported */
 
 /* ---- part 1: status, dtype codes, handles, views ------------------------- */
 
@@ -137,6 +138,11 @@ gd_status gd_backend_download(gd_backend *backend, gd_backend_buffer *buffer, si
 gd_status gd_backend_fill(gd_backend *backend, gd_backend_buffer *buffer, size_t offset,
                           size_t count, size_t elem_size, uint32_t pattern);
 
+/* backend.h:178-185.  Element i = low + (high - low) * u_i with u_i the 24 bits [40,64) of
+ * splitmix64(seed + i) scaled by 2^-24; F16 / BF16 / F32 destinations, anything else UNSUPPORTED. */
+gd_status gd_backend_rand_uniform(gd_backend *backend, gd_backend_buffer *buffer, size_t offset, size_t count,
+                                  uint32_t dtype, uint64_t seed, float low, float high);
+
 /* backend.h:788-791.  record_fence closes the scope opened by scope_begin. */
 gd_status gd_backend_record_fence(gd_backend *backend, gd_backend_fence *out_fence);
 void gd_backend_fence_destroy(gd_backend_fence *fence);
@@ -208,6 +214,19 @@ gd_status gd_backend_qkv_split_rope_forward(gd_backend *backend, const gd_backen
 /* backend.h:520-522.  out[r,c] = x12[r,c] * silu(x12[r,H+c]). */
 gd_status gd_backend_swiglu_split_forward(gd_backend *backend, const gd_backend_tensor_view *x12,
                                           const gd_backend_tensor_view *out);
+
+/* backend.h:579-591.  Copies a contiguous slice into its place inside the contiguous concatenated
+ * tensor: dst[outer, axis_offset + a, inner] = src[outer, a, inner] with a < slice_axis.  The
+ * reference's generator concatenates the last prompt rows with it. */
+typedef struct gd_backend_concat_args {
+    uint64_t count;
+    uint64_t inner;
+    uint64_t slice_axis;
+    uint64_t full_axis;
+    uint64_t axis_offset;
+} gd_backend_concat_args;
+gd_status gd_backend_concat_to_full(gd_backend *backend, const gd_backend_tensor_view *src,
+                                    const gd_backend_tensor_view *dst, const gd_backend_concat_args *args);
 
 /* backend.h:671-698.  Packed causal attention over cu_seqlens; stats may be
  * NULL (inference).  Head dim up to 128 (the reference stops at 64). */
@@ -403,6 +422,7 @@ gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t 
 /* Raw device address of a buffer (base of the allocation). */
 void *gd_backend_buffer_device_ptr(gd_backend_buffer *buffer);
 
+#pragma GCC visibility pop
 #ifdef __cplusplus
 }
 #endif

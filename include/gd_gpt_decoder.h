@@ -23,6 +23,7 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+#pragma GCC visibility push(default) /* the library is built with hidden visibility: only these are exported */
 
 typedef struct gd_gpt_config {
     int32_t vocab, d_model, n_layers, n_heads, head_dim, mlp_hidden;
@@ -93,6 +94,7 @@ gd_status gd_gpt_decoder_resident_end(gd_gpt_decoder *dec, int32_t *out_ids, flo
 gd_status gd_gpt_decoder_run_resident(gd_gpt_decoder *dec, const int32_t *first_ids, int32_t n_steps,
                                       int32_t *out_ids, float *out_gaps, float *step_ms);
 
+#pragma GCC visibility pop
 #ifdef __cplusplus
 }
 #endif

@@ -30,6 +30,7 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+#pragma GCC visibility push(default) /* the library is built with hidden visibility: only these are exported */
 
 const char *gd_status_string(gd_status status); /* status.h:21 */
 
@@ -273,6 +274,7 @@ gd_status gd_argmax_rows(gd_context *ctx, const gd_tensor *logits, gd_tensor *id
  * (examples/gpt_lm/gpt_lm_shared.c:1117-1169). */
 gd_status gd_gather_rows(gd_context *ctx, const gd_tensor *x, const gd_tensor *rows, gd_tensor *out);
 
+#pragma GCC visibility pop
 #ifdef __cplusplus
 }
 #endif

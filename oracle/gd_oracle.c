@@ -172,6 +172,20 @@ GDO_API void gdo_fill_normal_f16(uint16_t *values, size_t count, uint64_t seed, 
     }
 }
 
+/* reference src/backends/metal/primitives/random/metal_random.metal:8-30 (gd_backend_rand_uniform):
+ * element i is low + (high - low) * u with u = bits [40,64) of splitmix64(seed + i) times 2^-24,
+ * evaluated in F32 as one fused multiply-add (the shader source writes low + span * u and its compiler
+ * contracts by default; the HIP kernel pins the same single rounding), stored as F32. */
+GDO_API void gdo_rand_uniform_f32(float *values, size_t count, uint64_t seed, float low, float high)
+{
+    const float span = high - low;
+    for (size_t i = 0; i < count; ++i) {
+        const uint32_t mant = (uint32_t)((gdo_splitmix64(seed + (uint64_t)i) >> 40) & 0xffffffu);
+        const float u = (float)mant * (1.0f / 16777216.0f);
+        values[i] = fmaf(span, u, low);
+    }
+}
+
 /* Uniform integers in [lo, hi] from the same splitmix64 stream (modulo draw). */
 GDO_API void gdo_fill_uniform_i32(int32_t *values, size_t count, uint64_t seed, int32_t lo, int32_t hi)
 {

@@ -54,6 +54,7 @@ def _declare(l):
         "gdo_fill_normal": [_vp, C.c_size_t, _u64, _f32],
         "gdo_fill_normal_f16": [_vp, C.c_size_t, _u64, _f32],
         "gdo_fill_uniform_i32": [_vp, C.c_size_t, _u64, _i32, _i32],
+        "gdo_rand_uniform_f32": [_vp, C.c_size_t, _u64, C.c_float, C.c_float],
         "gdo_fill_tokens": [_vp, C.c_uint32, _f32],
         "gdo_fill_values": [_vp, C.c_size_t, _f32, _f32],
         "gdo_kv_cache_append": [_vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _i64, _i64],
@@ -130,6 +131,12 @@ def normal_f16(shape, seed, stddev=1.0):
     out = np.empty(n, np.uint16)
     lib().gdo_fill_normal_f16(_p(out), n, seed & 0xFFFFFFFFFFFFFFFF, stddev)
     return out.view(np.float16).reshape(shape)
+
+
+def rand_uniform_f32(count, seed, low, high):
+    out = np.empty(count, np.float32)
+    lib().gdo_rand_uniform_f32(_p(out), count, seed & 0xFFFFFFFFFFFFFFFF, low, high)
+    return out
 
 
 def uniform_i32(count, seed, lo, hi):

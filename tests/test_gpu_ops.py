@@ -540,6 +540,43 @@ def test_gather_rows_and_position_increment(backend, arena, oracle, gda):
     assert np.array_equal(p.read(), np.arange(1, 65))
 
 
+def test_rand_uniform_matches_the_counter_based_stream(backend, arena, oracle, gda):
+    n = 100003
+    want = oracle.rand_uniform_f32(n, 1234, -1.0, 1.0)
+    f32 = arena.alloc((n,), gda.F32)
+    backend.rand_uniform(f32, 1234, -1.0, 1.0)
+    assert np.array_equal(_bits(f32.read()), _bits(want))
+    f16 = arena.alloc((n,), gda.F16)
+    backend.rand_uniform(f16, 1234, -1.0, 1.0)
+    assert np.array_equal(_bits(f16.read()), _bits(want.astype(np.float16)))
+    odd = arena.alloc((1000,), gda.F32)  # a span that is not a power of two: the multiply-add rounds once
+    backend.rand_uniform(odd, 99, 0.25, 7.5)
+    assert np.array_equal(_bits(odd.read()), _bits(oracle.rand_uniform_f32(1000, 99, 0.25, 7.5)))
+    i32 = arena.alloc((8,), gda.I32)
+    st = gda.lib().gd_backend_rand_uniform(backend.handle, i32.buffer.handle, i32.offset, i32.count, i32.dtype, 1, 0.0, 1.0)
+    assert st == gda.UNSUPPORTED
+    st = gda.lib().gd_backend_rand_uniform(backend.handle, f32.buffer.handle, f32.offset, f32.count, f32.dtype, 1, 2.0, 1.0)
+    assert st == gda.INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.int32, np.uint8])
+def test_concat_to_full_places_slices_bit_exact(backend, arena, gda, dtype):
+    """np.concatenate is the reference: two slices along the middle axis, then along axis 0."""
+    rng = np.random.default_rng(5)
+    a = rng.integers(0, 200, (3, 2, 7)).astype(dtype)
+    b = rng.integers(0, 200, (3, 5, 7)).astype(dtype)
+    full = arena.from_numpy(np.zeros((3, 7, 7), dtype))
+    backend.concat_to_full(arena.from_numpy(a), full, 1, 0)
+    backend.concat_to_full(arena.from_numpy(b), full, 1, 2)
+    assert np.array_equal(full.read(), np.concatenate([a, b], axis=1))
+    rows = arena.from_numpy(np.zeros((6, 2, 7), dtype))
+    backend.concat_to_full(arena.from_numpy(a), rows, 0, 3)
+    got = rows.read()
+    assert np.array_equal(got[3:], a) and not got[:3].any()
+    bad = gda.ConcatArgs(a.size, 7, 2, 7, 6)  # slice would run past the end of the axis
+    assert backend.call("gd_backend_concat_to_full", arena.from_numpy(a).view(), full.view(), C.byref(bad)) == gda.INVALID_ARGUMENT
+
+
 # ---- fused operators (same rounding points as the separate ones) -----------------------------------------------
 
 @pytest.mark.parametrize("M,K,N", [(64, 512, 1536), (16, 2048, 96), (5, 136, 50), (70, 512, 64)])

@@ -84,6 +84,21 @@ def test_fill_normal_statistics_and_stream(oracle):
     assert np.array_equal(h, oracle.fill_normal(9, 5, 1.0).astype(np.float16))
 
 
+def test_rand_uniform_is_the_24_bit_draw_of_the_published_stream(oracle):
+    # u_i = top 24 bits of splitmix64(seed + i): with seed 1234567 element 0 uses Vigna's published
+    # first output 6457827717110365317, whose top 24 bits are 6457827717110365317 >> 40.
+    v = oracle.rand_uniform_f32(4, 1234567, 0.0, 1.0)
+    assert v[0] == np.float32((6457827717110365317 >> 40) / 16777216.0)
+    # affine map: exact for a power-of-two span, and the endpoints bound every draw
+    w = oracle.rand_uniform_f32(4, 1234567, -1.0, 1.0)
+    assert np.array_equal(w, (-1.0 + 2.0 * v.astype(np.float64)).astype(np.float32))
+    big = oracle.rand_uniform_f32(200000, 7, -1.0, 1.0).astype(np.float64)
+    assert big.min() >= -1.0 and big.max() < 1.0
+    assert abs(big.mean()) < 6e-3 and abs(big.var() - 1.0 / 3.0) < 3e-3
+    # element i of seed s is element 0 of seed s + i (counter-based, no carried state)
+    assert oracle.rand_uniform_f32(6, 11, 0.0, 1.0)[5] == oracle.rand_uniform_f32(1, 16, 0.0, 1.0)[0]
+
+
 def test_uniform_i32_range(oracle):
     v = oracle.uniform_i32(50000, 3, 1, 4096)
     assert v.min() >= 1 and v.max() <= 4096 and v.min() < 20 and v.max() > 4080
