@@ -8,7 +8,7 @@
 
 int gd_hip_launch_linear(hipStream_t stream, const void *x, const void *w, const void *bias, const void *residual,
                          const void *norm_w, void *y, const gd_hip_linear_params *params, int vector_ok,
-                         int min_workgroups);
+                         int kn_vector_ok, int store_vector_ok, int min_workgroups);
 
 static gd_status project_full(gd_backend *backend, const gd_backend_matrix_view *x, const gd_backend_matrix_view *w,
                               const gd_backend_vector_view *bias, const gd_backend_matrix_view *residual,
@@ -17,7 +17,7 @@ static gd_status project_full(gd_backend *backend, const gd_backend_matrix_view 
 {
     gd_hip_linear_params p;
     uint32_t K;
-    int vec;
+    int vec, kn_vec, store_vec;
     if (backend == NULL || !gd_hip_matrix_ok(x) || !gd_hip_matrix_ok(w) || !gd_hip_matrix_ok(y) ||
         (bias != NULL && !gd_hip_vector_ok(bias)) || (residual != NULL && !gd_hip_matrix_ok(residual)) ||
         (norm_w != NULL && !gd_hip_vector_ok(norm_w)))
@@ -57,10 +57,13 @@ static gd_status project_full(gd_backend *backend, const gd_backend_matrix_view 
     /* 16-byte fragment loads: x rows always, w rows when K-contiguous, the norm weight */
     vec = (K % 8u) == 0u && ((x->offset | x->row_bytes) & 15u) == 0u &&
           (!w_is_nk || ((w->offset | w->row_bytes) & 15u) == 0u) && (norm_w == NULL || (norm_w->offset & 15u) == 0u);
+    kn_vec = !w_is_nk && (p.N % 8u) == 0u && ((w->offset | w->row_bytes) & 15u) == 0u;
+    store_vec = ((y->offset | y->row_bytes) & 15u) == 0u &&
+                (residual == NULL || ((residual->offset | residual->row_bytes) & 15u) == 0u);
     return gd_hip_finish_op(backend, gd_hip_launch_linear(
         backend->stream, gd_hip_matrix_ptr(x), gd_hip_matrix_ptr(w), bias != NULL ? gd_hip_vector_ptr(bias) : NULL,
         residual != NULL ? gd_hip_matrix_ptr(residual) : NULL, norm_w != NULL ? gd_hip_vector_ptr(norm_w) : NULL,
-        gd_hip_matrix_ptr(y), &p, vec, 2 * backend->compute_units));
+        gd_hip_matrix_ptr(y), &p, vec, kn_vec, store_vec, 2 * backend->compute_units));
 }
 
 static gd_status project(gd_backend *backend, const gd_backend_matrix_view *x, const gd_backend_matrix_view *w,

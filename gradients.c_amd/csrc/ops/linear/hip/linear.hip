@@ -214,10 +214,17 @@ static void launch_stream(hipStream_t stream, const gd_half *x, const gd_half *w
 #undef GD_GO
 }
 
-/* vector_ok: K % 8 == 0 and every pointer / pitch allows 16-byte fragment loads */
+extern "C" int gd_hip_launch_linear_tile(hipStream_t stream, const void *x, const void *w, const void *bias,
+                                         const void *residual, const void *norm_w, void *y,
+                                         const gd_hip_linear_params *params, int big_tiles, int vector_store);
+
+/* vector_ok: K % 8 == 0 and every pointer / pitch allows 16-byte fragment loads (for w only when it is [N,K]);
+ * kn_vector_ok: w stored [K,N] with N % 8 == 0 and 16-byte aligned rows; store_vector_ok: y (and the residual)
+ * rows allow 16-byte accesses.  min_workgroups: about two per compute unit. */
 extern "C" int gd_hip_launch_linear(hipStream_t stream, const void *x, const void *w, const void *bias,
                                     const void *residual, const void *norm_w, void *y,
-                                    const gd_hip_linear_params *params, int vector_ok, int min_workgroups)
+                                    const gd_hip_linear_params *params, int vector_ok, int kn_vector_ok,
+                                    int store_vector_ok, int min_workgroups)
 {
     const gd_hip_linear_params &p = *params;
     const gd_half *xp = (const gd_half *)x, *wp = (const gd_half *)w, *bp = (const gd_half *)bias;
@@ -227,6 +234,12 @@ extern "C" int gd_hip_launch_linear(hipStream_t stream, const void *x, const voi
     if (!vector_ok || p.K == 0) {
         const uint64_t total = (uint64_t)p.M * p.N;
         gd_linear_scalar_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(xp, wp, bp, rp, np, yp, p);
+    } else if (p.M >= 128u && (p.w_is_nk || kn_vector_ok)) {
+        /* matrix-core bound: LDS-tiled kernel; the 256 x 256 tile once it still gives every compute unit
+         * a workgroup, the 128 x 128 tile below that */
+        const uint64_t big = (uint64_t)((p.M + 255u) / 256u) * ((p.N + 255u) / 256u);
+        const uint32_t units = min_workgroups > 0 ? (uint32_t)min_workgroups / 2u : 256u;
+        return gd_hip_launch_linear_tile(stream, x, w, bias, residual, norm_w, y, params, big >= units, store_vector_ok);
     } else {
         /* rows per workgroup: 16, 32 or 64.  More rows reuse each weight fragment for more MFMAs but
          * leave fewer workgroups; narrow outputs take 16 rows so that the grid still covers the chip

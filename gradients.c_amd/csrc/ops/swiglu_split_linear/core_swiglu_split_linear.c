@@ -1,11 +1,15 @@
 /*
  * gd_swiglu_split_linear (forward): y = linear(swiglu_split(x12), w [H, N], bias).  The reference
  * composes gd_swiglu_split and gd_linear and frees the activation span in inference
- * (src/ops/swiglu_split_linear/core_swiglu_split_linear.c:22-121,226-301); here the activation is
- * formed inside the projection kernel (gd_backend_swiglu_split_linear), keeping its F16 rounding,
- * so no intermediate tensor exists.
+ * (src/ops/swiglu_split_linear/core_swiglu_split_linear.c:22-121,226-301).  For the few rows of a decode
+ * step the activation is formed inside the projection kernel (gd_backend_swiglu_split_linear), keeping
+ * its F16 rounding, so no intermediate tensor exists.  For many rows (prefill) the reference's two-kernel
+ * form is faster: the activation goes to a scratch span that is released as soon as the projection is
+ * enqueued, and the projection then stages both operands straight into LDS.  Same arithmetic either way.
  */
 #include "../linear/linear_impl.h"
+
+#define GD_SWIGLU_UNFUSED_MIN_ROWS 128u
 
 gd_status gd_swiglu_split_linear(gd_context *ctx, const gd_tensor *x12, const gd_tensor *w, const gd_tensor *bias,
                                  gd_tensor *out)
@@ -26,8 +30,28 @@ gd_status gd_swiglu_split_linear(gd_context *ctx, const gd_tensor *x12, const gd
     if (!gd_op_rows_matrix_view(x12, &xm) || !gd_op_matrix_view(w, &wm) || !gd_op_rows_matrix_view(&o, &ym) ||
         (bias != NULL && !gd_op_vector_view(bias, &bv)))
         GD_FAIL(ctx, GD_ERR_INTERNAL, "swiglu_split_linear view construction failed");
-    GD_TRY(gd_op_backend_result(ctx, gd_backend_swiglu_split_linear(gd_context_backend(ctx), &xm, &wm, bias != NULL ? &bv : NULL, &ym),
-                                "backend swiglu_split_linear failed"));
+    if (ym.rows >= GD_SWIGLU_UNFUSED_MIN_ROWS) {
+        gd_tensor act;
+        gd_backend_tensor_view x12v, actv;
+        gd_backend_matrix_view am;
+        int64_t act_shape[2];
+        gd_status st;
+        act_shape[0] = (int64_t)ym.rows;
+        act_shape[1] = x12->shape[x12->rank - 1U] / 2;
+        GD_TRY(gd_tensor_alloc_like_shape(ctx, GD_DTYPE_F16, 2U, act_shape, &act)); /* top of the scratch stack */
+        if (!gd_op_tensor_view(x12, &x12v) || !gd_op_tensor_view(&act, &actv) || !gd_op_matrix_view(&act, &am))
+            GD_FAIL(ctx, GD_ERR_INTERNAL, "swiglu_split_linear view construction failed");
+        st = gd_backend_swiglu_split_forward(gd_context_backend(ctx), &x12v, &actv);
+        if (st == GD_OK) {
+            st = bias != NULL ? gd_backend_linear(gd_context_backend(ctx), &am, &wm, &bv, &ym)
+                              : gd_backend_matmul(gd_context_backend(ctx), &am, &wm, &ym);
+        }
+        gd_context_release_scratch(ctx, &act.storage); /* later kernels run after these two on the same stream */
+        GD_TRY(gd_op_backend_result(ctx, st, "backend swiglu_split_linear failed"));
+    } else {
+        GD_TRY(gd_op_backend_result(ctx, gd_backend_swiglu_split_linear(gd_context_backend(ctx), &xm, &wm, bias != NULL ? &bv : NULL, &ym),
+                                    "backend swiglu_split_linear failed"));
+    }
     *out = o;
     return GD_OK;
 }

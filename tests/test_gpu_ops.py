@@ -22,10 +22,14 @@ def _golden(name):
         return json.load(f)
 
 
-def _close(got, want, rtol=RTOL, atol=ATOL):
+def _close(got, want, rtol=RTOL, atol=ATOL, through=None):
+    """`through`: an intermediate the result was formed from by an F16 add; its magnitude, not the
+    (possibly cancelled) result's, sets the size of one rounding step."""
     got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
     err = np.abs(got - want)
     bound = atol + rtol * np.abs(want)
+    if through is not None:
+        bound = bound + rtol * np.abs(np.asarray(through, np.float64))
     assert np.all(err <= bound), f"max err {err.max():.3e}, worst excess {(err - bound).max():.3e}"
 
 
@@ -609,6 +613,67 @@ def test_fused_linear_swiglu_prologue_both_layouts(backend, arena, oracle, M, K,
     backend.fused_linear(arena.from_numpy(x12), arena.from_numpy(w), arena.from_numpy(bias), arena.from_numpy(res), None, y,
                          nk, 1, 1)
     _close(y.read(), oracle.add(res, oracle.swiglu_split_linear(x12, w_kn, bias)))
+
+
+# Many-row (prefill) projections: the LDS-tiled matrix-core kernel.  (300, 136, 200) runs the 128 x 128 tile
+# with ragged edges in all three dimensions, (2100, 200, 8200) the 256 x 256 tile (9 x 33 tiles), ragged too;
+# (640, 160, 384) and (2304, 160, 8192) are whole tiles with K a multiple of 32, which take the path that
+# stages operands straight into LDS (5 K tiles: pipeline fill, two steady-state tiles, drain).
+TILE_SHAPES = [(300, 136, 200), (128, 64, 128), (2100, 200, 8200), (640, 160, 384), (2304, 160, 8192), (256, 96, 256)]
+
+
+@pytest.mark.parametrize("M,K,N", TILE_SHAPES)
+@pytest.mark.parametrize("nk", [True, False])
+def test_many_row_projection_plain_and_bias_modes(backend, arena, oracle, M, K, N, nk):
+    x = oracle.normal_f16((M, K), 2300 + K, 1.0)
+    w_kn = oracle.normal_f16((K, N), 2301 + N, 0.05)
+    bias = oracle.normal_f16((N,), 2302, 0.5)
+    res = oracle.normal_f16((M, N), 2303, 1.0)
+    w = np.ascontiguousarray(w_kn.T) if nk else w_kn
+    w_nk = np.ascontiguousarray(w_kn.T)
+    tx, tw, tb, tr = (arena.from_numpy(a) for a in (x, w, bias, res))
+    y = arena.alloc((M, N), 1)
+    backend.fused_linear(tx, tw, None, None, None, y, nk, 0, 0)
+    _close(y.read(), oracle.linear_nt(x, w_nk))
+    backend.fused_linear(tx, tw, tb, None, None, y, nk, 1, 0)  # bias added in F32
+    _close(y.read(), oracle.linear(x, w_kn, bias))
+    backend.fused_linear(tx, tw, tb, tr, None, y, nk, 2, 0)  # bias added after the F16 rounding, then the residual
+    inter = oracle.linear_nt(x, w_nk, bias)
+    _close(y.read(), oracle.add(res, inter), through=inter)
+
+
+@pytest.mark.parametrize("M,K,N", TILE_SHAPES)
+@pytest.mark.parametrize("nk", [True, False])
+def test_many_row_projection_prologues(backend, arena, oracle, M, K, N, nk):
+    x12 = oracle.normal_f16((M, 2 * K), 2400 + K, 1.0)
+    x = np.ascontiguousarray(x12[:, :K])
+    nw = (1.0 + 0.1 * oracle.normal_f16((K,), 2401).astype(np.float32)).astype(np.float16)
+    w_kn = oracle.normal_f16((K, N), 2402 + N, 0.05)
+    bias = oracle.normal_f16((N,), 2403, 0.5)
+    w = np.ascontiguousarray(w_kn.T) if nk else w_kn
+    tw, tb = arena.from_numpy(w), arena.from_numpy(bias)
+    y = arena.alloc((M, N), 1)
+    backend.fused_linear(arena.from_numpy(x12), tw, tb, None, None, y, nk, 1, 1)
+    _close(y.read(), oracle.swiglu_split_linear(x12, w_kn, bias))
+    backend.fused_linear(arena.from_numpy(x), tw, tb, None, arena.from_numpy(nw), y, nk, 1, 2, 1e-5)
+    _close(y.read(), oracle.linear(oracle.rms_norm(x, nw, 1e-5), w_kn, bias))
+
+
+def test_many_row_projection_row_pitches_and_unaligned_output(backend, arena, oracle, gda):
+    """Row-strided x / y views (slices of wider matrices) and an output whose rows are not 16-byte aligned."""
+    M, K, N = 200, 96, 136
+    xw = oracle.normal_f16((M, K + 40), 2500)
+    w = oracle.normal_f16((N, K), 2501, 0.05)
+    tx = arena.from_numpy(xw)
+    ty = arena.from_numpy(np.full((M, N + 3), 7.0, np.float16))
+    xv = gda.MatrixView(tx.buffer.handle, tx.offset, M, K, (K + 40) * 2, gda.F16)
+    yv = gda.MatrixView(ty.buffer.handle, ty.offset + 2, M, N, (N + 3) * 2, gda.F16)
+    tw = arena.from_numpy(w)
+    assert backend.call("gd_backend_matmul_nt", C.byref(xv), tw.matrix(), C.byref(yv)) == 0
+    backend.flush()
+    got = ty.read()
+    _close(got[:, 1:N + 1], oracle.linear_nt(np.ascontiguousarray(xw[:, :K]), w))
+    assert np.all(got[:, 0] == 7.0) and np.all(got[:, N + 1:] == 7.0)
 
 
 def test_fused_linear_rejects_bad_arguments(backend, arena, gda):
