@@ -12,6 +12,10 @@ int gd_hip_launch_sdpa_varlen(hipStream_t stream, const void *q, const void *k, 
                               void *out, uint32_t n_rows, uint32_t batch, uint32_t hq, uint32_t hkv, uint32_t dh,
                               uint32_t causal, uint32_t window, uint32_t prefix_len, uint32_t max_seqlen, float scale,
                               int is_f16);
+int gd_hip_launch_sdpa_varlen_mfma(hipStream_t stream, const void *q, const void *k, const void *v, const int32_t *cu,
+                                   void *out, uint32_t n_rows, uint32_t batch, uint32_t hq, uint32_t hkv, uint32_t dh,
+                                   uint32_t causal, uint32_t window, uint32_t prefix_len, uint32_t max_seqlen,
+                                   float scale);
 
 gd_status gd_backend_sdpa_varlen(gd_backend *backend, const gd_backend_tensor_view *q,
                                  const gd_backend_tensor_view *k, const gd_backend_tensor_view *v,
@@ -39,6 +43,16 @@ gd_status gd_backend_sdpa_varlen(gd_backend *backend, const gd_backend_tensor_vi
     if (!(args->scale > 0.0f) || !isfinite(args->scale) || (args->prefix_len > 0u && args->causal == 0u) ||
         (args->max_seqlen > 0u && args->prefix_len > args->max_seqlen))
         return GD_ERR_INVALID_ARGUMENT;
+    /* matrix-core kernel: F16, head size 64 or 128, 16-byte aligned rows, 32-bit byte offsets into K and V */
+    if (q->dtype == GD_BACKEND_DTYPE_F16 && (q->shape[2] == 64 || q->shape[2] == 128) &&
+        ((q->offset | k->offset | v->offset | out->offset) & 15u) == 0u &&
+        (uint64_t)k->shape[0] * (uint64_t)k->shape[1] * (uint64_t)k->shape[2] * 2u < 0xffffffffull &&
+        args->sliding_window <= (uint32_t)INT32_MAX && args->prefix_len <= (uint32_t)INT32_MAX)
+        return gd_hip_finish_op(backend, gd_hip_launch_sdpa_varlen_mfma(
+            backend->stream, gd_hip_view_ptr(q), gd_hip_view_ptr(k), gd_hip_view_ptr(v),
+            (const int32_t *)gd_hip_view_ptr(cu_seqlens), gd_hip_view_ptr(out), (uint32_t)q->shape[0],
+            (uint32_t)(cu_seqlens->shape[0] - 1), (uint32_t)q->shape[1], (uint32_t)k->shape[1], (uint32_t)q->shape[2],
+            args->causal, args->sliding_window, args->prefix_len, args->max_seqlen, args->scale));
     return gd_hip_finish_op(backend, gd_hip_launch_sdpa_varlen(
         backend->stream, gd_hip_view_ptr(q), gd_hip_view_ptr(k), gd_hip_view_ptr(v),
         (const int32_t *)gd_hip_view_ptr(cu_seqlens), gd_hip_view_ptr(out), (uint32_t)q->shape[0],

@@ -335,6 +335,39 @@ def test_varlen_matches_oracle(backend, arena, oracle, H, Hkv, D, window, prefix
     _close(out.read(), oracle.sdpa_varlen(q, k, v, cu, 0.15, True, window, prefix, 256))
 
 
+@pytest.mark.parametrize("H,Hkv,D,causal,window,prefix", [
+    (4, 4, 64, True, 0, 0), (4, 2, 128, True, 0, 0), (2, 2, 128, True, 100, 0), (4, 1, 64, True, 70, 0),
+    (2, 1, 128, True, 40, 150), (2, 2, 64, True, 0, 200), (2, 2, 64, False, 0, 0), (2, 1, 128, False, 90, 0)])
+def test_varlen_many_blocks_matches_oracle(backend, arena, oracle, H, Hkv, D, causal, window, prefix):
+    """Segments longer than the 128-row query block and the 64-key block of the matrix-core kernel: block
+    edges, windows and prefixes that cross them, a segment that ends exactly on a block edge."""
+    lens = np.array([300, 128, 1, 577, 64, 65], np.int32)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    N = int(cu[-1])
+    q, k, v = oracle.normal_f16((N, H, D), 720), oracle.normal_f16((N, Hkv, D), 721), oracle.normal_f16((N, Hkv, D), 722)
+    out = arena.from_numpy(np.zeros(q.shape, np.float16))
+    scale = float(1.0 / np.sqrt(D))
+    backend.sdpa_varlen(arena.from_numpy(q), arena.from_numpy(k), arena.from_numpy(v), arena.from_numpy(cu), out,
+                        scale, causal, window, prefix, 0)
+    _close(out.read(), oracle.sdpa_varlen(q, k, v, cu, scale, causal, window, prefix, 0))
+
+
+def test_varlen_ignores_values_of_the_next_segment(backend, arena, oracle):
+    """Keys past a segment's end are never used, even if the neighbouring segment holds infinities."""
+    cu = np.array([0, 70, 140], np.int32)
+    q, k, v = (oracle.normal_f16((140, 2, 64), s) for s in (730, 731, 732))
+    v[70:] = np.inf
+    k[70:] = np.nan
+    out = arena.from_numpy(np.zeros(q.shape, np.float16))
+    backend.sdpa_varlen(arena.from_numpy(q), arena.from_numpy(k), arena.from_numpy(v), arena.from_numpy(cu), out,
+                        0.125, False, 0, 0, 0)
+    got = out.read()
+    assert np.all(np.isfinite(got[:70]))
+    kk, vv = k.copy(), v.copy()
+    kk[70:], vv[70:] = 0, 0
+    _close(got[:70], oracle.sdpa_varlen(q, kk, vv, cu, 0.125, False, 0, 0, 0)[:70])
+
+
 def test_varlen_max_seqlen_truncates(backend, arena, oracle):
     cu = np.array([0, 50, 60], np.int32)
     q, k, v = (oracle.normal_f16((60, 2, 64), s) for s in (710, 711, 712))
