@@ -140,12 +140,85 @@ def cpu_baseline(oracle, cfg_tuple, budget_s=12.0, max_steps=64):
                       f"F16 rows instead of a CPU prefill), {dt:.1f} s, oracle/gd_oracle.c with OpenMP"}
 
 
+C3_ARCH = (32768, 2048, 24, 16, 128, 5632)  # vocab, d_model, layers, heads, head_dim, mlp_hidden (configs[3], [4])
+
+
+def _event_ms(pkg, be, fn):
+    """Stream-event time of fn() (which only enqueues) on the backend stream."""
+    timer = pkg.Timer(be)
+    timer.start()
+    fn()
+    timer.stop()
+    ms = timer.elapsed_ms()
+    timer.close()
+    return ms
+
+
+def long_context_workload(a, pkg, oracle, D, which):
+    """configs[3]: B=16 sequences with 1024..4095 cached tokens (built by a real packed prefill), decode steps
+    with the positions held; configs[4]: 32 prompts of 64..2048 tokens, packed prefill, then 128 greedy steps with
+    growing caches (the reference generator's tok/s = prompts x generated / elapsed, clock started before prefill)."""
+    vocab, d_model, layers, heads, head_dim, hidden = C3_ARCH
+    B, T = (16, 4096) if which == 3 else (32, 4096)
+    rng = np.random.default_rng(1003 if which == 3 else 1004)
+    lens = rng.integers(1024, 4096, B) if which == 3 else rng.integers(64, 2049, B)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    n_tokens = int(cu[-1])
+    cfg = D.gpt_config(vocab, d_model, layers, heads, head_dim, hidden, T, B, window=0, tie_lm_head=False,
+                       seed=1000 + which)
+    t0 = time.perf_counter()
+    dec = D.GptDecoder(cfg, max_prefill_tokens=n_tokens)
+    init_s = time.perf_counter() - t0
+    prompt = oracle.uniform_i32(n_tokens, 1000 + which, 0, vocab - 1)
+    t0 = time.perf_counter()
+    _, first, _ = dec.prefill(prompt, cu, want_logits=False)
+    prefill_s = time.perf_counter() - t0
+    dense_flops = 2.0 * n_tokens * layers * (d_model * 3 * d_model + d_model * d_model + d_model * 2 * hidden + hidden * d_model)
+    attn_flops = 4.0 * head_dim * heads * layers * float(np.sum(lens.astype(np.float64) * (lens + 1) / 2))
+    steps = a.steps if which == 3 else 128
+    total = a.warmup + steps if which == 3 else steps
+    t0 = time.perf_counter()
+    dec.resident_begin(first, total + 1, hold_positions=(which == 3))
+    if which == 3:
+        dec.resident_run(a.warmup)
+        dec.resident_sync()
+        t0 = time.perf_counter()
+    dec.resident_run(steps)
+    dec.resident_sync()
+    elapsed = time.perf_counter() - t0
+    ids, _ = dec.resident_end()
+    assert ids.min() >= 0 and ids.max() < vocab
+    dec.close()
+    kv_bytes = float(np.sum(np.minimum(lens + 1, T))) * heads * head_dim * 2 * 2 * layers
+    weight_bytes = 2.0 * (layers * (d_model * 3 * d_model + d_model * d_model + d_model * 2 * hidden + hidden * d_model) + vocab * d_model)
+    line = {
+        "metric": f"decode tokens/sec at B={B}", "value": round(B * steps / elapsed, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": steps, "warmup": a.warmup if which == 3 else 0, "ms_per_step": round(elapsed * 1e3 / steps, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"configs[{which}]: scaled decoder (V32768 Dm2048 L24 H16 Dh128 Hm5632, untied head), "
+                               + ("B=16, caches of 1024..4095 tokens built by packed prefill, positions held"
+                                  if which == 3 else
+                                  "32 prompts of 64..2048 tokens, packed prefill then 128 greedy steps with growing caches"),
+                   "batch": B, "prompt_tokens": n_tokens, "prefill_seconds": round(prefill_s, 4),
+                   "prefill_tokens_per_s": round(n_tokens / prefill_s, 1),
+                   "prefill_tflops": round((dense_flops + attn_flops) / prefill_s / 1e12, 1),
+                   "weight_init_seconds": round(init_s, 1),
+                   "end_to_end_tokens_per_s": round(B * steps / (elapsed + prefill_s), 1),
+                   "step_hbm_floor_ms": round((kv_bytes + weight_bytes) / 8e12 * 1e3, 4)},
+        "roofline": None, "cpu_baseline": None,
+    }
+    print(json.dumps(line))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--workload", type=int, default=2, choices=(2, 3, 4),
+                    help="BASELINE.json configs index: 2 = the headline line (default); 3, 4 = the scaled decoder "
+                         "(reported without roofline / cpu_baseline objects)")
     ap.add_argument("--kernel-only", action="store_true",
                     help="only launch sdpa_decode at the benchmark shape plus calibration copies (for --pmc runs)")
     a = ap.parse_args()
@@ -159,6 +232,9 @@ def main():
         kernel_only(pkg)
         return
     from gradients_c_amd import decoder as D
+    if a.workload != 2:
+        long_context_workload(a, pkg, oracle, D, a.workload)
+        return
 
     B, T = 64, 512
     shape = (2048, 512, 3, 8, 64, 1536, T, B)

@@ -75,7 +75,8 @@ class SdpaDecodeArgs(C.Structure):
 
 
 class FusedLinearArgs(C.Structure):
-    _fields_ = [("w_is_nk", C.c_uint32), ("bias_mode", C.c_uint32), ("prologue", C.c_uint32), ("eps", C.c_float)]
+    _fields_ = [("w_is_nk", C.c_uint32), ("bias_mode", C.c_uint32), ("prologue", C.c_uint32), ("eps", C.c_float),
+                ("epilogue", C.c_uint32)]
 
 
 class ConcatArgs(C.Structure):
@@ -410,8 +411,8 @@ class Backend:
         _check(self.call("gd_backend_swiglu_split_linear", x12.matrix(), w.matrix(),
                          bias.vector() if bias else None, y.matrix()), "gd_backend_swiglu_split_linear")
 
-    def fused_linear(self, x, w, bias, residual, norm_weight, y, w_is_nk, bias_mode, prologue, eps=0.0):
-        a = FusedLinearArgs(int(w_is_nk), bias_mode, prologue, eps)
+    def fused_linear(self, x, w, bias, residual, norm_weight, y, w_is_nk, bias_mode, prologue, eps=0.0, epilogue=0):
+        a = FusedLinearArgs(int(w_is_nk), bias_mode, prologue, eps, epilogue)
         _check(self.call("gd_backend_fused_linear", x.matrix(), w.matrix(), bias.vector() if bias else None,
                          residual.matrix() if residual else None, norm_weight.vector() if norm_weight else None,
                          y.matrix(), C.byref(a)), "gd_backend_fused_linear")

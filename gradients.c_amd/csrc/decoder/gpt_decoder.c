@@ -55,27 +55,29 @@ static uint64_t mix64(uint64_t x)
 
 static uint64_t splitmix64(uint64_t x) { return mix64(x + UINT64_C(0x9e3779b97f4a7c15)); }
 
-static double uniform_open_closed(uint64_t *state)
+/* Draw number n (1-based) of the stream started at `seed`: the state advances by a constant, so any draw
+ * is addressable and the fill below can run in parallel and still equal the reference's sequential loop. */
+static double uniform_open_closed_at(uint64_t seed, uint64_t n)
 {
-    *state += UINT64_C(0x9e3779b97f4a7c15);
-    return ((double)(mix64(*state) >> 11) + 1.0) * (1.0 / 9007199254740992.0);
+    return ((double)(mix64(seed + n * UINT64_C(0x9e3779b97f4a7c15)) >> 11) + 1.0) * (1.0 / 9007199254740992.0);
 }
 
 static gd_status init_normal(gd_context *ctx, gd_tensor *t, uint64_t seed, float stddev)
 {
-    int64_t n;
+    int64_t n, pairs, pi;
     float *values;
-    uint64_t state = seed;
-    size_t i = 0U;
     gd_status st;
     TRY(gd_tensor_numel(t, &n));
     values = (float *)malloc((size_t)n * sizeof(float));
     if (values == NULL) return GD_ERR_OUT_OF_MEMORY;
-    while (i < (size_t)n) {
-        const double u1 = uniform_open_closed(&state), u2 = uniform_open_closed(&state);
+    pairs = (n + 1) / 2;
+#pragma omp parallel for schedule(static)
+    for (pi = 0; pi < pairs; ++pi) {
+        const double u1 = uniform_open_closed_at(seed, 2U * (uint64_t)pi + 1U);
+        const double u2 = uniform_open_closed_at(seed, 2U * (uint64_t)pi + 2U);
         const double radius = sqrt(-2.0 * log(u1)), angle = 6.283185307179586476925286766559 * u2;
-        values[i++] = (float)(radius * cos(angle) * (double)stddev);
-        if (i < (size_t)n) values[i++] = (float)(radius * sin(angle) * (double)stddev);
+        values[2 * pi] = (float)(radius * cos(angle) * (double)stddev);
+        if (2 * pi + 1 < n) values[2 * pi + 1] = (float)(radius * sin(angle) * (double)stddev);
     }
     st = gd_tensor_write_f32(ctx, t, values, (size_t)n);
     free(values);
@@ -458,7 +460,7 @@ static gd_status scratch_f16(gd_context *ctx, int64_t rows, int64_t cols, gd_ten
 /* y = [residual +] bias_mode(prologue(x) @ w) through gd_backend_fused_linear */
 static gd_status fused_project(gd_gpt_decoder *d, const gd_tensor *x, int64_t x_cols, const gpt_linear *lin,
                                const gd_tensor *w_override, const gd_tensor *bias, const gd_tensor *residual,
-                               const gd_tensor *norm_w, uint32_t prologue, int64_t n_out, gd_tensor *y)
+                               const gd_tensor *norm_w, uint32_t prologue, uint32_t epilogue, int64_t n_out, gd_tensor *y)
 {
     gd_backend_matrix_view xm, wm, rm, ym;
     gd_backend_vector_view bv, nv;
@@ -477,6 +479,7 @@ static gd_status fused_project(gd_gpt_decoder *d, const gd_tensor *x, int64_t x_
     a.bias_mode = lin->transposed ? 2U : 1U; /* [N,K]: matmul_nt + add (two roundings); [K,N]: fused F32 bias */
     a.prologue = prologue;
     a.eps = d->cfg.rms_eps;
+    a.epilogue = epilogue;
     st = gd_backend_fused_linear(gd_context_backend(d->ctx), &xm, &wm, &bv, residual != NULL ? &rm : NULL,
                                  norm_w != NULL ? &nv : NULL, &ym, &a);
     return st;
@@ -499,7 +502,7 @@ static gd_status enqueue_fused_step(gd_gpt_decoder *d, gd_tensor *logits)
     TRY(gd_embedding(ctx, &d->token_embedding, &d->ids_dev, &x));
     for (l = 0; l < c->n_layers; ++l) {
         const gpt_block *b = &d->blocks[l];
-        TRY(fused_project(d, &x, Dm, &b->qkv_proj, NULL, &b->qkv_proj.bias, NULL, &b->attn_norm_w, 2U, 3 * Dm, &qkv));
+        TRY(fused_project(d, &x, Dm, &b->qkv_proj, NULL, &b->qkv_proj.bias, NULL, &b->attn_norm_w, 2U, 0U, 3 * Dm, &qkv));
         TRY(scratch_f16(ctx, B, Dm, &q));
         tview(&qkv, &vqkv);
         tview(&d->pos_dev, &vpos);
@@ -517,9 +520,15 @@ static gd_status enqueue_fused_step(gd_gpt_decoder *d, gd_tensor *logits)
                                        (uint32_t)c->head_dim, &rope));
         TRY(gd_reshape(ctx, &q, gd_shape_make(4U, q_shape), &q4));
         TRY(gd_sdpa_decode_positions(ctx, &q4, &d->k_cache[l], &d->v_cache[l], &d->pos_dev, &sdpa, &attn));
-        TRY(fused_project(d, &attn, Dm, &b->attn_proj, NULL, &b->attn_proj.bias, &x, NULL, 0U, Dm, &x1));
-        TRY(fused_project(d, &x1, Dm, &b->up_gate, NULL, &b->up_gate.bias, NULL, &b->mlp_norm_w, 2U, 2 * Hm, &ug));
-        TRY(fused_project(d, &ug, 2 * Hm, &b->down_proj, NULL, &b->down_proj.bias, &x1, NULL, 1U, Dm, &x2));
+        TRY(fused_project(d, &attn, Dm, &b->attn_proj, NULL, &b->attn_proj.bias, &x, NULL, 0U, 0U, Dm, &x1));
+        if (B < 128) {
+            /* the gate is applied in the up/gate projection's epilogue: the [B,2Hm] intermediate is never stored */
+            TRY(fused_project(d, &x1, Dm, &b->up_gate, NULL, &b->up_gate.bias, NULL, &b->mlp_norm_w, 2U, 1U, Hm, &ug));
+            TRY(fused_project(d, &ug, Hm, &b->down_proj, NULL, &b->down_proj.bias, &x1, NULL, 0U, 0U, Dm, &x2));
+        } else {
+            TRY(fused_project(d, &x1, Dm, &b->up_gate, NULL, &b->up_gate.bias, NULL, &b->mlp_norm_w, 2U, 0U, 2 * Hm, &ug));
+            TRY(fused_project(d, &ug, 2 * Hm, &b->down_proj, NULL, &b->down_proj.bias, &x1, NULL, 1U, 0U, Dm, &x2));
+        }
         x = x2;
     }
     {
@@ -527,7 +536,7 @@ static gd_status enqueue_fused_step(gd_gpt_decoder *d, gd_tensor *logits)
         head_lin.weight = d->lm_head;
         head_lin.bias = d->lm_head_bias;
         head_lin.transposed = true;
-        TRY(fused_project(d, &x, Dm, &head_lin, NULL, &d->lm_head_bias, NULL, &d->final_norm_w, 2U, c->vocab, logits));
+        TRY(fused_project(d, &x, Dm, &head_lin, NULL, &d->lm_head_bias, NULL, &d->final_norm_w, 2U, 0U, c->vocab, logits));
     }
     return GD_OK;
 }

@@ -13,7 +13,7 @@ int gd_hip_launch_linear(hipStream_t stream, const void *x, const void *w, const
 static gd_status project_full(gd_backend *backend, const gd_backend_matrix_view *x, const gd_backend_matrix_view *w,
                               const gd_backend_vector_view *bias, const gd_backend_matrix_view *residual,
                               const gd_backend_vector_view *norm_w, float eps, const gd_backend_matrix_view *y,
-                              uint32_t w_is_nk, uint32_t epilogue, uint32_t prologue)
+                              uint32_t w_is_nk, uint32_t epilogue, uint32_t prologue, uint32_t gated)
 {
     gd_hip_linear_params p;
     uint32_t K;
@@ -33,9 +33,16 @@ static gd_status project_full(gd_backend *backend, const gd_backend_matrix_view 
     } else {
         K = x->cols;
     }
-    if (w_is_nk ? (w->cols != K || w->rows != y->cols) : (w->rows != K || w->cols != y->cols))
+    if (gated) {
+        /* swiglu epilogue: w [2H,K], bias [2H], y [M,H]; only the few-row kernel implements it */
+        if (!w_is_nk || residual != NULL) return GD_ERR_UNSUPPORTED;
+        if (w->cols != K || (w->rows & 1u) != 0u || w->rows / 2u != y->cols || (bias != NULL && bias->length != w->rows))
+            return GD_ERR_INVALID_ARGUMENT;
+        if (y->rows >= 128u) return GD_ERR_UNSUPPORTED;
+    } else if (w_is_nk ? (w->cols != K || w->rows != y->cols) : (w->rows != K || w->cols != y->cols)) {
         return GD_ERR_INVALID_ARGUMENT;
-    if (x->rows != y->rows || (bias != NULL && bias->length != y->cols) ||
+    }
+    if (x->rows != y->rows || (!gated && bias != NULL && bias->length != y->cols) ||
         (residual != NULL && (residual->rows != y->rows || residual->cols != y->cols)) ||
         ((prologue == GD_HIP_PRO_RMS_NORM) != (norm_w != NULL)) || (norm_w != NULL && (norm_w->length != K || !(eps > 0.0f))))
         return GD_ERR_INVALID_ARGUMENT;
@@ -54,6 +61,7 @@ static gd_status project_full(gd_backend *backend, const gd_backend_matrix_view 
     p.has_residual = residual != NULL ? 1u : 0u;
     p.ldr = residual != NULL ? (uint32_t)(residual->row_bytes / 2u) : 0u;
     p.eps = eps;
+    p.swiglu_cols = gated ? y->cols : 0u;
     /* 16-byte fragment loads: x rows always, w rows when K-contiguous, the norm weight */
     vec = (K % 8u) == 0u && ((x->offset | x->row_bytes) & 15u) == 0u &&
           (!w_is_nk || ((w->offset | w->row_bytes) & 15u) == 0u) && (norm_w == NULL || (norm_w->offset & 15u) == 0u);
@@ -71,7 +79,7 @@ static gd_status project(gd_backend *backend, const gd_backend_matrix_view *x, c
                          uint32_t epilogue, uint32_t swiglu)
 {
     return project_full(backend, x, w, bias, NULL, NULL, 0.0f, y, w_is_nk, epilogue,
-                        swiglu ? GD_HIP_PRO_SWIGLU : GD_HIP_PRO_NONE);
+                        swiglu ? GD_HIP_PRO_SWIGLU : GD_HIP_PRO_NONE, 0u);
 }
 
 gd_status gd_backend_matmul(gd_backend *backend, const gd_backend_matrix_view *x, const gd_backend_matrix_view *w,
@@ -112,8 +120,9 @@ gd_status gd_backend_fused_linear(gd_backend *backend, const gd_backend_matrix_v
                                   const gd_backend_matrix_view *residual, const gd_backend_vector_view *norm_weight,
                                   const gd_backend_matrix_view *y, const gd_backend_fused_linear_args *args)
 {
-    if (args == NULL || args->bias_mode > 2u || args->prologue > 2u || (args->bias_mode != 0u) != (bias != NULL))
+    if (args == NULL || args->bias_mode > 2u || args->prologue > 2u || args->epilogue > 1u ||
+        (args->bias_mode != 0u) != (bias != NULL))
         return GD_ERR_INVALID_ARGUMENT;
     return project_full(backend, x, w, bias, residual, norm_weight, args->eps, y, args->w_is_nk != 0u, args->bias_mode,
-                        args->prologue);
+                        args->prologue, args->epilogue);
 }

@@ -21,6 +21,8 @@ typedef struct gd_hip_linear_params {
     uint32_t has_residual;  /* 1: y = half(epilogue(acc)) + residual, residual [M,N] pitch ldr */
     uint32_t ldr;
     float eps;              /* rms_norm prologue */
+    uint32_t swiglu_cols;   /* 0, or H: w has 2H rows ([N,K] only); y [M,H] = half(u[:, :H] * silu(u[:, H:])) where u is
+                             * the projection after the bias epilogue, rounded to F16 like a stored intermediate */
 } gd_hip_linear_params;
 
 #endif

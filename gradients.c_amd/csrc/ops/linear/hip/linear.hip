@@ -29,6 +29,7 @@
  */
 #include "../../_shared/hip_device.h"
 #include "hip_linear_types.h"
+#include <type_traits>
 
 __device__ __forceinline__ float gd_lin_silu(float z)
 {
@@ -37,29 +38,157 @@ __device__ __forceinline__ float gd_lin_silu(float z)
     return z * (z >= 0.0f ? inv : e * inv);
 }
 
-template <int MT, int WAVES, bool W_NK, int PRO>
+template <int NT, int WAVES, bool W_NK, int PRO, bool RES>
 __global__ void __launch_bounds__(WAVES * 64)
 gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__ w,
                         const gd_half *__restrict__ bias, const gd_half *__restrict__ residual,
                         const gd_half *__restrict__ norm_w, gd_half *__restrict__ y, gd_hip_linear_params p,
                         uint32_t n_tiles)
 {
-    constexpr int U = 4; /* K steps whose loads are in flight together */
-    __shared__ float sm[WAVES][MT][64][4];
-    __shared__ float s_inv[MT * 16];
+    constexpr int U = NT >= 4 ? 2 : 4;  /* K steps per register set; two sets alternate */
+    constexpr int RES_STEPS = 8;        /* RES: the wavefront's whole K slice of the activation stays in registers */
+    constexpr uint32_t COLS = 16u * NT; /* output columns of a workgroup */
+    typedef short gd_short4 __attribute__((ext_vector_type(4)));
+    __shared__ float sm[WAVES][NT][64][4];
+    __shared__ float s_inv[16];
+    __shared__ float s_part[WAVES][16];
+    /* w stored [K,N]: a 32(k) x COLS(n) tile per wavefront, turned by the transposing LDS read */
+    __shared__ __align__(16) gd_half s_tr[W_NK ? 1 : WAVES][W_NK ? 8 : 32 * COLS];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int li = lane & 15, lg = lane >> 4;
     /* XCD-aware tile order: workgroup ids are dealt round-robin to the 8 XCDs, so give each XCD a
      * contiguous run of column tiles (neighbouring tiles share weight cache lines when w is [K,N]) */
     uint32_t tile = blockIdx.x;
     if ((n_tiles & 7u) == 0u) tile = (blockIdx.x & 7u) * (n_tiles >> 3) + (blockIdx.x >> 3);
-    const uint32_t n0 = tile * 16u;
-    const uint32_t m0 = blockIdx.y * (MT * 16u);
-    const uint32_t n = min(n0 + li, p.N - 1u); /* clamped: out-of-range columns are never stored */
+    /* gated (swiglu epilogue): the first NT/2 column tiles are value columns, the others the matching gate columns
+     * swiglu_cols further down the weight; the workgroup then owns COLS/2 output columns */
+    const bool gated = NT >= 2 && p.swiglu_cols != 0u;
+    const uint32_t n0 = tile * (gated ? COLS / 2u : COLS);
+    const uint32_t m0 = blockIdx.y * 16u;
+    const uint32_t mrow = min(m0 + (uint32_t)li, p.M - 1u);
 
-    if (PRO == GD_HIP_PRO_RMS_NORM) {
-        /* row norms of this tile: one wavefront per row, 8 halfs per lane and trip */
-        for (uint32_t r = wave; r < MT * 16u; r += WAVES) {
+    /* K range of this wavefront, in steps of 32 */
+    const uint32_t ksteps = (p.K + 31u) / 32u;
+    const uint32_t per_wave = (ksteps + WAVES - 1u) / WAVES;
+    const uint32_t s_begin = wave * per_wave, s_end = min(s_begin + per_wave, ksteps);
+
+    gd_half8 bf[2][U][NT];
+    gd_half8 af[2][RES ? 1 : U], zf[2][PRO == GD_HIP_PRO_SWIGLU ? U : 1], nf[2][(PRO == GD_HIP_PRO_RMS_NORM && !RES) ? U : 1];
+    gd_half8 ar[RES ? RES_STEPS : 1], nr[(RES && PRO == GD_HIP_PRO_RMS_NORM) ? RES_STEPS : 1];
+    const gd_half8 zero8 = (gd_half8)(gd_half)0.f;
+    const gd_half *xrow = x + (size_t)mrow * p.ldx;
+
+    /* requests the operands of steps s0 .. s0+U-1 into register set `set` */
+    auto load_set = [&](auto set_tag, uint32_t s0) __attribute__((always_inline)) {
+        constexpr int set = decltype(set_tag)::value;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const bool sok = (s0 + u) < s_end;
+            const uint32_t k = (s0 + u) * 32u + lg * 8u; /* K % 8 == 0: a fragment is all-valid or all-out */
+            const bool kok = sok && k < p.K;
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                bf[set][u][j] = zero8;
+                if (W_NK) {
+                    /* clamped: out-of-range columns are never stored */
+                    const uint32_t n = (gated && j >= NT / 2)
+                                           ? p.swiglu_cols + min(n0 + 16u * (uint32_t)(j - NT / 2) + (uint32_t)li, p.N - 1u)
+                                           : min(n0 + 16u * (uint32_t)j + (uint32_t)li, p.N - 1u);
+                    if (kok) bf[set][u][j] = *reinterpret_cast<const gd_half8 *>(w + (size_t)n * p.ldw + k);
+                } else {
+                    /* load j fetches k-rows j*32/NT .. of the 32 x COLS tile: 2*NT chunks of 8 columns per row */
+                    const uint32_t kr = (s0 + u) * 32u + (uint32_t)j * (32u / NT) + (uint32_t)lane / (2u * NT);
+                    const uint32_t nc = n0 + ((uint32_t)lane % (2u * NT)) * 8u;
+                    if (sok && kr < p.K && nc < p.N)
+                        bf[set][u][j] = *reinterpret_cast<const gd_half8 *>(w + (size_t)kr * p.ldw + nc);
+                }
+            }
+            if (!RES) {
+                af[set][u] = kok ? *reinterpret_cast<const gd_half8 *>(xrow + k) : zero8;
+                if (PRO == GD_HIP_PRO_SWIGLU) zf[set][u] = kok ? *reinterpret_cast<const gd_half8 *>(xrow + p.K + k) : zero8;
+                if (PRO == GD_HIP_PRO_RMS_NORM) nf[set][u] = kok ? *reinterpret_cast<const gd_half8 *>(norm_w + k) : zero8;
+            }
+        }
+    };
+
+    gd_float4 acc[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) acc[j] = (gd_float4){0.f, 0.f, 0.f, 0.f};
+    float minv = 1.f;
+
+    /* multiplies the steps of register set `set`; `base` = index of its first step within the wavefront's slice */
+    auto compute_set = [&](auto set_tag, auto base_tag) __attribute__((always_inline)) {
+        constexpr int set = decltype(set_tag)::value;
+        constexpr int base = decltype(base_tag)::value;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            gd_half8 a = RES ? ar[(base + u) < RES_STEPS ? (base + u) : 0] : af[set][u];
+            if (PRO == GD_HIP_PRO_SWIGLU) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) a[e] = (gd_half)((float)a[e] * gd_lin_silu((float)zf[set][u][e]));
+            }
+            if (PRO == GD_HIP_PRO_RMS_NORM) {
+                const gd_half8 nw = RES ? nr[(base + u) < RES_STEPS ? (base + u) : 0] : nf[set][u];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) a[e] = (gd_half)((float)a[e] * (float)nw[e] * minv);
+            }
+            if (!W_NK) {
+                gd_half *tr = &s_tr[wave][0];
+#pragma unroll
+                for (int j = 0; j < NT; ++j)
+                    *reinterpret_cast<gd_half8 *>(tr + ((uint32_t)j * (32u / NT) + (uint32_t)lane / (2u * NT)) * COLS +
+                                                  ((uint32_t)lane % (2u * NT)) * 8u) = bf[set][u][j];
+            }
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                gd_half8 b = bf[set][u][j];
+                if (!W_NK) {
+                    /* lane q + 4e of a 16-lane group addresses k-row 8*lg + e (+4), columns 4q .. 4q+3 of column tile j;
+                     * lane i then receives column i of four consecutive k-rows */
+                    const gd_half *src = &s_tr[wave][0] + (8 * lg + ((lane >> 2) & 3)) * COLS + 16 * j + (lane & 3) * 4;
+                    union { gd_short4 s[2]; gd_half8 h; } t2;
+                    t2.s[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) gd_short4 *)src);
+                    t2.s[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) gd_short4 *)(src + 4 * COLS));
+                    b = t2.h;
+                }
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[j], 0, 0, 0);
+            }
+        }
+    };
+    using gd_s0 = std::integral_constant<int, 0>;
+    using gd_s1 = std::integral_constant<int, 1>;
+
+    /* the first weights are requested before anything else so that the row norms below overlap their flight */
+    load_set(gd_s0{}, s_begin);
+
+    if (RES) {
+        /* the wavefront's whole activation slice (at most RES_STEPS steps): one batch of loads, and the row's sum of
+         * squares comes from these registers instead of a second pass over x */
+        float ss = 0.f;
+#pragma unroll
+        for (int r = 0; r < RES_STEPS; ++r) {
+            const uint32_t k = (s_begin + r) * 32u + lg * 8u;
+            const bool kok = (s_begin + r) < s_end && k < p.K;
+            ar[r] = kok ? *reinterpret_cast<const gd_half8 *>(xrow + k) : zero8;
+            if (PRO == GD_HIP_PRO_RMS_NORM) nr[r] = kok ? *reinterpret_cast<const gd_half8 *>(norm_w + k) : zero8;
+        }
+        if (PRO == GD_HIP_PRO_RMS_NORM) {
+#pragma unroll
+            for (int r = 0; r < RES_STEPS; ++r)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) ss = fmaf((float)ar[r][e], (float)ar[r][e], ss);
+            ss += __shfl_xor(ss, 16, 64);
+            ss += __shfl_xor(ss, 32, 64);
+            if (lg == 0) s_part[wave][li] = ss;
+            __syncthreads();
+            float tot = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < WAVES; ++wv) tot += s_part[wv][li];
+            minv = rsqrtf(tot / (float)p.K + p.eps);
+        }
+    } else if (PRO == GD_HIP_PRO_RMS_NORM) {
+        /* row norms by a separate pass over x: one wavefront per row, 8 halfs per lane and trip */
+        for (uint32_t r = wave; r < 16u; r += WAVES) {
             const uint32_t row = min(m0 + r, p.M - 1u);
             const gd_half *xr = x + (size_t)row * p.ldx;
             float ss = 0.f;
@@ -72,85 +201,74 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
             if (lane == 0) s_inv[r] = rsqrtf(ss / (float)p.K + p.eps);
         }
         __syncthreads();
+        minv = s_inv[li];
     }
 
-    /* K range of this wavefront, in steps of 32 */
-    const uint32_t ksteps = (p.K + 31u) / 32u;
-    const uint32_t per_wave = (ksteps + WAVES - 1u) / WAVES;
-    const uint32_t s_begin = wave * per_wave, s_end = min(s_begin + per_wave, ksteps);
-
-    gd_float4 acc[MT];
-#pragma unroll
-    for (int t = 0; t < MT; ++t) acc[t] = (gd_float4){0.f, 0.f, 0.f, 0.f};
-
-    uint32_t mrow[MT];
-    float minv[MT];
-#pragma unroll
-    for (int t = 0; t < MT; ++t) {
-        mrow[t] = min(m0 + t * 16u + li, p.M - 1u);
-        minv[t] = PRO == GD_HIP_PRO_RMS_NORM ? s_inv[t * 16 + li] : 1.f;
-    }
-
-    for (uint32_t s0 = s_begin; s0 < s_end; s0 += U) {
-        gd_half8 bf[U], af[U][MT], zf[U][MT], nf[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const uint32_t k = (s0 + u) * 32u + lg * 8u; /* K % 8 == 0: a fragment is all-valid or all-out */
-            const bool kok = (s0 + u) < s_end && k < p.K;
-            bf[u] = (gd_half8)(gd_half)0.f;
-            if (kok) {
-                if (W_NK) {
-                    bf[u] = *reinterpret_cast<const gd_half8 *>(w + (size_t)n * p.ldw + k);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) bf[u][e] = w[(size_t)(k + e) * p.ldw + n];
-                }
-                if (PRO == GD_HIP_PRO_RMS_NORM) nf[u] = *reinterpret_cast<const gd_half8 *>(norm_w + k);
-            }
-#pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                af[u][t] = (gd_half8)(gd_half)0.f;
-                if (kok) {
-                    const gd_half *xr = x + (size_t)mrow[t] * p.ldx + k;
-                    af[u][t] = *reinterpret_cast<const gd_half8 *>(xr);
-                    if (PRO == GD_HIP_PRO_SWIGLU) zf[u][t] = *reinterpret_cast<const gd_half8 *>(xr + p.K);
-                }
-            }
+    /* two register sets alternate: the next U steps are in flight while the current ones are multiplied */
+    if (RES) {
+        /* at most RES_STEPS steps: fully unrolled so that the resident fragments are indexed statically */
+        load_set(gd_s1{}, s_begin + U);
+        compute_set(gd_s0{}, std::integral_constant<int, 0>{});
+        if (2 * U < RES_STEPS) {
+            load_set(gd_s0{}, s_begin + 2u * U);
+            compute_set(gd_s1{}, std::integral_constant<int, U>{});
+            load_set(gd_s1{}, s_begin + 3u * U);
+            compute_set(gd_s0{}, std::integral_constant<int, 2 * U>{});
+            compute_set(gd_s1{}, std::integral_constant<int, 3 * U>{});
+        } else {
+            compute_set(gd_s1{}, std::integral_constant<int, U>{});
         }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const uint32_t k = (s0 + u) * 32u + lg * 8u;
-            const bool kok = (s0 + u) < s_end && k < p.K;
-#pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                gd_half8 a = af[u][t];
-                if (PRO == GD_HIP_PRO_SWIGLU && kok) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) a[e] = (gd_half)((float)a[e] * gd_lin_silu((float)zf[u][t][e]));
-                }
-                if (PRO == GD_HIP_PRO_RMS_NORM && kok) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) a[e] = (gd_half)((float)a[e] * (float)nf[u][e] * minv[t]);
-                }
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bf[u], acc[t], 0, 0, 0);
-            }
+    } else {
+        for (uint32_t s0 = s_begin; s0 < s_end; s0 += 2u * U) {
+            load_set(gd_s1{}, s0 + U);
+            compute_set(gd_s0{}, std::integral_constant<int, 0>{});
+            load_set(gd_s0{}, s0 + 2u * U);
+            compute_set(gd_s1{}, std::integral_constant<int, 0>{});
         }
     }
 
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
+    for (int j = 0; j < NT; ++j) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) sm[wave][t][lane][r] = acc[t][r];
+        for (int r = 0; r < 4; ++r) sm[wave][j][lane][r] = acc[j][r];
     }
     __syncthreads();
-    /* (result lane, register) pairs of the MT tiles are spread over the workgroup's threads */
-    for (int idx = threadIdx.x; idx < MT * 256; idx += WAVES * 64) {
-        const int t = idx >> 8, rl = idx & 63, rr = (idx >> 6) & 3;
-        const uint32_t col = n0 + (rl & 15);
-        const uint32_t row = m0 + t * 16u + 4u * (rl >> 4) + rr;
+    if (gated) {
+        for (int idx = threadIdx.x; idx < (NT / 2) * 256; idx += WAVES * 64) {
+            const int j = idx >> 8, rl = idx & 63, rr = (idx >> 6) & 3;
+            const uint32_t col = n0 + 16u * j + (rl & 15);
+            const uint32_t row = m0 + 4u * (rl >> 4) + rr;
+            float v1 = 0.f, v2 = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < WAVES; ++wv) {
+                v1 += sm[wv][j][rl][rr];
+                v2 += sm[wv][j + NT / 2][rl][rr];
+            }
+            if (row < p.M && col < p.N) {
+                gd_half h1, h2;
+                if (p.epilogue == GD_HIP_EPI_BIAS_F32) {
+                    h1 = (gd_half)(v1 + (float)bias[col]);
+                    h2 = (gd_half)(v2 + (float)bias[p.swiglu_cols + col]);
+                } else if (p.epilogue == GD_HIP_EPI_BIAS_F16) {
+                    h1 = (gd_half)v1 + bias[col];
+                    h2 = (gd_half)v2 + bias[p.swiglu_cols + col];
+                } else {
+                    h1 = (gd_half)v1;
+                    h2 = (gd_half)v2;
+                }
+                y[(size_t)row * p.ldy + col] = (gd_half)((float)h1 * gd_lin_silu((float)h2));
+            }
+        }
+        return;
+    }
+    /* (result lane, register) pairs of the NT tiles are spread over the workgroup's threads */
+    for (int idx = threadIdx.x; idx < NT * 256; idx += WAVES * 64) {
+        const int j = idx >> 8, rl = idx & 63, rr = (idx >> 6) & 3;
+        const uint32_t col = n0 + 16u * j + (rl & 15);
+        const uint32_t row = m0 + 4u * (rl >> 4) + rr;
         float v = 0.f;
 #pragma unroll
-        for (int wv = 0; wv < WAVES; ++wv) v += sm[wv][t][rl][rr];
+        for (int wv = 0; wv < WAVES; ++wv) v += sm[wv][j][rl][rr];
         if (row < p.M && col < p.N) {
             gd_half h;
             if (p.epilogue == GD_HIP_EPI_BIAS_F32) h = (gd_half)(v + (float)bias[col]);
@@ -194,22 +312,25 @@ gd_linear_scalar_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
     y[(size_t)m * p.ldy + n] = h;
 }
 
-template <int MT, int WAVES>
+template <int NT, int WAVES>
 static void launch_stream(hipStream_t stream, const gd_half *x, const gd_half *w, const gd_half *bias,
                           const gd_half *residual, const gd_half *norm_w, gd_half *y, const gd_hip_linear_params &p)
 {
-    const uint32_t n_tiles = (p.N + 15u) / 16u;
-    dim3 grid(n_tiles, (p.M + MT * 16u - 1u) / (MT * 16u));
+    const uint32_t cols = p.swiglu_cols != 0u ? 8u * NT : 16u * NT; /* output columns per workgroup */
+    const uint32_t n_tiles = (p.N + cols - 1u) / cols;
+    dim3 grid(n_tiles, (p.M + 15u) / 16u);
     const int threads = WAVES * 64;
-#define GD_GO(NK, PRO) gd_linear_stream_kernel<MT, WAVES, NK, PRO><<<grid, threads, 0, stream>>>(x, w, bias, residual, norm_w, y, p, n_tiles)
+    /* the whole K slice of a wavefront fits the resident registers (8 steps of 32) */
+    const bool res = ((p.K + 31u) / 32u + WAVES - 1u) / WAVES <= 8u;
+#define GD_GO(NK, PRO, RES) gd_linear_stream_kernel<NT, WAVES, NK, PRO, RES><<<grid, threads, 0, stream>>>(x, w, bias, residual, norm_w, y, p, n_tiles)
     if (p.w_is_nk) {
-        if (p.prologue == GD_HIP_PRO_SWIGLU) GD_GO(true, GD_HIP_PRO_SWIGLU);
-        else if (p.prologue == GD_HIP_PRO_RMS_NORM) GD_GO(true, GD_HIP_PRO_RMS_NORM);
-        else GD_GO(true, GD_HIP_PRO_NONE);
+        if (p.prologue == GD_HIP_PRO_SWIGLU) GD_GO(true, GD_HIP_PRO_SWIGLU, false);
+        else if (p.prologue == GD_HIP_PRO_RMS_NORM) { if (res) GD_GO(true, GD_HIP_PRO_RMS_NORM, true); else GD_GO(true, GD_HIP_PRO_RMS_NORM, false); }
+        else GD_GO(true, GD_HIP_PRO_NONE, false);
     } else {
-        if (p.prologue == GD_HIP_PRO_SWIGLU) GD_GO(false, GD_HIP_PRO_SWIGLU);
-        else if (p.prologue == GD_HIP_PRO_RMS_NORM) GD_GO(false, GD_HIP_PRO_RMS_NORM);
-        else GD_GO(false, GD_HIP_PRO_NONE);
+        if (p.prologue == GD_HIP_PRO_SWIGLU) GD_GO(false, GD_HIP_PRO_SWIGLU, false);
+        else if (p.prologue == GD_HIP_PRO_RMS_NORM) { if (res) GD_GO(false, GD_HIP_PRO_RMS_NORM, true); else GD_GO(false, GD_HIP_PRO_RMS_NORM, false); }
+        else GD_GO(false, GD_HIP_PRO_NONE, false);
     }
 #undef GD_GO
 }
@@ -231,23 +352,26 @@ extern "C" int gd_hip_launch_linear(hipStream_t stream, const void *x, const voi
     const gd_half *rp = (const gd_half *)residual, *np = (const gd_half *)norm_w;
     gd_half *yp = (gd_half *)y;
     if (p.M == 0 || p.N == 0) return (int)hipSuccess;
-    if (!vector_ok || p.K == 0) {
+    if (!vector_ok || p.K == 0 || (!p.w_is_nk && !kn_vector_ok)) {
         const uint64_t total = (uint64_t)p.M * p.N;
         gd_linear_scalar_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(xp, wp, bp, rp, np, yp, p);
-    } else if (p.M >= 128u && (p.w_is_nk || kn_vector_ok)) {
+    } else if (p.M >= 128u && (p.w_is_nk || kn_vector_ok) && p.swiglu_cols == 0u) {
         /* matrix-core bound: LDS-tiled kernel; the 256 x 256 tile once it still gives every compute unit
          * a workgroup, the 128 x 128 tile below that */
         const uint64_t big = (uint64_t)((p.M + 255u) / 256u) * ((p.N + 255u) / 256u);
         const uint32_t units = min_workgroups > 0 ? (uint32_t)min_workgroups / 2u : 256u;
         return gd_hip_launch_linear_tile(stream, x, w, bias, residual, norm_w, y, params, big >= units, store_vector_ok);
     } else {
-        /* rows per workgroup: 16, 32 or 64.  More rows reuse each weight fragment for more MFMAs but
-         * leave fewer workgroups; narrow outputs take 16 rows so that the grid still covers the chip
-         * (the re-read weights come from L2). */
-        const uint64_t n_tiles = (p.N + 15u) / 16u;
-        const uint32_t target = min_workgroups > 0 ? (uint32_t)min_workgroups : 512u;
-        if (p.M > 32u && n_tiles * ((p.M + 63u) / 64u) >= target) launch_stream<4, 8>(stream, xp, wp, bp, rp, np, yp, p);
-        else if (p.M > 16u && n_tiles * ((p.M + 31u) / 32u) >= target) launch_stream<2, 8>(stream, xp, wp, bp, rp, np, yp, p);
+        /* columns per workgroup: 64, 32 or 16 (rows: always 16, further rows in grid.y; their weight re-reads
+         * come from L2).  More columns reuse each activation fragment for more MFMAs and repeat the prologue
+         * in fewer workgroups, but leave fewer workgroups; the grid keeps at least one per compute unit. */
+        const uint64_t mt = (p.M + 15u) / 16u;
+        const uint32_t target = min_workgroups > 0 ? (uint32_t)min_workgroups / 2u : 256u;
+        if (p.swiglu_cols != 0u) { /* value and gate tiles side by side: 32 or 16 output columns per workgroup */
+            if (((p.N + 31u) / 32u) * mt >= target) launch_stream<4, 8>(stream, xp, wp, bp, rp, np, yp, p);
+            else launch_stream<2, 8>(stream, xp, wp, bp, rp, np, yp, p);
+        } else if (((p.N + 63u) / 64u) * mt >= target) launch_stream<4, 8>(stream, xp, wp, bp, rp, np, yp, p);
+        else if (((p.N + 31u) / 32u) * mt >= target) launch_stream<2, 8>(stream, xp, wp, bp, rp, np, yp, p);
         else launch_stream<1, 8>(stream, xp, wp, bp, rp, np, yp, p);
     }
     return (int)hipGetLastError();

@@ -200,7 +200,8 @@ class GptDecoder:
             # every operator output of every layer lives until the step ends (bump allocation):
             # 13 d_model-wide and one 2*hidden-wide F16 tensor per layer and row, 256-byte padded
             per_row = 2 * (13 * cfg.d_model + 2 * cfg.mlp_hidden) + 14 * 256
-            scratch_slot_bytes = (rows * per_row * cfg.n_layers * 2 + rows * cfg.d_model * 4
+            # + one transient activation of the many-row swiglu path, 10 % slack
+            scratch_slot_bytes = (int(rows * per_row * cfg.n_layers * 1.1) + rows * (cfg.d_model * 4 + cfg.mlp_hidden * 2)
                                   + cfg.batch * cfg.vocab * 4 + (64 << 20))
         self.ctx = Context(l.gd_gpt_params_bytes(C.byref(cfg)), l.gd_gpt_state_bytes(C.byref(cfg)),
                            scratch_slot_bytes, data_slot_bytes=max(1 << 20, 16 * rows + (1 << 16)))

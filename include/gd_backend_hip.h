@@ -338,12 +338,15 @@ gd_status gd_backend_linear_nt(gd_backend *backend, const gd_backend_matrix_view
  *   u = half(t)                                      bias_mode 0 (bias must be NULL)
  *     | half(t + bias)                               bias_mode 1 (gd_linear)
  *     | half(half(t) + bias)                         bias_mode 2 (gd_linear_transposed_weight)
- *   y = u, or half(residual + u) when residual != NULL (gd_add). */
+ *   y = u, or half(residual + u) when residual != NULL (gd_add)                      epilogue 0
+ *     | half(u[:, :H] * silu(u[:, H:])), w [2H,K], bias [2H], y [M,H]                epilogue 1 (the gd_swiglu_split
+ *       that follows the up/gate projection; w_is_nk only, no residual, fewer than 128 rows, else UNSUPPORTED) */
 typedef struct gd_backend_fused_linear_args {
     uint32_t w_is_nk;
     uint32_t bias_mode;
     uint32_t prologue;
     float eps;
+    uint32_t epilogue;
 } gd_backend_fused_linear_args;
 gd_status gd_backend_fused_linear(gd_backend *backend, const gd_backend_matrix_view *x,
                                   const gd_backend_matrix_view *w, const gd_backend_vector_view *bias,

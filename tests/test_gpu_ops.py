@@ -30,7 +30,10 @@ def _close(got, want, rtol=RTOL, atol=ATOL, through=None):
     bound = atol + rtol * np.abs(want)
     if through is not None:
         bound = bound + rtol * np.abs(np.asarray(through, np.float64))
-    assert np.all(err <= bound), f"max err {err.max():.3e}, worst excess {(err - bound).max():.3e}"
+    if not np.all(err <= bound):
+        at = np.unravel_index(np.argmax(err - bound), err.shape)
+        raise AssertionError(f"max err {err.max():.3e}, worst excess {(err - bound).max():.3e} at {at}: got {got[at]!r} "
+                             f"want {want[at]!r} bound {bound[at]:.3e}")
 
 
 def _bits(a):
@@ -707,6 +710,32 @@ def test_many_row_projection_row_pitches_and_unaligned_output(backend, arena, or
     got = ty.read()
     _close(got[:, 1:N + 1], oracle.linear_nt(np.ascontiguousarray(xw[:, :K]), w))
     assert np.all(got[:, 0] == 7.0) and np.all(got[:, N + 1:] == 7.0)
+
+
+@pytest.mark.parametrize("M,K,H", [(64, 512, 1536), (16, 2048, 5632), (5, 136, 24), (33, 64, 40)])
+def test_fused_linear_swiglu_epilogue(backend, arena, oracle, gda, M, K, H):
+    """rms_norm -> up/gate projection (+ F16 bias) -> swiglu_split in one launch equals the three separate operators."""
+    x = oracle.normal_f16((M, K), 2600 + K, 1.3)
+    nw = (1.0 + 0.1 * oracle.normal_f16((K,), 2601).astype(np.float32)).astype(np.float16)
+    w = oracle.normal_f16((2 * H, K), 2602 + H, 0.05)
+    bias = oracle.normal_f16((2 * H,), 2603, 0.5)
+    y = arena.alloc((M, H), 1)
+    tx, tw, tb, tn = (arena.from_numpy(a) for a in (x, w, bias, nw))
+    backend.fused_linear(tx, tw, tb, None, tn, y, True, 2, 2, 1e-5, epilogue=1)
+    def scale(u, b):
+        # one rounding step of the value (before its bias was added: the sum may cancel) times the gate, or of
+        # the gate times the value
+        u, b = u.astype(np.float64), b.astype(np.float64)
+        return (np.abs(u[:, :H]) + np.abs(b[:H])) * (1.0 + np.abs(u[:, H:]) + np.abs(b[H:]))
+
+    u = oracle.linear_nt(oracle.rms_norm(x, nw, 1e-5), w, bias)
+    _close(y.read(), oracle.swiglu_split(u), through=scale(u, bias))
+    backend.fused_linear(tx, tw, None, None, None, y, True, 0, 0, 0.0, epilogue=1)
+    u = oracle.linear_nt(x, w)
+    _close(y.read(), oracle.swiglu_split(u), through=scale(u, np.zeros_like(bias)))
+    a = gda.FusedLinearArgs(0, 0, 0, 0.0, 1)  # the gated epilogue needs the [N,K] weight layout
+    wk = arena.alloc((K, 2 * H), gda.F16)
+    assert backend.call("gd_backend_fused_linear", tx.matrix(), wk.matrix(), None, None, None, y.matrix(), C.byref(a)) == gda.UNSUPPORTED
 
 
 def test_fused_linear_rejects_bad_arguments(backend, arena, gda):
