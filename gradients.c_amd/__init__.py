@@ -139,6 +139,9 @@ _SIGNATURES = {
     "gd_backend_gather_rows": [_vp, _TV, _TV, _TV],
     "gd_backend_add_scalar_i32": [_vp, _TV, _TV, C.c_int32],
     "gd_backend_decode_advance": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, _TV, C.c_int32],
+    "gd_backend_fused_qkv_rope_append": [_vp, _MV, _MV, _VV, _VV, _TV, _TV, _TV, _TV, _TV, C.c_uint32, C.c_uint32,
+                                         C.POINTER(RopeArgs), C.POINTER(FusedLinearArgs)],
+    "gd_backend_argmax_advance": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, C.c_int32],
     "gd_backend_copy": [_vp, _vp, C.c_size_t, _vp, C.c_size_t, C.c_size_t],
     "gd_backend_timer_create": [_vp, C.POINTER(_vp)],
     "gd_backend_timer_start": [_vp],
@@ -429,6 +432,14 @@ class Backend:
         a = RopeArgs(theta, head_dim, 0)
         _check(self.call("gd_backend_qkv_rope_append", qkv.view(), pos.view(), cache_pos.view(), q.view(),
                          k_cache.view(), v_cache.view(), n_heads, head_dim, C.byref(a)), "gd_backend_qkv_rope_append")
+
+    def fused_qkv_rope_append(self, x, w, bias, norm_weight, pos, cache_pos, q, k_cache, v_cache, n_heads, head_dim,
+                              bias_mode, prologue, eps=0.0, theta=10000.0):
+        ra, fa = RopeArgs(theta, head_dim, 0), FusedLinearArgs(1, bias_mode, prologue, eps, 0)
+        _check(self.call("gd_backend_fused_qkv_rope_append", x.matrix(), w.matrix(), bias.vector() if bias else None,
+                         norm_weight.vector() if norm_weight else None, pos.view(), cache_pos.view(), q.view(),
+                         k_cache.view(), v_cache.view(), n_heads, head_dim, C.byref(ra), C.byref(fa)),
+               "gd_backend_fused_qkv_rope_append")
 
     def swiglu_split_forward(self, x12, out):
         _check(self.call("gd_backend_swiglu_split_forward", x12.view(), out.view()), "gd_backend_swiglu_split_forward")

@@ -36,7 +36,7 @@ struct gd_gpt_decoder {
     gd_tensor *k_cache, *v_cache;
     int32_t *pos; /* host copy of the live lengths */
     /* device-resident decode state (state arena) */
-    gd_tensor ids_dev, pos_dev, step_dev;
+    gd_tensor ids_dev, pos_dev, step_dev, step_rows_dev; /* step counters: one for the whole batch / one per row */
     /* open resident session */
     bool resident_open;
     int32_t resident_max_steps, resident_steps, resident_hold, resident_unfused;
@@ -121,7 +121,7 @@ size_t gd_gpt_params_bytes(const gd_gpt_config *c)
 size_t gd_gpt_state_bytes(const gd_gpt_config *c)
 {
     const size_t cache = pad256((size_t)c->batch * (size_t)c->max_seq * (size_t)c->n_heads * (size_t)c->head_dim * 2U);
-    return cache * 2U * (size_t)c->n_layers + 3U * pad256((size_t)c->batch * 4U) + 4096U;
+    return cache * 2U * (size_t)c->n_layers + 4U * pad256((size_t)c->batch * 4U) + 4096U;
 }
 
 gd_status gd_gpt_decoder_create(gd_context *ctx, const gd_gpt_config *cfg, gd_gpt_decoder **out)
@@ -184,6 +184,7 @@ gd_status gd_gpt_decoder_create(gd_context *ctx, const gd_gpt_config *cfg, gd_gp
     STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_I32, gd_shape_make(1U, bdim), 256U, &d->ids_dev));
     STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_I32, gd_shape_make(1U, bdim), 256U, &d->pos_dev));
     STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_I32, gd_shape_make(1U, one), 256U, &d->step_dev));
+    STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_I32, gd_shape_make(1U, bdim), 256U, &d->step_rows_dev));
 #undef STEP
     if (st != GD_OK) {
         gd_gpt_decoder_destroy(d);
@@ -502,9 +503,7 @@ static gd_status enqueue_fused_step(gd_gpt_decoder *d, gd_tensor *logits)
     TRY(gd_embedding(ctx, &d->token_embedding, &d->ids_dev, &x));
     for (l = 0; l < c->n_layers; ++l) {
         const gpt_block *b = &d->blocks[l];
-        TRY(fused_project(d, &x, Dm, &b->qkv_proj, NULL, &b->qkv_proj.bias, NULL, &b->attn_norm_w, 2U, 0U, 3 * Dm, &qkv));
         TRY(scratch_f16(ctx, B, Dm, &q));
-        tview(&qkv, &vqkv);
         tview(&d->pos_dev, &vpos);
         tview(&d->k_cache[l], &vk);
         tview(&d->v_cache[l], &vv);
@@ -516,8 +515,28 @@ static gd_status enqueue_fused_step(gd_gpt_decoder *d, gd_tensor *logits)
         vq.rank = 3U;
         vq.shape[0] = B; vq.shape[1] = c->n_heads; vq.shape[2] = c->head_dim;
         vq.strides[0] = Dm; vq.strides[1] = c->head_dim; vq.strides[2] = 1;
-        TRY(gd_backend_qkv_rope_append(be, &vqkv, &vpos, &vpos, &vq, &vk, &vv, (uint32_t)c->n_heads,
-                                       (uint32_t)c->head_dim, &rope));
+        if (B < 128 && (c->head_dim % 32) == 0) {
+            /* qkv projection with rotation and cache append in its epilogue: the [B,3Dm] intermediate is never stored */
+            gd_backend_matrix_view xm, wm;
+            gd_backend_vector_view bv, nv;
+            gd_backend_fused_linear_args fa;
+            mview(&x, B, Dm, &xm);
+            mview(&b->qkv_proj.weight, 3 * Dm, Dm, &wm);
+            vview(&b->qkv_proj.bias, &bv);
+            vview(&b->attn_norm_w, &nv);
+            fa.w_is_nk = 1U;
+            fa.bias_mode = 2U;
+            fa.prologue = 2U;
+            fa.eps = c->rms_eps;
+            fa.epilogue = 0U;
+            TRY(gd_backend_fused_qkv_rope_append(be, &xm, &wm, &bv, &nv, &vpos, &vpos, &vq, &vk, &vv, (uint32_t)c->n_heads,
+                                                 (uint32_t)c->head_dim, &rope, &fa));
+        } else {
+            TRY(fused_project(d, &x, Dm, &b->qkv_proj, NULL, &b->qkv_proj.bias, NULL, &b->attn_norm_w, 2U, 0U, 3 * Dm, &qkv));
+            tview(&qkv, &vqkv);
+            TRY(gd_backend_qkv_rope_append(be, &vqkv, &vpos, &vpos, &vq, &vk, &vv, (uint32_t)c->n_heads,
+                                           (uint32_t)c->head_dim, &rope));
+        }
         TRY(gd_reshape(ctx, &q, gd_shape_make(4U, q_shape), &q4));
         TRY(gd_sdpa_decode_positions(ctx, &q4, &d->k_cache[l], &d->v_cache[l], &d->pos_dev, &sdpa, &attn));
         TRY(fused_project(d, &attn, Dm, &b->attn_proj, NULL, &b->attn_proj.bias, &x, NULL, 0U, 0U, Dm, &x1));
@@ -555,8 +574,16 @@ static gd_status enqueue_resident_step(gd_gpt_decoder *d)
         }
         TRY(head(d, &x, &logits, &next, &gaps));
     } else {
+        /* greedy pick, token feedback, position and record keeping in one launch */
+        gd_backend_tensor_view vl;
         TRY(enqueue_fused_step(d, &logits));
-        TRY(gd_argmax_rows(ctx, &logits, &next, &gaps));
+        tview(&logits, &vl);
+        view1(&d->ids_dev, &vi);
+        view1(&d->pos_dev, &vp);
+        view1(&d->step_rows_dev, &vs);
+        view1(&d->resident_out_ids, &vo);
+        view1(&d->resident_out_gaps, &vog);
+        return gd_backend_argmax_advance(gd_context_backend(ctx), &vl, &vi, &vp, &vs, &vo, &vog, d->resident_hold ? 0 : 1);
     }
     view1(&next, &vn);
     view1(&gaps, &vg);
@@ -596,6 +623,7 @@ gd_status gd_gpt_decoder_resident_begin(gd_gpt_decoder *d, const int32_t *first_
     TRY(gd_tensor_write(ctx, &d->ids_dev, first_ids, (size_t)d->cfg.batch * sizeof(int32_t)));
     TRY(gd_tensor_write(ctx, &d->pos_dev, d->pos, (size_t)d->cfg.batch * sizeof(int32_t)));
     TRY(gd_tensor_write(ctx, &d->step_dev, &zero, sizeof(zero)));
+    TRY(gd_tensor_zero_(ctx, &d->step_rows_dev));
     TRY(gd_begin_step(ctx, GD_SCOPE_INFER, gd_batch_empty()));
     d->resident_open = true;
     d->resident_graph = NULL;

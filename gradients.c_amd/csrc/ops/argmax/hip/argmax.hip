@@ -39,10 +39,21 @@ __device__ __forceinline__ gd_top2 gd_top2_merge(const gd_top2 &a, const gd_top2
     return r;
 }
 
-template <typename T>
+/* what a device-resident decode loop does with the chosen token, per row (one workgroup per row, so every
+ * row keeps its own step counter) */
+struct gd_hip_advance {
+    int32_t *positions;     /* [rows] += pos_delta */
+    int32_t *step_counters; /* [rows]: s = counter, record into slot s when s < max_steps, counter = s + 1 */
+    int32_t *out_ids;       /* [max_steps * rows] */
+    float *out_gaps;        /* [max_steps * rows] or NULL */
+    uint32_t max_steps;
+    int32_t pos_delta;
+};
+
+template <typename T, bool ADVANCE>
 __global__ void __launch_bounds__(GD_ARGMAX_THREADS)
 gd_argmax_rows_kernel(const T *__restrict__ logits, int32_t *__restrict__ ids, float *__restrict__ gap,
-                      uint64_t cols)
+                      uint64_t cols, gd_hip_advance adv)
 {
     __shared__ gd_top2 sm[GD_ARGMAX_THREADS / 64];
     const T *row = logits + (uint64_t)blockIdx.x * cols;
@@ -64,19 +75,43 @@ gd_argmax_rows_kernel(const T *__restrict__ logits, int32_t *__restrict__ ids, f
     if (threadIdx.x == 0) {
         gd_top2 r = sm[0];
         for (int w = 1; w < GD_ARGMAX_THREADS / 64; ++w) r = gd_top2_merge(r, sm[w]);
-        ids[blockIdx.x] = r.idx < 0 ? 0 : r.idx;
-        if (gap != nullptr)
-            gap[blockIdx.x] = (r.idx >= 0 && r.second > GD_NEG_INF) ? r.best - r.second : __builtin_inff();
+        const int32_t token = r.idx < 0 ? 0 : r.idx;
+        const float g = (r.idx >= 0 && r.second > GD_NEG_INF) ? r.best - r.second : __builtin_inff();
+        ids[blockIdx.x] = token;
+        if (gap != nullptr) gap[blockIdx.x] = g;
+        if (ADVANCE) {
+            const int32_t s = adv.step_counters[blockIdx.x];
+            adv.positions[blockIdx.x] += adv.pos_delta;
+            if (s >= 0 && (uint32_t)s < adv.max_steps) {
+                adv.out_ids[(size_t)s * gridDim.x + blockIdx.x] = token;
+                if (adv.out_gaps != nullptr) adv.out_gaps[(size_t)s * gridDim.x + blockIdx.x] = g;
+            }
+            adv.step_counters[blockIdx.x] = s + 1;
+        }
     }
 }
 
 extern "C" int gd_hip_launch_argmax_rows(hipStream_t stream, const void *logits, int32_t *ids, float *gap,
                                          uint64_t rows, uint64_t cols, int is_f16)
 {
+    const gd_hip_advance none = {nullptr, nullptr, nullptr, nullptr, 0u, 0};
     if (rows == 0) return (int)hipSuccess;
     if (is_f16)
-        gd_argmax_rows_kernel<gd_half><<<(unsigned)rows, GD_ARGMAX_THREADS, 0, stream>>>((const gd_half *)logits, ids, gap, cols);
+        gd_argmax_rows_kernel<gd_half, false><<<(unsigned)rows, GD_ARGMAX_THREADS, 0, stream>>>((const gd_half *)logits, ids, gap, cols, none);
     else
-        gd_argmax_rows_kernel<float><<<(unsigned)rows, GD_ARGMAX_THREADS, 0, stream>>>((const float *)logits, ids, gap, cols);
+        gd_argmax_rows_kernel<float, false><<<(unsigned)rows, GD_ARGMAX_THREADS, 0, stream>>>((const float *)logits, ids, gap, cols, none);
+    return (int)hipGetLastError();
+}
+
+extern "C" int gd_hip_launch_argmax_advance(hipStream_t stream, const void *logits, int32_t *ids, uint64_t rows,
+                                            uint64_t cols, int is_f16, int32_t *positions, int32_t *step_counters,
+                                            int32_t *out_ids, float *out_gaps, uint32_t max_steps, int32_t pos_delta)
+{
+    const gd_hip_advance adv = {positions, step_counters, out_ids, out_gaps, max_steps, pos_delta};
+    if (rows == 0) return (int)hipSuccess;
+    if (is_f16)
+        gd_argmax_rows_kernel<gd_half, true><<<(unsigned)rows, GD_ARGMAX_THREADS, 0, stream>>>((const gd_half *)logits, ids, nullptr, cols, adv);
+    else
+        gd_argmax_rows_kernel<float, true><<<(unsigned)rows, GD_ARGMAX_THREADS, 0, stream>>>((const float *)logits, ids, nullptr, cols, adv);
     return (int)hipGetLastError();
 }

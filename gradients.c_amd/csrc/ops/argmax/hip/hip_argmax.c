@@ -1,4 +1,4 @@
-/* Host dispatch of gd_backend_argmax_rows (no counterpart in the reference's backend). */
+/* Host dispatch of gd_backend_argmax_rows and gd_backend_argmax_advance (no counterpart in the reference's backend). */
 #include "../../../backends/hip/backend_hip_internal.h"
 
 int gd_hip_launch_argmax_rows(hipStream_t stream, const void *logits, int32_t *ids, float *gap, uint64_t rows,
@@ -22,4 +22,41 @@ gd_status gd_backend_argmax_rows(gd_backend *backend, const gd_backend_tensor_vi
     return gd_hip_finish_op(backend, gd_hip_launch_argmax_rows(
         backend->stream, gd_hip_view_ptr(logits), (int32_t *)gd_hip_view_ptr(ids),
         gap != NULL ? (float *)gd_hip_view_ptr(gap) : NULL, rows, cols, logits->dtype == GD_BACKEND_DTYPE_F16));
+}
+
+int gd_hip_launch_argmax_advance(hipStream_t stream, const void *logits, int32_t *ids, uint64_t rows, uint64_t cols,
+                                 int is_f16, int32_t *positions, int32_t *step_counters, int32_t *out_ids,
+                                 float *out_gaps, uint32_t max_steps, int32_t pos_delta);
+
+static int i32_rows(const gd_backend_tensor_view *v, uint64_t rows)
+{
+    return gd_hip_view_ok(v) && v->dtype == GD_BACKEND_DTYPE_I32 && v->count == (size_t)rows && (v->offset & 3u) == 0u;
+}
+
+gd_status gd_backend_argmax_advance(gd_backend *backend, const gd_backend_tensor_view *logits,
+                                    const gd_backend_tensor_view *ids, const gd_backend_tensor_view *positions,
+                                    const gd_backend_tensor_view *step_counters,
+                                    const gd_backend_tensor_view *out_ids, const gd_backend_tensor_view *out_gaps,
+                                    int32_t pos_delta)
+{
+    uint64_t rows, cols, max_steps;
+    if (backend == NULL || !gd_hip_view_ok(logits) || logits->rank != 2u || !gd_hip_view_ok(out_ids) ||
+        (out_gaps != NULL && !gd_hip_view_ok(out_gaps)))
+        return GD_ERR_INVALID_ARGUMENT;
+    if ((logits->dtype != GD_BACKEND_DTYPE_F16 && logits->dtype != GD_BACKEND_DTYPE_F32) ||
+        out_ids->dtype != GD_BACKEND_DTYPE_I32 || (out_gaps != NULL && out_gaps->dtype != GD_BACKEND_DTYPE_F32))
+        return GD_ERR_UNSUPPORTED;
+    rows = (uint64_t)logits->shape[0];
+    cols = (uint64_t)logits->shape[1];
+    if (rows == 0u || rows > 0x7fffffffu || cols > 0x7fffffffu || !i32_rows(ids, rows) || !i32_rows(positions, rows) ||
+        !i32_rows(step_counters, rows) || (out_ids->count % rows) != 0u || (out_ids->offset & 3u) != 0u ||
+        (out_gaps != NULL && (out_gaps->count != out_ids->count || (out_gaps->offset & 3u) != 0u)))
+        return GD_ERR_INVALID_ARGUMENT;
+    max_steps = out_ids->count / rows;
+    if (max_steps > 0xffffffffu) return GD_ERR_INVALID_ARGUMENT;
+    return gd_hip_finish_op(backend, gd_hip_launch_argmax_advance(
+        backend->stream, gd_hip_view_ptr(logits), (int32_t *)gd_hip_view_ptr(ids), rows, cols,
+        logits->dtype == GD_BACKEND_DTYPE_F16, (int32_t *)gd_hip_view_ptr(positions),
+        (int32_t *)gd_hip_view_ptr(step_counters), (int32_t *)gd_hip_view_ptr(out_ids),
+        out_gaps != NULL ? (float *)gd_hip_view_ptr(out_gaps) : NULL, (uint32_t)max_steps, pos_delta));
 }

@@ -8,7 +8,7 @@
 
 int gd_hip_launch_linear(hipStream_t stream, const void *x, const void *w, const void *bias, const void *residual,
                          const void *norm_w, void *y, const gd_hip_linear_params *params, int vector_ok,
-                         int kn_vector_ok, int store_vector_ok, int min_workgroups);
+                         int kn_vector_ok, int store_vector_ok, int min_workgroups, const gd_hip_rope_epilogue *rope);
 
 static gd_status project_full(gd_backend *backend, const gd_backend_matrix_view *x, const gd_backend_matrix_view *w,
                               const gd_backend_vector_view *bias, const gd_backend_matrix_view *residual,
@@ -62,16 +62,19 @@ static gd_status project_full(gd_backend *backend, const gd_backend_matrix_view 
     p.ldr = residual != NULL ? (uint32_t)(residual->row_bytes / 2u) : 0u;
     p.eps = eps;
     p.swiglu_cols = gated ? y->cols : 0u;
+    p.rope_heads = p.rope_head_dim = p.rope_tmax = 0u;
+    p.rope_freq_scale = 0.0f;
     /* 16-byte fragment loads: x rows always, w rows when K-contiguous, the norm weight */
     vec = (K % 8u) == 0u && ((x->offset | x->row_bytes) & 15u) == 0u &&
           (!w_is_nk || ((w->offset | w->row_bytes) & 15u) == 0u) && (norm_w == NULL || (norm_w->offset & 15u) == 0u);
     kn_vec = !w_is_nk && (p.N % 8u) == 0u && ((w->offset | w->row_bytes) & 15u) == 0u;
     store_vec = ((y->offset | y->row_bytes) & 15u) == 0u &&
                 (residual == NULL || ((residual->offset | residual->row_bytes) & 15u) == 0u);
+    if (gated && !vec) return GD_ERR_UNSUPPORTED;
     return gd_hip_finish_op(backend, gd_hip_launch_linear(
         backend->stream, gd_hip_matrix_ptr(x), gd_hip_matrix_ptr(w), bias != NULL ? gd_hip_vector_ptr(bias) : NULL,
         residual != NULL ? gd_hip_matrix_ptr(residual) : NULL, norm_w != NULL ? gd_hip_vector_ptr(norm_w) : NULL,
-        gd_hip_matrix_ptr(y), &p, vec, kn_vec, store_vec, 2 * backend->compute_units));
+        gd_hip_matrix_ptr(y), &p, vec, kn_vec, store_vec, 2 * backend->compute_units, NULL));
 }
 
 static gd_status project(gd_backend *backend, const gd_backend_matrix_view *x, const gd_backend_matrix_view *w,
@@ -125,4 +128,80 @@ gd_status gd_backend_fused_linear(gd_backend *backend, const gd_backend_matrix_v
         return GD_ERR_INVALID_ARGUMENT;
     return project_full(backend, x, w, bias, residual, norm_weight, args->eps, y, args->w_is_nk != 0u, args->bias_mode,
                         args->prologue, args->epilogue);
+}
+
+#include <math.h>
+
+/* qkv projection of a decode step with the rotation and the cache append in its epilogue */
+gd_status gd_backend_fused_qkv_rope_append(gd_backend *backend, const gd_backend_matrix_view *x,
+                                           const gd_backend_matrix_view *w, const gd_backend_vector_view *bias,
+                                           const gd_backend_vector_view *norm_weight,
+                                           const gd_backend_tensor_view *pos_ids, const gd_backend_tensor_view *cache_pos,
+                                           const gd_backend_tensor_view *q, const gd_backend_tensor_view *k_cache,
+                                           const gd_backend_tensor_view *v_cache, uint32_t n_heads, uint32_t head_dim,
+                                           const gd_backend_rope_args *rope_args,
+                                           const gd_backend_fused_linear_args *args)
+{
+    gd_hip_linear_params p;
+    gd_hip_rope_epilogue r;
+    uint64_t area;
+    uint32_t i;
+    if (backend == NULL || args == NULL || rope_args == NULL || !gd_hip_matrix_ok(x) || !gd_hip_matrix_ok(w) ||
+        (bias != NULL && !gd_hip_vector_ok(bias)) || (norm_weight != NULL && !gd_hip_vector_ok(norm_weight)) ||
+        !gd_hip_view_ok(pos_ids) || !gd_hip_view_ok(cache_pos) || !gd_hip_view_ok(q) || !gd_hip_view_ok(k_cache) ||
+        !gd_hip_view_ok(v_cache) || n_heads == 0u || head_dim == 0u || pos_ids->rank != 1u || cache_pos->rank != 1u ||
+        q->rank != 3u || k_cache->rank != 4u || v_cache->rank != 4u || args->bias_mode > 2u || args->epilogue != 0u ||
+        (args->prologue != GD_HIP_PRO_NONE && args->prologue != GD_HIP_PRO_RMS_NORM) ||
+        (args->bias_mode != 0u) != (bias != NULL) || (args->prologue == GD_HIP_PRO_RMS_NORM) != (norm_weight != NULL))
+        return GD_ERR_INVALID_ARGUMENT;
+    if (x->dtype != GD_BACKEND_DTYPE_F16 || w->dtype != GD_BACKEND_DTYPE_F16 || q->dtype != GD_BACKEND_DTYPE_F16 ||
+        k_cache->dtype != GD_BACKEND_DTYPE_F16 || v_cache->dtype != GD_BACKEND_DTYPE_F16 ||
+        (bias != NULL && bias->dtype != GD_BACKEND_DTYPE_F16) ||
+        (norm_weight != NULL && norm_weight->dtype != GD_BACKEND_DTYPE_F16) ||
+        pos_ids->dtype != GD_BACKEND_DTYPE_I32 || cache_pos->dtype != GD_BACKEND_DTYPE_I32)
+        return GD_ERR_UNSUPPORTED;
+    area = (uint64_t)n_heads * head_dim;
+    for (i = 0u; i < 4u; ++i) {
+        if (k_cache->shape[i] != v_cache->shape[i]) return GD_ERR_INVALID_ARGUMENT;
+    }
+    if (area * 3u > 0xffffffffu || w->rows != (uint32_t)(area * 3u) || w->cols != x->cols ||
+        (bias != NULL && bias->length != w->rows) || (norm_weight != NULL && (norm_weight->length != x->cols || !(args->eps > 0.0f))) ||
+        pos_ids->shape[0] != (int64_t)x->rows || cache_pos->shape[0] != (int64_t)x->rows ||
+        q->shape[0] != (int64_t)x->rows || q->shape[1] != (int64_t)n_heads || q->shape[2] != (int64_t)head_dim ||
+        k_cache->shape[0] != (int64_t)x->rows || k_cache->shape[2] != (int64_t)n_heads ||
+        k_cache->shape[3] != (int64_t)head_dim || k_cache->shape[1] > (int64_t)INT32_MAX || !(rope_args->theta > 0.0f) ||
+        rope_args->n_dims != head_dim || ((pos_ids->offset | cache_pos->offset) & 3u) != 0u)
+        return GD_ERR_INVALID_ARGUMENT;
+    /* the few-row kernel with column pairs (c, c + head_dim/2) in one workgroup: [N,K] weight, NeoX pairing,
+     * head size a multiple of 32, fewer than 128 rows, 16-byte aligned operand rows */
+    if (args->w_is_nk == 0u || rope_args->interleaved != 0u || (head_dim % 32u) != 0u || x->rows >= 128u ||
+        (x->cols % 8u) != 0u || ((x->offset | x->row_bytes | w->offset | w->row_bytes) & 15u) != 0u ||
+        (norm_weight != NULL && (norm_weight->offset & 15u) != 0u) ||
+        ((q->offset | k_cache->offset | v_cache->offset) & 1u) != 0u)
+        return GD_ERR_UNSUPPORTED;
+    p.M = x->rows;
+    p.N = w->rows;
+    p.K = x->cols;
+    p.ldx = (uint32_t)(x->row_bytes / 2u);
+    p.ldw = (uint32_t)(w->row_bytes / 2u);
+    p.ldy = 0u;
+    p.epilogue = bias != NULL ? args->bias_mode : GD_HIP_EPI_NONE;
+    p.w_is_nk = 1u;
+    p.prologue = args->prologue;
+    p.has_residual = 0u;
+    p.ldr = 0u;
+    p.eps = args->eps;
+    p.swiglu_cols = 0u;
+    p.rope_heads = n_heads;
+    p.rope_head_dim = head_dim;
+    p.rope_tmax = (uint32_t)k_cache->shape[1];
+    p.rope_freq_scale = -2.0f * log2f(rope_args->theta) / (float)head_dim;
+    r.rope_pos = (const int32_t *)gd_hip_view_ptr(pos_ids);
+    r.cache_pos = (const int32_t *)gd_hip_view_ptr(cache_pos);
+    r.q = gd_hip_view_ptr(q);
+    r.k_cache = gd_hip_view_ptr(k_cache);
+    r.v_cache = gd_hip_view_ptr(v_cache);
+    return gd_hip_finish_op(backend, gd_hip_launch_linear(
+        backend->stream, gd_hip_matrix_ptr(x), gd_hip_matrix_ptr(w), bias != NULL ? gd_hip_vector_ptr(bias) : NULL, NULL,
+        norm_weight != NULL ? gd_hip_vector_ptr(norm_weight) : NULL, NULL, &p, 1, 0, 0, 2 * backend->compute_units, &r));
 }

@@ -23,6 +23,16 @@ typedef struct gd_hip_linear_params {
     float eps;              /* rms_norm prologue */
     uint32_t swiglu_cols;   /* 0, or H: w has 2H rows ([N,K] only); y [M,H] = half(u[:, :H] * silu(u[:, H:])) where u is
                              * the projection after the bias epilogue, rounded to F16 like a stored intermediate */
+    /* rope + cache append epilogue (rope_head_dim != 0): the projection is the qkv projection of a decode step,
+     * N = 3 * heads * head_dim; see gd_hip_rope_epilogue */
+    uint32_t rope_heads, rope_head_dim, rope_tmax;
+    float rope_freq_scale;
 } gd_hip_linear_params;
+
+/* destinations of the rope + append epilogue: q [M,H,D]; caches [M,Tmax,H,D]; positions I32 [M] */
+typedef struct gd_hip_rope_epilogue {
+    const int32_t *rope_pos, *cache_pos;
+    void *q, *k_cache, *v_cache;
+} gd_hip_rope_epilogue;
 
 #endif

@@ -29,6 +29,7 @@
  */
 #include "../../_shared/hip_device.h"
 #include "hip_linear_types.h"
+#include "../../qkv_split_rope/hip/rope_device.h"
 #include <type_traits>
 
 __device__ __forceinline__ float gd_lin_silu(float z)
@@ -43,7 +44,7 @@ __global__ void __launch_bounds__(WAVES * 64)
 gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__ w,
                         const gd_half *__restrict__ bias, const gd_half *__restrict__ residual,
                         const gd_half *__restrict__ norm_w, gd_half *__restrict__ y, gd_hip_linear_params p,
-                        uint32_t n_tiles)
+                        uint32_t n_tiles, gd_hip_rope_epilogue rope)
 {
     constexpr int U = NT >= 4 ? 2 : 4;  /* K steps per register set; two sets alternate */
     constexpr int RES_STEPS = 8;        /* RES: the wavefront's whole K slice of the activation stays in registers */
@@ -62,8 +63,15 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
     if ((n_tiles & 7u) == 0u) tile = (blockIdx.x & 7u) * (n_tiles >> 3) + (blockIdx.x >> 3);
     /* gated (swiglu epilogue): the first NT/2 column tiles are value columns, the others the matching gate columns
      * swiglu_cols further down the weight; the workgroup then owns COLS/2 output columns */
-    const bool gated = NT >= 2 && p.swiglu_cols != 0u;
-    const uint32_t n0 = tile * (gated ? COLS / 2u : COLS);
+    /* roped (rope + append epilogue): the same pairing inside one head: columns c and c + head_dim/2 */
+    const bool roped = NT >= 2 && p.rope_head_dim != 0u;
+    const bool gated = NT >= 2 && (p.swiglu_cols != 0u || roped);
+    const uint32_t pair_offset = roped ? p.rope_head_dim / 2u : p.swiglu_cols;
+    uint32_t n0 = tile * (gated ? COLS / 2u : COLS);
+    if (roped) {
+        const uint32_t per_head = (p.rope_head_dim / 2u) / (COLS / 2u); /* workgroups per head and section */
+        n0 = (tile / per_head) * p.rope_head_dim + (tile % per_head) * (COLS / 2u);
+    }
     const uint32_t m0 = blockIdx.y * 16u;
     const uint32_t mrow = min(m0 + (uint32_t)li, p.M - 1u);
 
@@ -92,7 +100,7 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
                 if (W_NK) {
                     /* clamped: out-of-range columns are never stored */
                     const uint32_t n = (gated && j >= NT / 2)
-                                           ? p.swiglu_cols + min(n0 + 16u * (uint32_t)(j - NT / 2) + (uint32_t)li, p.N - 1u)
+                                           ? pair_offset + min(n0 + 16u * (uint32_t)(j - NT / 2) + (uint32_t)li, p.N - 1u)
                                            : min(n0 + 16u * (uint32_t)j + (uint32_t)li, p.N - 1u);
                     if (kok) bf[set][u][j] = *reinterpret_cast<const gd_half8 *>(w + (size_t)n * p.ldw + k);
                 } else {
@@ -248,15 +256,41 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
                 gd_half h1, h2;
                 if (p.epilogue == GD_HIP_EPI_BIAS_F32) {
                     h1 = (gd_half)(v1 + (float)bias[col]);
-                    h2 = (gd_half)(v2 + (float)bias[p.swiglu_cols + col]);
+                    h2 = (gd_half)(v2 + (float)bias[pair_offset + col]);
                 } else if (p.epilogue == GD_HIP_EPI_BIAS_F16) {
                     h1 = (gd_half)v1 + bias[col];
-                    h2 = (gd_half)v2 + bias[p.swiglu_cols + col];
+                    h2 = (gd_half)v2 + bias[pair_offset + col];
                 } else {
                     h1 = (gd_half)v1;
                     h2 = (gd_half)v2;
                 }
-                y[(size_t)row * p.ldy + col] = (gd_half)((float)h1 * gd_lin_silu((float)h2));
+                if (!roped) {
+                    y[(size_t)row * p.ldy + col] = (gd_half)((float)h1 * gd_lin_silu((float)h2));
+                } else {
+                    /* col = (section * heads + head) * head_dim + pair: q is rotated into its own tensor, k rotated and
+                     * v copied into row cache_pos of the sequence's caches (skipped when that row does not exist) */
+                    const uint32_t D = p.rope_head_dim, area = p.rope_heads * D;
+                    const uint32_t section = col / area, within = col % area, pair = within % D;
+                    gd_half o1 = h1, o2 = h2;
+                    if (section < 2u) {
+                        float c, sn;
+                        gd_rope_cos_sin((float)rope.rope_pos[row], pair, p.rope_freq_scale, &c, &sn);
+                        gd_rope_rotate((float)h1, (float)h2, c, sn, &o1, &o2);
+                    }
+                    if (section == 0u) {
+                        gd_half *dst = (gd_half *)rope.q + (size_t)row * area + within;
+                        dst[0] = o1;
+                        dst[D / 2u] = o2;
+                    } else {
+                        const int32_t cp = rope.cache_pos[row];
+                        if (cp >= 0 && (uint32_t)cp < p.rope_tmax) {
+                            gd_half *dst = (gd_half *)(section == 1u ? rope.k_cache : rope.v_cache) +
+                                           ((size_t)row * p.rope_tmax + (size_t)cp) * area + within;
+                            dst[0] = o1;
+                            dst[D / 2u] = o2;
+                        }
+                    }
+                }
             }
         }
         return;
@@ -314,15 +348,17 @@ gd_linear_scalar_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
 
 template <int NT, int WAVES>
 static void launch_stream(hipStream_t stream, const gd_half *x, const gd_half *w, const gd_half *bias,
-                          const gd_half *residual, const gd_half *norm_w, gd_half *y, const gd_hip_linear_params &p)
+                          const gd_half *residual, const gd_half *norm_w, gd_half *y, const gd_hip_linear_params &p,
+                          const gd_hip_rope_epilogue &rope)
 {
-    const uint32_t cols = p.swiglu_cols != 0u ? 8u * NT : 16u * NT; /* output columns per workgroup */
-    const uint32_t n_tiles = (p.N + cols - 1u) / cols;
+    const bool paired = p.swiglu_cols != 0u || p.rope_head_dim != 0u;
+    const uint32_t cols = paired ? 8u * NT : 16u * NT; /* first-of-pair / plain output columns per workgroup */
+    const uint32_t n_tiles = p.rope_head_dim != 0u ? (p.N / 2u) / cols : (p.N + cols - 1u) / cols;
     dim3 grid(n_tiles, (p.M + 15u) / 16u);
     const int threads = WAVES * 64;
     /* the whole K slice of a wavefront fits the resident registers (8 steps of 32) */
     const bool res = ((p.K + 31u) / 32u + WAVES - 1u) / WAVES <= 8u;
-#define GD_GO(NK, PRO, RES) gd_linear_stream_kernel<NT, WAVES, NK, PRO, RES><<<grid, threads, 0, stream>>>(x, w, bias, residual, norm_w, y, p, n_tiles)
+#define GD_GO(NK, PRO, RES) gd_linear_stream_kernel<NT, WAVES, NK, PRO, RES><<<grid, threads, 0, stream>>>(x, w, bias, residual, norm_w, y, p, n_tiles, rope)
     if (p.w_is_nk) {
         if (p.prologue == GD_HIP_PRO_SWIGLU) GD_GO(true, GD_HIP_PRO_SWIGLU, false);
         else if (p.prologue == GD_HIP_PRO_RMS_NORM) { if (res) GD_GO(true, GD_HIP_PRO_RMS_NORM, true); else GD_GO(true, GD_HIP_PRO_RMS_NORM, false); }
@@ -345,8 +381,10 @@ extern "C" int gd_hip_launch_linear_tile(hipStream_t stream, const void *x, cons
 extern "C" int gd_hip_launch_linear(hipStream_t stream, const void *x, const void *w, const void *bias,
                                     const void *residual, const void *norm_w, void *y,
                                     const gd_hip_linear_params *params, int vector_ok, int kn_vector_ok,
-                                    int store_vector_ok, int min_workgroups)
+                                    int store_vector_ok, int min_workgroups, const gd_hip_rope_epilogue *rope_epilogue)
 {
+    const gd_hip_rope_epilogue no_rope = {nullptr, nullptr, nullptr, nullptr, nullptr};
+    const gd_hip_rope_epilogue &rope = rope_epilogue != nullptr ? *rope_epilogue : no_rope;
     const gd_hip_linear_params &p = *params;
     const gd_half *xp = (const gd_half *)x, *wp = (const gd_half *)w, *bp = (const gd_half *)bias;
     const gd_half *rp = (const gd_half *)residual, *np = (const gd_half *)norm_w;
@@ -355,7 +393,7 @@ extern "C" int gd_hip_launch_linear(hipStream_t stream, const void *x, const voi
     if (!vector_ok || p.K == 0 || (!p.w_is_nk && !kn_vector_ok)) {
         const uint64_t total = (uint64_t)p.M * p.N;
         gd_linear_scalar_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(xp, wp, bp, rp, np, yp, p);
-    } else if (p.M >= 128u && (p.w_is_nk || kn_vector_ok) && p.swiglu_cols == 0u) {
+    } else if (p.M >= 128u && (p.w_is_nk || kn_vector_ok) && p.swiglu_cols == 0u && p.rope_head_dim == 0u) {
         /* matrix-core bound: LDS-tiled kernel; the 256 x 256 tile once it still gives every compute unit
          * a workgroup, the 128 x 128 tile below that */
         const uint64_t big = (uint64_t)((p.M + 255u) / 256u) * ((p.N + 255u) / 256u);
@@ -367,12 +405,15 @@ extern "C" int gd_hip_launch_linear(hipStream_t stream, const void *x, const voi
          * in fewer workgroups, but leave fewer workgroups; the grid keeps at least one per compute unit. */
         const uint64_t mt = (p.M + 15u) / 16u;
         const uint32_t target = min_workgroups > 0 ? (uint32_t)min_workgroups / 2u : 256u;
-        if (p.swiglu_cols != 0u) { /* value and gate tiles side by side: 32 or 16 output columns per workgroup */
-            if (((p.N + 31u) / 32u) * mt >= target) launch_stream<4, 8>(stream, xp, wp, bp, rp, np, yp, p);
-            else launch_stream<2, 8>(stream, xp, wp, bp, rp, np, yp, p);
-        } else if (((p.N + 63u) / 64u) * mt >= target) launch_stream<4, 8>(stream, xp, wp, bp, rp, np, yp, p);
-        else if (((p.N + 31u) / 32u) * mt >= target) launch_stream<2, 8>(stream, xp, wp, bp, rp, np, yp, p);
-        else launch_stream<1, 8>(stream, xp, wp, bp, rp, np, yp, p);
+        if (p.rope_head_dim != 0u) { /* pairs (c, c + head_dim/2): 32 or 16 pairs per workgroup; head_dim % 32 == 0 */
+            if ((p.rope_head_dim % 64u) == 0u && (p.N / 64u) * mt >= target) launch_stream<4, 8>(stream, xp, wp, bp, rp, np, yp, p, rope);
+            else launch_stream<2, 8>(stream, xp, wp, bp, rp, np, yp, p, rope);
+        } else if (p.swiglu_cols != 0u) { /* value and gate tiles side by side: 32 or 16 output columns per workgroup */
+            if (((p.N + 31u) / 32u) * mt >= target) launch_stream<4, 8>(stream, xp, wp, bp, rp, np, yp, p, rope);
+            else launch_stream<2, 8>(stream, xp, wp, bp, rp, np, yp, p, rope);
+        } else if (((p.N + 63u) / 64u) * mt >= target) launch_stream<4, 8>(stream, xp, wp, bp, rp, np, yp, p, rope);
+        else if (((p.N + 31u) / 32u) * mt >= target) launch_stream<2, 8>(stream, xp, wp, bp, rp, np, yp, p, rope);
+        else launch_stream<1, 8>(stream, xp, wp, bp, rp, np, yp, p, rope);
     }
     return (int)hipGetLastError();
 }

@@ -9,19 +9,7 @@
  * NeoX layout, D % 16 == 0: one thread owns 8 consecutive pairs of one (token, head): two 16-byte
  * loads per tensor (low half and high half of the head), two 16-byte stores.
  */
-#include "../../_shared/hip_device.h"
-
-/* Explicitly rounded steps so every kernel of this file produces the same bits for the same input. */
-__device__ __forceinline__ void gd_rope_cos_sin(float fpos, uint32_t pair, float freq_scale, float *c, float *s)
-{
-    sincosf(__fmul_rn(fpos, exp2f(__fmul_rn((float)pair, freq_scale))), s, c);
-}
-
-__device__ __forceinline__ void gd_rope_rotate(float x0, float x1, float c, float s, gd_half *o0, gd_half *o1)
-{
-    *o0 = (gd_half)__fmaf_rn(x0, c, -__fmul_rn(x1, s));
-    *o1 = (gd_half)__fmaf_rn(x0, s, __fmul_rn(x1, c));
-}
+#include "rope_device.h"
 
 /* cache_pos == nullptr: k and v go to row n of [N,H,D] tensors (split form).  Otherwise they go to
  * row cache_pos[n] of sequence n in [N,Tmax,H,D] caches (decode form, one new token per sequence);

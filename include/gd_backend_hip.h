@@ -391,6 +391,31 @@ gd_status gd_backend_decode_advance(gd_backend *backend, const gd_backend_tensor
                                     const gd_backend_tensor_view *out_ids,
                                     const gd_backend_tensor_view *out_gaps, int32_t pos_delta);
 
+/* gd_backend_fused_linear (prologue 0 or 2, w [3*H*D, K] with w_is_nk = 1, any bias mode) followed by
+ * gd_backend_qkv_rope_append on its result, in one launch: the [B, 3*H*D] projection is never stored; its q
+ * columns are rotated into q [B,H,D], its k columns rotated and its v columns copied into row cache_pos[b] of the
+ * caches [B,Tmax,H,D] (sequences whose position is negative or >= Tmax keep their caches).  Same rounding points
+ * as the separate operators.  NeoX pairing, head_dim % 32 == 0, fewer than 128 rows, else UNSUPPORTED. */
+gd_status gd_backend_fused_qkv_rope_append(gd_backend *backend, const gd_backend_matrix_view *x,
+                                           const gd_backend_matrix_view *w, const gd_backend_vector_view *bias,
+                                           const gd_backend_vector_view *norm_weight,
+                                           const gd_backend_tensor_view *pos_ids, const gd_backend_tensor_view *cache_pos,
+                                           const gd_backend_tensor_view *q, const gd_backend_tensor_view *k_cache,
+                                           const gd_backend_tensor_view *v_cache, uint32_t n_heads, uint32_t head_dim,
+                                           const gd_backend_rope_args *rope_args,
+                                           const gd_backend_fused_linear_args *args);
+
+/* gd_backend_argmax_rows and the bookkeeping of gd_backend_decode_advance in one launch, for a loop that
+ * feeds its own tokens: ids[b] = greedy token of logits row b; positions[b] += pos_delta;
+ * s = step_counters[b]; when s < max_steps (= out_ids count / rows), out_ids[s*B + b] = token and
+ * (out_gaps != NULL) out_gaps[s*B + b] = best - runner-up; step_counters[b] = s + 1.  Every row keeps its
+ * own counter (I32 [B]) because every row is handled by its own workgroup. */
+gd_status gd_backend_argmax_advance(gd_backend *backend, const gd_backend_tensor_view *logits,
+                                    const gd_backend_tensor_view *ids, const gd_backend_tensor_view *positions,
+                                    const gd_backend_tensor_view *step_counters,
+                                    const gd_backend_tensor_view *out_ids, const gd_backend_tensor_view *out_gaps,
+                                    int32_t pos_delta);
+
 /* Device copy between buffers, enqueued like an operator. */
 gd_status gd_backend_copy(gd_backend *backend, gd_backend_buffer *dst, size_t dst_offset,
                           gd_backend_buffer *src, size_t src_offset, size_t nbytes);

@@ -738,6 +738,56 @@ def test_fused_linear_swiglu_epilogue(backend, arena, oracle, gda, M, K, H):
     assert backend.call("gd_backend_fused_linear", tx.matrix(), wk.matrix(), None, None, None, y.matrix(), C.byref(a)) == gda.UNSUPPORTED
 
 
+@pytest.mark.parametrize("B,H,D,K", [(64, 8, 64, 512), (16, 16, 128, 2048), (5, 3, 32, 72), (33, 2, 96, 64)])
+def test_fused_qkv_rope_append_equals_separate_ops(backend, arena, oracle, gda, B, H, D, K):
+    """rms_norm -> qkv projection (+F16 bias) -> rope -> cache append in one launch against the fused projection
+    followed by the rope + append operator.  The projection result is rounded to F16 at the same point, so v is
+    bit-identical; the rotation runs in a different kernel, where the compiler may contract the trigonometric range
+    reduction differently: q and k agree to one F16 unit in the last place in all but a few elements per thousand."""
+    Tmax = 24
+    x = oracle.normal_f16((B, K), 2700 + K, 1.2)
+    nw = (1.0 + 0.1 * oracle.normal_f16((K,), 2701).astype(np.float32)).astype(np.float16)
+    w = oracle.normal_f16((3 * H * D, K), 2702 + D, 0.05)
+    bias = oracle.normal_f16((3 * H * D,), 2703, 0.3)
+    pos = oracle.uniform_i32(B, 2704, 0, 4000)
+    cpos = oracle.uniform_i32(B, 2705, 0, Tmax - 1)
+    cpos[0] = -1
+    if B > 2:
+        cpos[2] = Tmax
+    k0, v0 = oracle.normal_f16((B, Tmax, H, D), 2706), oracle.normal_f16((B, Tmax, H, D), 2707)
+    tx, tw, tb, tn = (arena.from_numpy(a) for a in (x, w, bias, nw))
+    tp, tc = arena.from_numpy(pos), arena.from_numpy(cpos)
+    q1, k1, v1 = arena.alloc((B, H, D), 1), arena.from_numpy(k0), arena.from_numpy(v0)
+    backend.fused_qkv_rope_append(tx, tw, tb, tn, tp, tc, q1, k1, v1, H, D, 2, 2, 1e-5)
+    qkv = arena.alloc((B, 3 * H * D), 1)
+    q2, k2, v2 = arena.alloc((B, H, D), 1), arena.from_numpy(k0), arena.from_numpy(v0)
+    backend.fused_linear(tx, tw, tb, None, tn, qkv, True, 2, 2, 1e-5)
+    backend.qkv_rope_append(qkv, tp, tc, q2, k2, v2, H, D)
+    def one_ulp(a, b):
+        a32, b32 = a.astype(np.float32), b.astype(np.float32)
+        ulp = np.spacing(np.maximum(np.abs(a), np.abs(b)).astype(np.float16)).astype(np.float32)
+        assert np.all(np.abs(a32 - b32) <= ulp)
+        assert np.count_nonzero(_bits(a) != _bits(b)) <= max(2, a.size // 500)
+
+    one_ulp(q1.read(), q2.read())
+    one_ulp(k1.read(), k2.read())
+    assert np.array_equal(_bits(v1.read()), _bits(v2.read()))
+    # and against the oracle chain, to tolerance
+    u = oracle.linear_nt(oracle.rms_norm(x, nw, 1e-5), w, bias)
+    qo, ko, vo = oracle.qkv_split_rope(u, pos, H, D)
+    _close(q1.read(), qo, atol=4e-3)
+    got_k = k1.read()
+    for b in range(B):
+        if 0 <= cpos[b] < Tmax:
+            _close(got_k[b, cpos[b]], ko[b], atol=4e-3)
+    # without norm and bias
+    backend.fused_qkv_rope_append(tx, tw, None, None, tp, tc, q1, k1, v1, H, D, 0, 0)
+    backend.fused_linear(tx, tw, None, None, None, qkv, True, 0, 0)
+    backend.qkv_rope_append(qkv, tp, tc, q2, k2, v2, H, D)
+    one_ulp(q1.read(), q2.read())
+    one_ulp(k1.read(), k2.read())
+
+
 def test_fused_linear_rejects_bad_arguments(backend, arena, gda):
     x, w, y = arena.alloc((4, 16), gda.F16), arena.alloc((8, 16), gda.F16), arena.alloc((4, 8), gda.F16)
     b = arena.alloc((8,), gda.F16)
