@@ -141,7 +141,7 @@ _SIGNATURES = {
     "gd_backend_decode_advance": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, _TV, C.c_int32],
     "gd_backend_fused_qkv_rope_append": [_vp, _MV, _MV, _VV, _VV, _TV, _TV, _TV, _TV, _TV, C.c_uint32, C.c_uint32,
                                          C.POINTER(RopeArgs), C.POINTER(FusedLinearArgs)],
-    "gd_backend_argmax_advance": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, C.c_int32],
+    "gd_backend_argmax_advance": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, C.c_int32, _TV, _TV],
     "gd_backend_copy": [_vp, _vp, C.c_size_t, _vp, C.c_size_t, C.c_size_t],
     "gd_backend_timer_create": [_vp, C.POINTER(_vp)],
     "gd_backend_timer_start": [_vp],

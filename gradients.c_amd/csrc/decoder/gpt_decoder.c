@@ -37,6 +37,8 @@ struct gd_gpt_decoder {
     int32_t *pos; /* host copy of the live lengths */
     /* device-resident decode state (state arena) */
     gd_tensor ids_dev, pos_dev, step_dev, step_rows_dev; /* step counters: one for the whole batch / one per row */
+    gd_tensor x0_dev;     /* [B, Dm]: embedding rows of the tokens the fused resident step starts from */
+    bool resident_x0;     /* x0_dev is kept current by the greedy-pick kernel */
     /* open resident session */
     bool resident_open;
     int32_t resident_max_steps, resident_steps, resident_hold, resident_unfused;
@@ -121,7 +123,8 @@ size_t gd_gpt_params_bytes(const gd_gpt_config *c)
 size_t gd_gpt_state_bytes(const gd_gpt_config *c)
 {
     const size_t cache = pad256((size_t)c->batch * (size_t)c->max_seq * (size_t)c->n_heads * (size_t)c->head_dim * 2U);
-    return cache * 2U * (size_t)c->n_layers + 4U * pad256((size_t)c->batch * 4U) + 4096U;
+    return cache * 2U * (size_t)c->n_layers + 4U * pad256((size_t)c->batch * 4U) +
+           pad256((size_t)c->batch * (size_t)c->d_model * 2U) + 4096U;
 }
 
 gd_status gd_gpt_decoder_create(gd_context *ctx, const gd_gpt_config *cfg, gd_gpt_decoder **out)
@@ -185,6 +188,10 @@ gd_status gd_gpt_decoder_create(gd_context *ctx, const gd_gpt_config *cfg, gd_gp
     STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_I32, gd_shape_make(1U, bdim), 256U, &d->pos_dev));
     STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_I32, gd_shape_make(1U, one), 256U, &d->step_dev));
     STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_I32, gd_shape_make(1U, bdim), 256U, &d->step_rows_dev));
+    {
+        int64_t xdim[2] = {cfg->batch, cfg->d_model};
+        STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_F16, gd_shape_make(2U, xdim), 256U, &d->x0_dev));
+    }
 #undef STEP
     if (st != GD_OK) {
         gd_gpt_decoder_destroy(d);
@@ -500,7 +507,8 @@ static gd_status enqueue_fused_step(gd_gpt_decoder *d, gd_tensor *logits)
     gd_backend_tensor_view vqkv, vpos, vq, vk, vv;
     int64_t q_shape[4] = {B, 1, c->n_heads, c->head_dim};
     int32_t l;
-    TRY(gd_embedding(ctx, &d->token_embedding, &d->ids_dev, &x));
+    if (d->resident_x0) x = d->x0_dev;
+    else TRY(gd_embedding(ctx, &d->token_embedding, &d->ids_dev, &x));
     for (l = 0; l < c->n_layers; ++l) {
         const gpt_block *b = &d->blocks[l];
         TRY(scratch_f16(ctx, B, Dm, &q));
@@ -583,7 +591,15 @@ static gd_status enqueue_resident_step(gd_gpt_decoder *d)
         view1(&d->step_rows_dev, &vs);
         view1(&d->resident_out_ids, &vo);
         view1(&d->resident_out_gaps, &vog);
-        return gd_backend_argmax_advance(gd_context_backend(ctx), &vl, &vi, &vp, &vs, &vo, &vog, d->resident_hold ? 0 : 1);
+        if (d->resident_x0) {
+            gd_backend_tensor_view vt, vx;
+            tview(&d->token_embedding, &vt);
+            tview(&d->x0_dev, &vx);
+            return gd_backend_argmax_advance(gd_context_backend(ctx), &vl, &vi, &vp, &vs, &vo, &vog,
+                                             d->resident_hold ? 0 : 1, &vt, &vx);
+        }
+        return gd_backend_argmax_advance(gd_context_backend(ctx), &vl, &vi, &vp, &vs, &vo, &vog, d->resident_hold ? 0 : 1,
+                                         NULL, NULL);
     }
     view1(&next, &vn);
     view1(&gaps, &vg);
@@ -635,6 +651,19 @@ gd_status gd_gpt_decoder_resident_begin(gd_gpt_decoder *d, const int32_t *first_
     dims[0] = (int64_t)max_steps * d->cfg.batch;
     st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_I32, gd_shape_make(1U, dims), 256U, &d->resident_out_ids);
     if (st == GD_OK) st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F32, gd_shape_make(1U, dims), 256U, &d->resident_out_gaps);
+    /* fused step: the greedy-pick kernel leaves the next input rows in x0_dev; the first ones are gathered here */
+    d->resident_x0 = !d->resident_unfused && (d->cfg.d_model % 8) == 0;
+    if (st == GD_OK && d->resident_x0) {
+        gd_backend_tensor_view vt, vi, vx;
+        gd_backend_embedding_args ea;
+        tview(&d->token_embedding, &vt);
+        tview(&d->ids_dev, &vi);
+        tview(&d->x0_dev, &vx);
+        ea.ids_count = (uint64_t)d->cfg.batch;
+        ea.vocab = (uint64_t)d->cfg.vocab;
+        ea.dim = (uint64_t)d->cfg.d_model;
+        st = gd_backend_embedding_forward(be, &vt, &vi, &vx, &ea);
+    }
     /* the first step runs eagerly (it also sizes the attention workspace); later steps replay a graph */
     if (st == GD_OK) st = enqueue_resident_step(d);
     if (st == GD_OK) d->resident_steps = 1;

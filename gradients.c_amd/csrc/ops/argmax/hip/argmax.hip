@@ -48,6 +48,10 @@ struct gd_hip_advance {
     float *out_gaps;        /* [max_steps * rows] or NULL */
     uint32_t max_steps;
     int32_t pos_delta;
+    /* optional: the chosen token's embedding row is copied to row b of next_x (the next step's input) */
+    const unsigned char *table; /* [vocab, row_bytes] */
+    unsigned char *next_x;      /* [rows, row_bytes] */
+    uint32_t row_bytes;         /* multiple of 16 */
 };
 
 template <typename T, bool ADVANCE>
@@ -56,6 +60,7 @@ gd_argmax_rows_kernel(const T *__restrict__ logits, int32_t *__restrict__ ids, f
                       uint64_t cols, gd_hip_advance adv)
 {
     __shared__ gd_top2 sm[GD_ARGMAX_THREADS / 64];
+    __shared__ int32_t s_token;
     const T *row = logits + (uint64_t)blockIdx.x * cols;
     gd_top2 t;
     t.best = GD_NEG_INF;
@@ -87,14 +92,21 @@ gd_argmax_rows_kernel(const T *__restrict__ logits, int32_t *__restrict__ ids, f
                 if (adv.out_gaps != nullptr) adv.out_gaps[(size_t)s * gridDim.x + blockIdx.x] = g;
             }
             adv.step_counters[blockIdx.x] = s + 1;
+            s_token = token;
         }
+    }
+    if (ADVANCE && adv.table != nullptr) {
+        __syncthreads();
+        const gd_u128 *src = reinterpret_cast<const gd_u128 *>(adv.table + (size_t)s_token * adv.row_bytes);
+        gd_u128 *dst = reinterpret_cast<gd_u128 *>(adv.next_x + (size_t)blockIdx.x * adv.row_bytes);
+        for (uint32_t c = threadIdx.x; c < adv.row_bytes / 16u; c += GD_ARGMAX_THREADS) dst[c] = src[c];
     }
 }
 
 extern "C" int gd_hip_launch_argmax_rows(hipStream_t stream, const void *logits, int32_t *ids, float *gap,
                                          uint64_t rows, uint64_t cols, int is_f16)
 {
-    const gd_hip_advance none = {nullptr, nullptr, nullptr, nullptr, 0u, 0};
+    const gd_hip_advance none = {nullptr, nullptr, nullptr, nullptr, 0u, 0, nullptr, nullptr, 0u};
     if (rows == 0) return (int)hipSuccess;
     if (is_f16)
         gd_argmax_rows_kernel<gd_half, false><<<(unsigned)rows, GD_ARGMAX_THREADS, 0, stream>>>((const gd_half *)logits, ids, gap, cols, none);
@@ -105,9 +117,11 @@ extern "C" int gd_hip_launch_argmax_rows(hipStream_t stream, const void *logits,
 
 extern "C" int gd_hip_launch_argmax_advance(hipStream_t stream, const void *logits, int32_t *ids, uint64_t rows,
                                             uint64_t cols, int is_f16, int32_t *positions, int32_t *step_counters,
-                                            int32_t *out_ids, float *out_gaps, uint32_t max_steps, int32_t pos_delta)
+                                            int32_t *out_ids, float *out_gaps, uint32_t max_steps, int32_t pos_delta,
+                                            const void *table, void *next_x, uint32_t row_bytes)
 {
-    const gd_hip_advance adv = {positions, step_counters, out_ids, out_gaps, max_steps, pos_delta};
+    const gd_hip_advance adv = {positions, step_counters, out_ids, out_gaps, max_steps, pos_delta,
+                                (const unsigned char *)table, (unsigned char *)next_x, row_bytes};
     if (rows == 0) return (int)hipSuccess;
     if (is_f16)
         gd_argmax_rows_kernel<gd_half, true><<<(unsigned)rows, GD_ARGMAX_THREADS, 0, stream>>>((const gd_half *)logits, ids, nullptr, cols, adv);

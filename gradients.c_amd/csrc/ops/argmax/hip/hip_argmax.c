@@ -26,7 +26,8 @@ gd_status gd_backend_argmax_rows(gd_backend *backend, const gd_backend_tensor_vi
 
 int gd_hip_launch_argmax_advance(hipStream_t stream, const void *logits, int32_t *ids, uint64_t rows, uint64_t cols,
                                  int is_f16, int32_t *positions, int32_t *step_counters, int32_t *out_ids,
-                                 float *out_gaps, uint32_t max_steps, int32_t pos_delta);
+                                 float *out_gaps, uint32_t max_steps, int32_t pos_delta, const void *table, void *next_x,
+                                 uint32_t row_bytes);
 
 static int i32_rows(const gd_backend_tensor_view *v, uint64_t rows)
 {
@@ -37,9 +38,10 @@ gd_status gd_backend_argmax_advance(gd_backend *backend, const gd_backend_tensor
                                     const gd_backend_tensor_view *ids, const gd_backend_tensor_view *positions,
                                     const gd_backend_tensor_view *step_counters,
                                     const gd_backend_tensor_view *out_ids, const gd_backend_tensor_view *out_gaps,
-                                    int32_t pos_delta)
+                                    int32_t pos_delta, const gd_backend_tensor_view *table,
+                                    const gd_backend_tensor_view *next_x)
 {
-    uint64_t rows, cols, max_steps;
+    uint64_t rows, cols, max_steps, row_bytes = 0u;
     if (backend == NULL || !gd_hip_view_ok(logits) || logits->rank != 2u || !gd_hip_view_ok(out_ids) ||
         (out_gaps != NULL && !gd_hip_view_ok(out_gaps)))
         return GD_ERR_INVALID_ARGUMENT;
@@ -53,10 +55,20 @@ gd_status gd_backend_argmax_advance(gd_backend *backend, const gd_backend_tensor
         (out_gaps != NULL && (out_gaps->count != out_ids->count || (out_gaps->offset & 3u) != 0u)))
         return GD_ERR_INVALID_ARGUMENT;
     max_steps = out_ids->count / rows;
-    if (max_steps > 0xffffffffu) return GD_ERR_INVALID_ARGUMENT;
+    if (max_steps > 0xffffffffu || (table == NULL) != (next_x == NULL)) return GD_ERR_INVALID_ARGUMENT;
+    if (table != NULL) {
+        if (!gd_hip_view_ok(table) || !gd_hip_view_ok(next_x) || table->rank != 2u || next_x->rank != 2u ||
+            (uint64_t)table->shape[0] != cols || (uint64_t)next_x->shape[0] != rows || next_x->shape[1] != table->shape[1])
+            return GD_ERR_INVALID_ARGUMENT;
+        if (table->dtype != next_x->dtype || gd_hip_dtype_size(table->dtype) == 0u) return GD_ERR_UNSUPPORTED;
+        row_bytes = (uint64_t)table->shape[1] * gd_hip_dtype_size(table->dtype);
+        if ((row_bytes & 15u) != 0u || row_bytes > 0xffffffffu || ((table->offset | next_x->offset) & 15u) != 0u)
+            return GD_ERR_UNSUPPORTED;
+    }
     return gd_hip_finish_op(backend, gd_hip_launch_argmax_advance(
         backend->stream, gd_hip_view_ptr(logits), (int32_t *)gd_hip_view_ptr(ids), rows, cols,
         logits->dtype == GD_BACKEND_DTYPE_F16, (int32_t *)gd_hip_view_ptr(positions),
         (int32_t *)gd_hip_view_ptr(step_counters), (int32_t *)gd_hip_view_ptr(out_ids),
-        out_gaps != NULL ? (float *)gd_hip_view_ptr(out_gaps) : NULL, (uint32_t)max_steps, pos_delta));
+        out_gaps != NULL ? (float *)gd_hip_view_ptr(out_gaps) : NULL, (uint32_t)max_steps, pos_delta,
+        table != NULL ? gd_hip_view_ptr(table) : NULL, next_x != NULL ? gd_hip_view_ptr(next_x) : NULL, (uint32_t)row_bytes));
 }

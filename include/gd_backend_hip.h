@@ -409,12 +409,15 @@ gd_status gd_backend_fused_qkv_rope_append(gd_backend *backend, const gd_backend
  * feeds its own tokens: ids[b] = greedy token of logits row b; positions[b] += pos_delta;
  * s = step_counters[b]; when s < max_steps (= out_ids count / rows), out_ids[s*B + b] = token and
  * (out_gaps != NULL) out_gaps[s*B + b] = best - runner-up; step_counters[b] = s + 1.  Every row keeps its
- * own counter (I32 [B]) because every row is handled by its own workgroup. */
+ * own counter (I32 [B]) because every row is handled by its own workgroup.  With table [V, Dm] and next_x
+ * [B, Dm] (both or neither; V = logits columns, rows of 16-byte multiples) the token's embedding row is also
+ * copied to next_x[b], which makes the next step's gd_backend_embedding_forward unnecessary. */
 gd_status gd_backend_argmax_advance(gd_backend *backend, const gd_backend_tensor_view *logits,
                                     const gd_backend_tensor_view *ids, const gd_backend_tensor_view *positions,
                                     const gd_backend_tensor_view *step_counters,
                                     const gd_backend_tensor_view *out_ids, const gd_backend_tensor_view *out_gaps,
-                                    int32_t pos_delta);
+                                    int32_t pos_delta, const gd_backend_tensor_view *table,
+                                    const gd_backend_tensor_view *next_x);
 
 /* Device copy between buffers, enqueued like an operator. */
 gd_status gd_backend_copy(gd_backend *backend, gd_backend_buffer *dst, size_t dst_offset,
