@@ -96,6 +96,8 @@ gd_status gd_backend_create_default(gd_backend **out_backend)
     b->sdpa_waves = env_int("GD_HIP_SDPA_WAVES", 0, 4, 8);
     b->sdpa_unroll = env_int("GD_HIP_SDPA_UNROLL", 0, 4, 8);
     b->sdpa_nontemporal = env_int("GD_HIP_SDPA_NONTEMPORAL", 0, 0, 1);
+    b->linear_tiles = env_int("GD_HIP_LINEAR_TILES", 0, 1, 4);
+    b->linear_waves = env_int("GD_HIP_LINEAR_WAVES", 0, 4, 8);
     *out_backend = b;
     return GD_OK;
 }
@@ -141,6 +143,16 @@ gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t 
     if (strcmp(name, "sdpa_nontemporal") == 0) {
         if (value != 0 && value != 1) return GD_ERR_INVALID_ARGUMENT;
         backend->sdpa_nontemporal = (int)value;
+        return GD_OK;
+    }
+    if (strcmp(name, "linear_tiles") == 0) {
+        if (value != 0 && value != 1 && value != 2 && value != 4) return GD_ERR_INVALID_ARGUMENT;
+        backend->linear_tiles = (int)value;
+        return GD_OK;
+    }
+    if (strcmp(name, "linear_waves") == 0) {
+        if (value != 0 && value != 4 && value != 8) return GD_ERR_INVALID_ARGUMENT;
+        backend->linear_waves = (int)value;
         return GD_OK;
     }
     if (strcmp(name, "sdpa_waves") == 0 || strcmp(name, "sdpa_unroll") == 0) {

@@ -27,6 +27,7 @@ typedef struct gd_hip_linear_params {
      * N = 3 * heads * head_dim; see gd_hip_rope_epilogue */
     uint32_t rope_heads, rope_head_dim, rope_tmax;
     float rope_freq_scale;
+    uint32_t force_tiles, force_waves; /* tunables: 0 = automatic */
 } gd_hip_linear_params;
 
 /* destinations of the rope + append epilogue: q [M,H,D]; caches [M,Tmax,H,D]; positions I32 [M] */

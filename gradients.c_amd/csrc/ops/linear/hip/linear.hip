@@ -402,18 +402,30 @@ extern "C" int gd_hip_launch_linear(hipStream_t stream, const void *x, const voi
     } else {
         /* columns per workgroup: 64, 32 or 16 (rows: always 16, further rows in grid.y; their weight re-reads
          * come from L2).  More columns reuse each activation fragment for more MFMAs and repeat the prologue
-         * in fewer workgroups, but leave fewer workgroups; the grid keeps at least one per compute unit. */
+         * in fewer workgroups, but leave fewer workgroups; the grid keeps at least one per compute unit.
+         * Paired modes (swiglu / rope epilogue) need 2 or 4 tiles; rope with 4 tiles needs head_dim % 64 == 0. */
         const uint64_t mt = (p.M + 15u) / 16u;
         const uint32_t target = min_workgroups > 0 ? (uint32_t)min_workgroups / 2u : 256u;
-        if (p.rope_head_dim != 0u) { /* pairs (c, c + head_dim/2): 32 or 16 pairs per workgroup; head_dim % 32 == 0 */
-            if ((p.rope_head_dim % 64u) == 0u && (p.N / 64u) * mt >= target) launch_stream<4, 8>(stream, xp, wp, bp, rp, np, yp, p, rope);
-            else launch_stream<2, 8>(stream, xp, wp, bp, rp, np, yp, p, rope);
-        } else if (p.swiglu_cols != 0u) { /* value and gate tiles side by side: 32 or 16 output columns per workgroup */
-            if (((p.N + 31u) / 32u) * mt >= target) launch_stream<4, 8>(stream, xp, wp, bp, rp, np, yp, p, rope);
-            else launch_stream<2, 8>(stream, xp, wp, bp, rp, np, yp, p, rope);
-        } else if (((p.N + 63u) / 64u) * mt >= target) launch_stream<4, 8>(stream, xp, wp, bp, rp, np, yp, p, rope);
-        else if (((p.N + 31u) / 32u) * mt >= target) launch_stream<2, 8>(stream, xp, wp, bp, rp, np, yp, p, rope);
-        else launch_stream<1, 8>(stream, xp, wp, bp, rp, np, yp, p, rope);
+        const bool paired = p.rope_head_dim != 0u || p.swiglu_cols != 0u;
+        const uint32_t outs = p.rope_head_dim != 0u ? p.N / 2u : p.N; /* columns that count towards the grid */
+        const uint32_t per4 = paired ? 32u : 64u, per2 = paired ? 16u : 32u;
+        uint32_t nt;
+        const uint64_t wgs4 = ((outs + per4 - 1u) / per4) * mt;
+        if (wgs4 >= target || (p.K >= 1024u && wgs4 * 2u >= target && p.rope_head_dim == 0u)) nt = 4u; /* deep K: the repeated prologue weighs more */
+        else if (paired || ((outs + per2 - 1u) / per2) * mt >= target) nt = 2u;
+        else nt = 1u;
+        if (p.force_tiles != 0u && !(paired && p.force_tiles == 1u)) nt = p.force_tiles;
+        if (p.rope_head_dim != 0u && nt == 4u && (p.rope_head_dim % 64u) != 0u) nt = 2u;
+        /* short K: splitting it eight ways leaves a wavefront one or two steps; four wavefronts then */
+        uint32_t waves = (p.K + 31u) / 32u <= 16u ? 4u : 8u;
+        if (p.force_waves != 0u) waves = p.force_waves;
+#define GD_LS(NTV, WV) launch_stream<NTV, WV>(stream, xp, wp, bp, rp, np, yp, p, rope)
+        if (waves == 4u) {
+            if (nt == 4u) GD_LS(4, 4); else if (nt == 2u) GD_LS(2, 4); else GD_LS(1, 4);
+        } else {
+            if (nt == 4u) GD_LS(4, 8); else if (nt == 2u) GD_LS(2, 8); else GD_LS(1, 8);
+        }
+#undef GD_LS
     }
     return (int)hipGetLastError();
 }
