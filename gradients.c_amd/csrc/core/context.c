@@ -153,6 +153,11 @@ gd_status gd_context_create(const gd_memory_config *config, gd_context **out_ctx
         st = arena_init(backend, &ctx->data.slots[i], GD_ARENA_DATA, (int32_t)i, cfg.data_slot_bytes, align);
         if (st == GD_OK) ctx->data.count = i + 1U;
     }
+    if (st == GD_OK) {
+        ctx->pack_count = (size_t)1U << 21; /* 4 MiB per transfer call */
+        ctx->pack = (uint16_t *)heap_alloc(ctx->pack_count * sizeof(uint16_t));
+        if (ctx->pack == NULL) st = GD_ERR_OUT_OF_MEMORY;
+    }
     if (st != GD_OK) {
         gd_context_destroy(ctx);
         return st;
@@ -173,6 +178,7 @@ void gd_context_destroy(gd_context *ctx)
         arena_destroy(&ctx->data.slots[i]);
     }
     if (ctx->backend != NULL) gd_backend_destroy(ctx->backend);
+    free(ctx->pack);
     free(ctx);
 }
 

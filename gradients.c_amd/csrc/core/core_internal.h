@@ -44,6 +44,10 @@ struct gd_context {
     uint64_t scope_count;
     gd_status status;
     char error[160];
+    /* F32 <-> F16 conversion staging of gd_tensor_write_f32 / read_f32, allocated with the context so that
+     * transfers inside a step need no heap */
+    uint16_t *pack;
+    size_t pack_count;
 };
 
 /* reference src/core/memory.c:126-134: latch status + message, return the status */

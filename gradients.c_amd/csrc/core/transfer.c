@@ -136,21 +136,22 @@ static gd_status check_f32(gd_context *ctx, const gd_tensor *t, size_t count)
     return GD_OK;
 }
 
-#define GD_PACK_BLOCK 8192U
 
 gd_status gd_tensor_write_f32(gd_context *ctx, gd_tensor *dst, const float *src, size_t count)
 {
-    uint16_t block[GD_PACK_BLOCK];
+    uint16_t *block;
     size_t done = 0U;
     gd_status st;
     if (ctx == NULL || dst == NULL || src == NULL) return GD_ERR_INVALID_ARGUMENT;
     st = check_f32(ctx, dst, count);
     if (st != GD_OK) return st;
     if (dst->dtype == GD_DTYPE_F32) return gd_tensor_write(ctx, dst, src, count * sizeof(float));
+    block = ctx->pack;
     while (done < count) {
-        const size_t n = count - done < GD_PACK_BLOCK ? count - done : GD_PACK_BLOCK;
-        size_t i;
-        for (i = 0U; i < n; ++i) block[i] = gd_f32_to_f16_bits(src[done + i]);
+        const size_t n = count - done < ctx->pack_count ? count - done : ctx->pack_count;
+        int64_t i;
+#pragma omp parallel for schedule(static) if (n > 65536U)
+        for (i = 0; i < (int64_t)n; ++i) block[i] = gd_f32_to_f16_bits(src[done + (size_t)i]);
         st = gd_backend_upload(gd_context_backend(ctx), (gd_backend_buffer *)dst->storage.buffer,
                                dst->storage.offset + dst->view_offset + done * 2U, block, n * 2U);
         if (st != GD_OK) return gd_context_set_error(ctx, st, "backend upload failed");
@@ -163,15 +164,16 @@ gd_status gd_tensor_write_f32(gd_context *ctx, gd_tensor *dst, const float *src,
 
 gd_status gd_tensor_read_f32(gd_context *ctx, const gd_tensor *src, float *dst, size_t count)
 {
-    uint16_t block[GD_PACK_BLOCK];
+    uint16_t *block;
     size_t done = 0U;
     gd_status st;
     if (ctx == NULL || src == NULL || dst == NULL) return GD_ERR_INVALID_ARGUMENT;
     st = check_f32(ctx, src, count);
     if (st != GD_OK) return st;
     if (src->dtype == GD_DTYPE_F32) return gd_tensor_read(ctx, src, dst, count * sizeof(float));
+    block = ctx->pack;
     while (done < count) {
-        const size_t n = count - done < GD_PACK_BLOCK ? count - done : GD_PACK_BLOCK;
+        const size_t n = count - done < ctx->pack_count ? count - done : ctx->pack_count;
         size_t i;
         st = gd_backend_download(gd_context_backend(ctx), (gd_backend_buffer *)src->storage.buffer,
                                  src->storage.offset + src->view_offset + done * 2U, block, n * 2U);

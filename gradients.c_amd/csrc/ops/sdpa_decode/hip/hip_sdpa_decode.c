@@ -64,7 +64,7 @@ static gd_status dispatch(gd_backend *backend, const gd_backend_tensor_view *q, 
     p.nsplit = 1u;
     p.waves = backend->sdpa_waves == 4 ? 4u : 8u;
     /* measured on MI355X: 8 rows in flight suit 128-byte rows (D = 64), 4 suit 256-byte rows (D = 128) */
-    p.unroll = backend->sdpa_unroll != 0 ? (uint32_t)backend->sdpa_unroll : (p.dh == 64u ? 8u : 4u);
+    p.unroll = backend->sdpa_unroll != 0 ? (uint32_t)backend->sdpa_unroll : 4u; /* 4: every workgroup of a 512-item launch is resident at once */
     p.nontemporal = backend->sdpa_nontemporal != 0 ? 1u : 0u;
     group = p.hq / p.hkv;
     if (q->dtype == GD_BACKEND_DTYPE_F16 && p.tq == 1u && (p.dh == 64u || p.dh == 128u) && p.prefix_len == 0u &&

@@ -70,3 +70,5 @@ def test_product_package_does_not_import_the_oracle():
             if f.endswith((".py", ".c", ".h", ".hip", ".cpp")) or f == "Makefile":
                 text = open(os.path.join(dirpath, f), errors="replace").read()
                 assert "gd_oracle" not in text and "libgd_oracle" not in text and "oracle/" not in text, f
+                # nor the device-less test backend: the product has no CPU path
+                assert "null_backend" not in text and "libgradients_host" not in text and "tests/host" not in text, f
