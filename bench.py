@@ -28,7 +28,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per sdpa_decode launch at this shape from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
 # profiles/sdpa_decode_config2_pmc.md (fetch scaled by the factor a 64 MiB device copy shows in the same run)
-SDPA_TRAFFIC_BYTES = 67316700
+SDPA_TRAFFIC_BYTES = 67327400
 
 
 def _package():
@@ -81,7 +81,7 @@ def sdpa_roofline(dec, D, pkg, iters=200):
     algo_bytes = B * keys * H * Dh * 2 * 2 + 2 * B * H * Dh * 2 + 4 * B
     sec = ms / 1e3 / iters
     gbs = algo_bytes / sec / 1e9
-    return {"bound": "hbm", "kernel": "gd_sdpa_decode_split_kernel<64,1,8,8>", "achieved": round(gbs, 1),
+    return {"bound": "hbm", "kernel": "gd_sdpa_decode_split_kernel<64,1,8,4>", "achieved": round(gbs, 1),
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": SDPA_TRAFFIC_BYTES,
             "algorithmic_bytes_per_launch": algo_bytes, "us_per_launch": round(sec * 1e6, 3), "launches": iters}
 
@@ -175,6 +175,12 @@ def long_context_workload(a, pkg, oracle, D, which):
     prefill_s = time.perf_counter() - t0
     dense_flops = 2.0 * n_tokens * layers * (d_model * 3 * d_model + d_model * d_model + d_model * 2 * hidden + hidden * d_model)
     attn_flops = 4.0 * head_dim * heads * layers * float(np.sum(lens.astype(np.float64) * (lens + 1) / 2))
+    if a.prefill_only:
+        dec.close()
+        print(json.dumps({"prefill_only": f"configs[{which}]", "prompt_tokens": n_tokens, "prefill_seconds": round(prefill_s, 4),
+                          "prefill_tokens_per_s": round(n_tokens / prefill_s, 1),
+                          "prefill_tflops": round((dense_flops + attn_flops) / prefill_s / 1e12, 1)}))
+        return
     steps = a.steps if which == 3 else 128
     total = a.warmup + steps if which == 3 else steps
     t0 = time.perf_counter()
@@ -219,6 +225,8 @@ def main():
     ap.add_argument("--workload", type=int, default=2, choices=(2, 3, 4),
                     help="BASELINE.json configs index: 2 = the headline line (default); 3, 4 = the scaled decoder "
                          "(reported without roofline / cpu_baseline objects)")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="with --workload 3 or 4: stop after the packed prefill (for kernel traces of the prefill kernels)")
     ap.add_argument("--kernel-only", action="store_true",
                     help="only launch sdpa_decode at the benchmark shape plus calibration copies (for --pmc runs)")
     a = ap.parse_args()
