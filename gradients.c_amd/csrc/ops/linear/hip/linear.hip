@@ -373,7 +373,8 @@ static void launch_stream(hipStream_t stream, const gd_half *x, const gd_half *w
 
 extern "C" int gd_hip_launch_linear_tile(hipStream_t stream, const void *x, const void *w, const void *bias,
                                          const void *residual, const void *norm_w, void *y,
-                                         const gd_hip_linear_params *params, int big_tiles, int vector_store);
+                                         const gd_hip_linear_params *params, int big_tiles, int vector_store,
+                                         int compute_units);
 
 /* vector_ok: K % 8 == 0 and every pointer / pitch allows 16-byte fragment loads (for w only when it is [N,K]);
  * kn_vector_ok: w stored [K,N] with N % 8 == 0 and 16-byte aligned rows; store_vector_ok: y (and the residual)
@@ -398,7 +399,7 @@ extern "C" int gd_hip_launch_linear(hipStream_t stream, const void *x, const voi
          * a workgroup, the 128 x 128 tile below that */
         const uint64_t big = (uint64_t)((p.M + 255u) / 256u) * ((p.N + 255u) / 256u);
         const uint32_t units = min_workgroups > 0 ? (uint32_t)min_workgroups / 2u : 256u;
-        return gd_hip_launch_linear_tile(stream, x, w, bias, residual, norm_w, y, params, big >= units, store_vector_ok);
+        return gd_hip_launch_linear_tile(stream, x, w, bias, residual, norm_w, y, params, big >= units, store_vector_ok, (int)units);
     } else {
         /* columns per workgroup: 64, 32 or 16 (rows: always 16, further rows in grid.y; their weight re-reads
          * come from L2).  More columns reuse each activation fragment for more MFMAs and repeat the prologue

@@ -9,36 +9,39 @@
  * wavefront owns (BM/2) x (BN/2) as WM x WN tiles of v_mfma_f32_32x32x16_f16 (4 x 4 tiles = 256
  * accumulator registers per lane for the 256 tile, one wavefront per SIMD).  Every MFMA fragment
  * (row l%32, 8 consecutive k starting at 8*(l/32)) is one 16-byte LDS read; a 4 x 4 wavefront tile reads
- * 8 fragments for 16 MFMAs.
+ * 8 fragments for 16 MFMAs.  The weight fragment is the first MFMA operand, so a lane ends up with four
+ * consecutive output columns of one row per register quad (result layout of a 32x32 tile: lane l holds
+ * activation row l%32; register 4q+r holds weight row 8q + 4*(l/32) + r).
  *
- * Two ways of staging the operand tiles in LDS:
- *  - direct (no prologue, whole tiles, K % 32 == 0): global -> LDS loads that bypass the registers, K in
- *    tiles of 32 through four LDS stages with three tiles in flight; serves both weight layouts (a [K,N]
- *    weight is staged as it lies and transposed by ds_read_b64_tr_b16).  Described at the code.
- *  - through registers (prologues, ragged tiles): K in tiles of 64, two LDS stages; the next tile's global
- *    loads are issued before the matrix instructions of the current one and stored to the other stage
- *    during its last two steps.  Chunk c of row r sits at r*8 + (c ^ (r & 7) ^ ((r >> 3) & 7)): the first
- *    xor makes the fragment reads of 8 neighbouring rows hit 8 different bank groups, the second does the
- *    same for the transposing store of a [K,N] weight (a thread gathers an 8(k) x 8(n) block with eight
- *    16-byte row loads, transposes it in registers and stores eight k-contiguous chunks).
+ * Workgroups are persistent: the grid has one workgroup per compute unit, which walks the output tiles
+ * t, t + grid, ...  The operand loads of the next tile are requested before the epilogue of the current
+ * one, so their latency and the epilogue's stores overlap.
  *
- * What bounds the direct path on MI355X (8192^3, measured by leaving out one side): matrix instructions
- * plus fragment reads alone 1.55 PFLOP/s, operand staging alone (8.6 GB through L2 -> LDS at about
- * 12-13 TB/s, 90 % L2 hits) 1.5 PFLOP/s-equivalent, both together 1.05 PFLOP/s: the two sides are balanced
- * and share the LDS, so neither hides completely behind the other.
+ * K advances in tiles of 64 through two LDS stages.  Two ways of staging:
+ *  - direct (no prologue, whole tiles, K % 64 == 0): global -> LDS loads that bypass the registers, serving
+ *    both weight layouts (a [K,N] weight is staged as it lies and transposed by ds_read_b64_tr_b16).  The
+ *    instruction stream of a K tile is laid out by hand, see the code.
+ *  - through registers (prologues, ragged tiles): the next tile's global loads are issued before the matrix
+ *    instructions of the current one and stored to the other stage during its last two steps.
+ * LDS has 64 banks of 4 bytes on this chip and serves 16 lanes of a 16-byte read at a time; chunk c (16
+ * bytes = 8 k) of row r sits at r*8 + (c ^ swizzle(r)) with swizzles that make any 16 consecutive rows of
+ * one k chunk hit all 64 banks (measured: no bank conflict cycles).
+ *
+ * What bounds it on MI355X: under this load the chip clocks at about 1.55 GHz (counter GRBM_GUI_ACTIVE
+ * against the kernel's duration), which puts the matrix peak at about 1.6 PFLOP/s, 64 % of the published
+ * 2.5 at 2.4 GHz; the vendor library reaches 1.0-1.5 PFLOP/s on the same shapes.
  *
  * Prologues are applied while the activation tile moves from registers to LDS (rounded to F16 there,
  * like the reference's separate kernels): the swiglu gate reads the second half of the row, the
  * rms_norm scale uses per-row factors computed by the workgroup before the main loop.
  *
- * Epilogue.  Accumulators (+ bias, in F32 or after the F16 rounding, by mode) are rounded to F16 into
- * the now idle LDS, then written with 16-byte row-contiguous stores, adding the residual in F16.
+ * Epilogue.  In WM passes of 64 rows: accumulators (+ bias, in F32 or after the F16 rounding, by mode) are
+ * rounded to F16 and written as 8-byte pieces into a separate 64-row LDS buffer, then read back as 16-byte
+ * row pieces and stored, adding the residual in F16.
  *
- * Workgroup order: ids are dealt round-robin to the 8 XCDs, so the id is first remapped to give
- * each XCD a contiguous run of tiles, and runs walk 8 tile rows by column so that the 32 workgroups
+ * Tile order: workgroup ids are dealt round-robin to the 8 XCDs, so the tile index is first remapped to
+ * give each XCD a contiguous run of tiles, and runs walk 8 tile rows by column so that the workgroups
  * resident on one XCD share a few activation and weight panels in its L2.
- *
- * MFMA result layout (32x32 tile): lane l holds column l%32; register 4q+r holds row 8q + 4*(l/32) + r.
  */
 #include "../../_shared/hip_device.h"
 #include "hip_linear_types.h"
@@ -80,40 +83,38 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
     constexpr uint32_t BM = 64u * WM, BN = 64u * WN;
     constexpr int A_PER = BM / 32;                 /* 16-byte chunks of the activation tile per thread */
     constexpr int B_PER = W_NK ? (int)(BN / 32) : 8; /* weight chunks per thread */
+    constexpr uint32_t STAGE_BYTES = 2u * (BM + BN) * 8u * 16u; /* both stages of both operands */
     extern __shared__ __align__(16) unsigned char gd_tile_smem[];
-    __shared__ float s_inv[PRO == GD_HIP_PRO_RMS_NORM ? BM : 1];
     gd_half8 *sA = reinterpret_cast<gd_half8 *>(gd_tile_smem); /* [2][BM*8] */
     gd_half8 *sB = sA + 2u * BM * 8u;                          /* [2][BN*8] */
+    unsigned char *epi = gd_tile_smem + STAGE_BYTES;           /* [64][BN] halfs */
+    float *s_inv = reinterpret_cast<float *>(epi); /* [BM] row factors of rms_norm; live during the main loop only */
 
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint32_t wm = wave >> 1, wn = wave & 1u;
-
-    /* tile of this workgroup */
-    uint32_t pid = blockIdx.x;
     const uint32_t total = tiles_m * tiles_n;
-    if ((total & 7u) == 0u) pid = (pid & 7u) * (total >> 3) + (pid >> 3);
-    const uint32_t width = 8u * tiles_n;
-    const uint32_t first_m = (pid / width) * 8u;
-    const uint32_t gsz = min(tiles_m - first_m, 8u);
-    const uint32_t tile_m = first_m + (pid % width) % gsz;
-    const uint32_t tile_n = (pid % width) / gsz;
-    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+    constexpr bool DIRECT = PRO == GD_HIP_PRO_NONE;
+    uint32_t m0 = 0u, n0 = 0u; /* origin of the current tile */
+    auto locate = [&](uint32_t t, uint32_t &tm0, uint32_t &tn0) __attribute__((always_inline)) {
+        uint32_t pid = t;
+        if ((total & 7u) == 0u) pid = (pid & 7u) * (total >> 3) + (pid >> 3);
+        const uint32_t width = 8u * tiles_n;
+        const uint32_t first_m = (pid / width) * 8u;
+        const uint32_t gsz = min(tiles_m - first_m, 8u);
+        tm0 = (first_m + (pid % width) % gsz) * BM;
+        tn0 = ((pid % width) / gsz) * BN;
+    };
+    auto direct_ok = [&](uint32_t tm0, uint32_t tn0) __attribute__((always_inline)) {
+        return DIRECT && tm0 + BM <= p.M && tn0 + BN <= p.N && (p.K % 64u) == 0u && p.K >= 128u;
+    };
 
-    if (PRO == GD_HIP_PRO_RMS_NORM) {
-        for (uint32_t r = wave; r < BM; r += 4u) {
-            const uint32_t row = min(m0 + r, p.M - 1u);
-            const gd_half *xr = x + (size_t)row * p.ldx;
-            float ss = 0.f;
-            for (uint32_t k = lane * 8u; k < p.K; k += 512u) {
-                const gd_half8 v = *reinterpret_cast<const gd_half8 *>(xr + k);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) ss = fmaf((float)v[e], (float)v[e], ss);
-            }
-            ss = gd_wave_sum(ss);
-            if (lane == 0u) s_inv[r] = rsqrtf(ss / (float)p.K + p.eps);
-        }
-        __syncthreads();
-    }
+    uint32_t tid_opaque = threadIdx.x;
+    bool prefetched = false; /* the first two K tiles of the current output tile are already requested */
+    for (uint32_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+    /* Everything below is derived from the thread id anew for every tile: were it loop-invariant, the
+     * compiler would hoist some hundred addresses and offsets out of the tile loop and spill them. */
+    asm volatile("" : "+v"(tid_opaque));
+    const uint32_t tid = tid_opaque, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t wm = wave >> 1, wn = wave & 1u;
+    locate(tile, m0, n0);
 
     /* staging coordinates */
     const uint32_t a_c = tid & 7u, a_r = tid >> 3; /* activation: chunk a_c of rows a_r + 32*i */
@@ -126,10 +127,6 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
     gd_half8 ra[A_PER], rz[PRO == GD_HIP_PRO_SWIGLU ? A_PER : 1], rb[B_PER], rn;
     const gd_half8 zero8 = (gd_half8)(gd_half)0.f;
     const uint32_t ktiles = (p.K + GD_TILE_BK - 1u) / GD_TILE_BK;
-    /* interior tile: every staged chunk is in range, so the main loop carries no guards (one basic
-     * block, which lets the scheduler interleave memory operations with the matrix instructions) */
-    const bool interior = m0 + BM <= p.M && n0 + BN <= p.N && (p.K % GD_TILE_BK) == 0u;
-    const bool interior_direct = m0 + BM <= p.M && n0 + BN <= p.N && (p.K % 32u) == 0u && p.K >= 96u;
 
     /* ---- staging through registers (any prologue, either weight layout, ragged tiles) ---------------- */
     auto load_tile = [&](uint32_t kt, auto guarded_tag) __attribute__((always_inline)) {
@@ -202,63 +199,59 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
     };
 
     /* ---- staging straight into LDS (plain activation, interior tiles) -----------------------------
-     * Global -> LDS loads that bypass the registers.  What limits this kernel is the round trip of the
-     * operand tiles through the vector memory path (about 64 KB per compute unit and 64 k), so this path
-     * keeps three K tiles in flight: K advances in tiles of 32 (rows of 4 chunks) through 4 LDS stages.
-     * A wavefront-wide 16-byte load writes 64 consecutive chunks = 16 rows of an LDS tile; lane L fills
-     * position L%4 of row L/4 and therefore fetches the global chunk that the swizzle puts there
-     * (chunk c of row r sits at r*4 + (c ^ ((r >> 2) & 3))).  Wavefront w stages rows
-     * [w*BM/4, (w+1)*BM/4) of the activation tile and the same share of the weight tile.
+     * A wavefront-wide 16-byte load writes 64 consecutive chunks = 8 rows of an LDS tile, whole 128-byte
+     * lines per row; lane L fills position L%8 of row L/8 and therefore fetches the global chunk that the
+     * swizzle puts there (chunk c of row r sits at r*8 + (c ^ (r & 7) ^ ((r >> 3) & 1))).  Wavefront w
+     * stages rows [w*BM/4, (w+1)*BM/4) of the activation tile and the same share of the weight tile.
      *
-     * A weight stored [K,N] is staged as it lies: 32 k-rows of BN halfs per stage, a wavefront load
+     * A weight stored [K,N] is staged as it lies: 64 k-rows of BN halfs per stage, a wavefront load
      * filling 1024 / (2*BN) whole rows, with chunk p of k-row r at position p ^ ((r & 3) << 2).  Its
      * fragments come from ds_read_b64_tr_b16, which hands lane i of a 16-lane group element i%4 of the
      * 8-byte words addressed by lanes i/4, i/4 + 4, i/4 + 8, i/4 + 12: lane q + 4e addresses k-row e,
      * columns 4q..4q+3, so lane i receives four consecutive k of column i.  Two such reads (k 0-3, 4-7)
      * make one MFMA operand; the xor spreads the four k-rows of a read over all banks. */
-    constexpr bool DIRECT = PRO == GD_HIP_PRO_NONE;
-    constexpr uint32_t DBK = 32u, DSTAGES = 4u;
-    constexpr int A_DIRECT = BM / 64, B_DIRECT = BN / 64; /* loads per wavefront, K tile and operand */
-    const uint32_t d_off_a = ((lane >> 2) * p.ldx + ((lane & 3u) ^ ((lane >> 4) & 3u)) * 8u) * 2u; /* bytes */
+    constexpr uint32_t DBK = 64u, CH = 8u, RW = 8u; /* K tile, chunks per staged row, rows per wavefront load */
+    constexpr int A_DIRECT = BM / 4 / RW, B_DIRECT = BN / 4 / RW; /* loads per wavefront, K tile and operand */
+    constexpr int PER_TILE = A_DIRECT + B_DIRECT;
+    const uint32_t d_lane_chunk = (lane & 7u) ^ ((lane >> 3) & 7u);
+    /* rows 8..15 of every 16 (odd wavefront loads) use the swizzle with bit 0 flipped */
+    const uint32_t d_off_a = ((lane >> 3) * p.ldx + d_lane_chunk * 8u) * 2u; /* bytes */
+    const uint32_t d_off_a1 = ((lane >> 3) * p.ldx + (d_lane_chunk ^ 1u) * 8u) * 2u;
     constexpr uint32_t CPR = BN / 8u, RPL = 64u / CPR; /* [K,N] stage: chunks per k-row, k-rows per wavefront load */
-    const uint32_t d_off_b = W_NK ? ((lane >> 2) * p.ldw + ((lane & 3u) ^ ((lane >> 4) & 3u)) * 8u) * 2u
-                                  : ((lane / CPR) * p.ldw) * 2u;
-    gd_half8 *dA = reinterpret_cast<gd_half8 *>(gd_tile_smem); /* [4][BM*4] */
-    gd_half8 *dB = dA + DSTAGES * BM * 4u;                     /* [4][BN*4] */
+    const uint32_t d_off_b = W_NK ? ((lane >> 3) * p.ldw + d_lane_chunk * 8u) * 2u : ((lane / CPR) * p.ldw) * 2u;
+    const uint32_t d_off_b1 = ((lane >> 3) * p.ldw + (d_lane_chunk ^ 1u) * 8u) * 2u;
+    gd_half8 *dA = reinterpret_cast<gd_half8 *>(gd_tile_smem); /* [2][BM*8] */
+    gd_half8 *dB = dA + 2u * BM * CH;                          /* [2][BN*8] */
     const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)gd_tile_smem;
-    auto direct_loads = [&](uint32_t kt) __attribute__((always_inline)) {
-        const uint32_t stage = kt & (DSTAGES - 1u);
-#pragma unroll
-        for (int t = 0; t < A_DIRECT; ++t) {
-            const uint32_t row0 = wave_u * (BM / 4u) + (uint32_t)t * 16u;
-            gd_tile_load_lds16(x + (size_t)(m0 + row0) * p.ldx + kt * DBK, d_off_a,
-                               lds_base + (stage * BM * 4u + row0 * 4u) * 16u);
+    /* item t < A_DIRECT: a wavefront load of the activation tile; A_DIRECT <= t: one of the weight tile */
+    auto direct_load_item = [&](uint32_t tm0, uint32_t tn0, uint32_t kt, uint32_t t) __attribute__((always_inline)) {
+        const uint32_t stage = kt & 1u;
+        if (t < (uint32_t)A_DIRECT) {
+            const uint32_t row0 = wave_u * (BM / 4u) + t * RW;
+            gd_tile_load_lds16(x + (size_t)(tm0 + row0) * p.ldx + kt * DBK, (t & 1u) ? d_off_a1 : d_off_a,
+                               lds_base + (stage * BM * CH + row0 * CH) * 16u);
+        } else if (W_NK) {
+            const uint32_t tb = t - (uint32_t)A_DIRECT;
+            const uint32_t row0 = wave_u * (BN / 4u) + tb * RW;
+            gd_tile_load_lds16(w + (size_t)(tn0 + row0) * p.ldw + kt * DBK, (tb & 1u) ? d_off_b1 : d_off_b,
+                               lds_base + ((2u * BM + stage * BN) * CH + row0 * CH) * 16u);
+        } else {
+            /* k-rows kr0 .. kr0+RPL-1 of the tile; lane L fills position L%CPR of row kr0 + L/CPR */
+            const uint32_t tb = t - (uint32_t)A_DIRECT;
+            const uint32_t kr0 = (wave_u * (uint32_t)B_DIRECT + tb) * RPL;
+            const uint32_t row = (RPL >= 4u ? 0u : ((tb * RPL) & 3u)) + lane / CPR; /* row & 3 */
+            const uint32_t chunk = (lane % CPR) ^ ((row & 3u) << 2);
+            gd_tile_load_lds16(w + (size_t)(kt * DBK + kr0) * p.ldw + tn0, d_off_b + chunk * 16u,
+                               lds_base + ((2u * BM + stage * BN) * CH + kr0 * CPR) * 16u);
         }
+    };
+    auto direct_loads = [&](uint32_t tm0, uint32_t tn0, uint32_t kt) __attribute__((always_inline)) {
 #pragma unroll
-        for (int t = 0; t < B_DIRECT; ++t) {
-            if (W_NK) {
-                const uint32_t row0 = wave_u * (BN / 4u) + (uint32_t)t * 16u;
-                gd_tile_load_lds16(w + (size_t)(n0 + row0) * p.ldw + kt * DBK, d_off_b,
-                                   lds_base + ((DSTAGES * BM + stage * BN) * 4u + row0 * 4u) * 16u);
-            } else {
-                /* k-rows kr0 .. kr0+RPL-1 of the tile; lane L fills position L%CPR of row kr0 + L/CPR */
-                const uint32_t kr0 = (wave_u * (uint32_t)B_DIRECT + (uint32_t)t) * RPL;
-                const uint32_t row = (RPL >= 4u ? 0u : (((uint32_t)t * RPL) & 3u)) + lane / CPR; /* row & 3 */
-                const uint32_t chunk = (lane % CPR) ^ ((row & 3u) << 2);
-                gd_tile_load_lds16(w + (size_t)(kt * DBK + kr0) * p.ldw + n0, d_off_b + chunk * 16u,
-                                   lds_base + ((DSTAGES * BM + stage * BN) * 4u + kr0 * CPR) * 16u);
-            }
-        }
+        for (uint32_t t = 0; t < (uint32_t)PER_TILE; ++t) direct_load_item(tm0, tn0, kt, t);
     };
 
     gd_float16 acc[WM][WN];
-#pragma unroll
-    for (int i = 0; i < WM; ++i)
-#pragma unroll
-        for (int j = 0; j < WN; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
     const uint32_t frag_row = lane & 31u, frag_c = lane >> 5;
     const uint32_t a_frag_row = wm * (WM * 32u) + frag_row, b_frag_row = wn * (WN * 32u) + frag_row;
@@ -275,12 +268,12 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
         for (int i = 0; i < WM; ++i)
 #pragma unroll
             for (int j = 0; j < WN; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
     };
 
     constexpr uint32_t STEPS = GD_TILE_BK / 16u;
-    /* One K tile, 4 steps of 16: the fragments of step s+1 are read while the matrix cores work on step s.
-     * Register path: the next tile's global loads are issued first and stored to the other LDS stage
+    /* Register path, one K tile of 4 steps of 16: the fragments of step s+1 are read while the matrix cores
+     * work on step s; the next tile's global loads are issued first and stored to the other LDS stage
      * during the last two steps. */
     auto k_tile_regs = [&](uint32_t kt, auto guarded_tag, auto more_tag) __attribute__((always_inline)) {
         constexpr bool MORE = decltype(more_tag)::value;
@@ -303,146 +296,269 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
         }
         __syncthreads();
     };
-    /* Direct path, K tile kt of 32 (2 steps of 16) in stage kt % 4.  On entry the loads of tiles kt .. kt+2
-     * are in flight; the wait leaves the newer ones outstanding, the barrier makes every wavefront's share
-     * of tile kt visible and proves that stage (kt+3) % 4, read during tile kt-1, is free again. */
-    auto direct_frags = [&](const gd_half8 *cA, const gd_half8 *cB, uint32_t ks, gd_half8 (&fa)[WM], gd_half8 (&fb)[WN])
-        __attribute__((always_inline)) {
+
+    auto direct_frag_a = [&](const gd_half8 *cA, uint32_t ks, uint32_t i) __attribute__((always_inline)) {
         const uint32_t c = ks * 2u + frag_c;
-#pragma unroll
-        for (int i = 0; i < WM; ++i) {
-            const uint32_t r = a_frag_row + i * 32u;
-            fa[i] = cA[r * 4u + (c ^ ((r >> 2) & 3u))];
-        }
-#pragma unroll
-        for (int j = 0; j < WN; ++j) {
-            if (W_NK) {
-                const uint32_t r = b_frag_row + j * 32u;
-                fb[j] = cB[r * 4u + (c ^ ((r >> 2) & 3u))];
-            } else {
-                /* lane l = 16g + (q + 4e): k-rows ks*16 + 8*(g/2) + e (+4 for the second read), columns
-                 * 16*(g%2) + 4q .. +3 of this 32-column block */
-                const uint32_t g = lane >> 4, q = lane & 3u, e = (lane >> 2) & 3u;
-                const uint32_t col = wn * (WN * 32u) + (uint32_t)j * 32u + 16u * (g & 1u) + 4u * q;
-                const uint32_t krow = ks * 16u + 8u * (g >> 1) + e; /* krow & 3 == e for both reads */
-                const uint32_t byte0 = krow * (BN * 2u) + (((col >> 3) ^ (e << 2)) << 4) + (q & 1u) * 8u;
-                const unsigned char *base = reinterpret_cast<const unsigned char *>(cB);
-                typedef short gd_short4 __attribute__((ext_vector_type(4)));
-                const gd_short4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (__attribute__((address_space(3))) gd_short4 *)(base + byte0));
-                const gd_short4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (__attribute__((address_space(3))) gd_short4 *)(base + byte0 + 4u * (BN * 2u)));
-                union { gd_short4 s[2]; gd_half8 h; } u;
-                u.s[0] = lo;
-                u.s[1] = hi;
-                fb[j] = u.h;
-            }
+        const uint32_t r = a_frag_row + i * 32u;
+        return cA[r * CH + (c ^ (r & 7u) ^ ((r >> 3) & 1u))];
+    };
+    auto direct_frag_b = [&](const gd_half8 *cB, uint32_t ks, uint32_t j) __attribute__((always_inline)) {
+        if (W_NK) {
+            const uint32_t c = ks * 2u + frag_c;
+            const uint32_t r = b_frag_row + j * 32u;
+            return cB[r * CH + (c ^ (r & 7u) ^ ((r >> 3) & 1u))];
+        } else {
+            /* lane l = 16g + (q + 4e): k-rows ks*16 + 8*(g/2) + e (+4 for the second read), columns
+             * 16*(g%2) + 4q .. +3 of this 32-column block */
+            const uint32_t g = lane >> 4, q = lane & 3u, e = (lane >> 2) & 3u;
+            const uint32_t col = wn * (WN * 32u) + j * 32u + 16u * (g & 1u) + 4u * q;
+            const uint32_t krow = ks * 16u + 8u * (g >> 1) + e; /* krow & 3 == e for both reads */
+            const uint32_t byte0 = krow * (BN * 2u) + (((col >> 3) ^ (e << 2)) << 4) + (q & 1u) * 8u;
+            const unsigned char *base = reinterpret_cast<const unsigned char *>(cB);
+            typedef short gd_short4 __attribute__((ext_vector_type(4)));
+            const gd_short4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) gd_short4 *)(base + byte0));
+            const gd_short4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) gd_short4 *)(base + byte0 + 4u * (BN * 2u)));
+            union { gd_short4 s[2]; gd_half8 h; } u;
+            u.s[0] = lo;
+            u.s[1] = hi;
+            return u.h;
         }
     };
-    auto k_tile_direct = [&](uint32_t kt, auto newer_tag) __attribute__((always_inline)) {
-        constexpr int TAG = decltype(newer_tag)::value; /* 2: steady state (requests tile kt+3); 3, 1, 0: tail */
-        constexpr int NEWER = TAG == 3 ? 2 : TAG;          /* tiles requested after kt that may stay in flight */
-        constexpr int PER_TILE = A_DIRECT + B_DIRECT;
-        /* s_waitcnt vmcnt(NEWER * PER_TILE), other counters unconstrained */
-        constexpr int VM = NEWER * PER_TILE;
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (VM & 15) | ((VM >> 4) << 14));
-        __syncthreads();
-        if (TAG == 2) direct_loads(kt + 3u);
-        const uint32_t stage = kt & (DSTAGES - 1u);
-        const gd_half8 *cA = dA + stage * BM * 4u, *cB = dB + stage * BN * 4u;
-        gd_half8 fa[2][WM], fb[2][WN];
-        direct_frags(cA, cB, 0u, fa[0], fb[0]);
-        direct_frags(cA, cB, 1u, fa[1], fb[1]);
-        multiply(fa[0], fb[0]);
-        multiply(fa[1], fb[1]);
+    /* Direct path, one wavefront's instruction stream for a K tile (4 steps of 16 matrix instructions),
+     * pinned with scheduling barriers: every matrix instruction is followed by at most one fragment read or
+     * one global -> LDS load, so the matrix pipe never waits for an LDS round trip.
+     *   steps 0-2 of tile kt: their first matrix instructions are followed by the fragment reads of the next
+     *   step (into the other register set);
+     *   step 3: wait for this wavefront's loads of tile kt+1, barrier (tile kt+1 visible to all, stage kt%2
+     *           read by all), then read step 0 of tile kt+1 and, behind the later matrix instructions,
+     *           request the first half of tile kt+2 into the freed stage; step 0 of the next tile requests
+     *           the second half.
+     * TAIL 0: steady state; 1: tile kt+1 exists but not kt+2; 2: last tile. */
+    gd_half8 qa[2][WM], qb[2][WN];
+    constexpr uint32_t NM = WM * WN, NR = WM + WN, NL = PER_TILE / 2;
+    constexpr uint32_t RPM = NM >= 2u * NR ? 1u : (2u * NR + NM - 1u) / NM; /* fragment reads per matrix instruction */
+    constexpr uint32_t LPM = NM >= 2u * NL ? 1u : (2u * NL + NM - 1u) / NM; /* loads per matrix instruction */
+    auto direct_step = [&](uint32_t kt, auto ks_tag, auto tail_tag) __attribute__((always_inline)) {
+        constexpr uint32_t KS = decltype(ks_tag)::value;
+        constexpr int TAIL = decltype(tail_tag)::value;
+        constexpr uint32_t CUR = KS & 1u, NXT = CUR ^ 1u;
+        constexpr bool READS = KS < 3u || TAIL < 2;
+        constexpr bool LOADS = (KS == 3u && TAIL == 0) || (KS == 0u && TAIL < 2);
+        const uint32_t rstage = KS < 3u ? (kt & 1u) : ((kt + 1u) & 1u);
+        const gd_half8 *cA = dA + rstage * BM * CH, *cB = dB + rstage * BN * CH;
+        const uint32_t rks = KS < 3u ? KS + 1u : 0u;
+        const bool loads_on = KS == 3u || kt >= 1u; /* tiles 0 and 1 are requested before the loop */
+        if (KS == 3u && TAIL < 2) {
+            __builtin_amdgcn_s_waitcnt(0x0070); /* vmcnt(0) lgkmcnt(0) */
+            __syncthreads();
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (uint32_t idx = 0; idx < NM; ++idx) {
+            const uint32_t i = idx / WN, j = idx % WN;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qb[CUR][j], qa[CUR][i], acc[i][j], 0, 0, 0);
+            if (READS) {
+#pragma unroll
+                for (uint32_t r = min(idx * RPM, NR); r < min((idx + 1u) * RPM, NR); ++r) {
+                    /* a0 b0 a1 b1 ...: the order in which the next step consumes them */
+                    if ((r & 1u) == 0u) qa[NXT][r >> 1] = direct_frag_a(cA, rks, r >> 1);
+                    else qb[NXT][r >> 1] = direct_frag_b(cB, rks, r >> 1);
+                }
+            }
+            if (LOADS && loads_on && idx >= NM - NL / LPM) {
+#pragma unroll
+                for (uint32_t t = (idx - (NM - NL / LPM)) * LPM; t < (idx - (NM - NL / LPM) + 1u) * LPM; ++t)
+                    direct_load_item(m0, n0, KS == 3u ? kt + 2u : kt + 1u, KS == 3u ? t : NL + t);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto k_tile_direct = [&](uint32_t kt, auto tail_tag) __attribute__((always_inline)) {
+        direct_step(kt, std::integral_constant<uint32_t, 0>{}, tail_tag);
+        direct_step(kt, std::integral_constant<uint32_t, 1>{}, tail_tag);
+        direct_step(kt, std::integral_constant<uint32_t, 2>{}, tail_tag);
+        direct_step(kt, std::integral_constant<uint32_t, 3>{}, tail_tag);
     };
     using gd_t = std::true_type;
     using gd_f = std::false_type;
 
-    if (DIRECT && interior_direct) {
-        const uint32_t dtiles = p.K / DBK; /* >= 3 */
-        direct_loads(0u);
-        direct_loads(1u);
-        direct_loads(2u);
-        uint32_t kt = 0;
-        for (; kt + 3u < dtiles; ++kt) k_tile_direct(kt, std::integral_constant<int, 2>{});
-        /* the last three tiles request nothing new; the newer loads are 2, 1, 0 tiles' worth */
-        k_tile_direct(kt, std::integral_constant<int, 3>{});
-        k_tile_direct(kt + 1u, std::integral_constant<int, 1>{});
-        k_tile_direct(kt + 2u, std::integral_constant<int, 0>{});
-        __syncthreads(); /* every wavefront has read its fragments before the epilogue reuses the LDS */
-    } else {
-        load_tile(0u, gd_t{});
-        store_tile(0u);
-        __syncthreads();
-        if (interior) {
-            for (uint32_t kt = 0; kt + 1u < ktiles; ++kt) k_tile_regs(kt, gd_f{}, gd_t{});
-            k_tile_regs(ktiles - 1u, gd_f{}, gd_f{});
-        } else {
-            for (uint32_t kt = 0; kt + 1u < ktiles; ++kt) k_tile_regs(kt, gd_t{}, gd_t{});
-            k_tile_regs(ktiles - 1u, gd_t{}, gd_f{});
-        }
-    }
-
-    /* epilogue: bias and F16 rounding in registers, then through LDS for row-contiguous stores */
-    gd_half *sC = reinterpret_cast<gd_half *>(gd_tile_smem); /* [BM][BN] halfs = the staging buffers' size */
-    auto round_tiles = [&](auto mode_tag) __attribute__((always_inline)) {
-        constexpr uint32_t MODE = decltype(mode_tag)::value;
+    /* 8-byte pieces of the epilogue buffer: piece u of row e sits at e*EU + (u ^ (e & 31)), which spreads the
+     * 32 rows that one wavefront store touches over all banks; a 16-byte read-back takes pieces 2v, 2v+1 */
+    constexpr uint32_t EU = BN / 4u;
+    typedef _Float16 gd_half4 __attribute__((ext_vector_type(4)));
+    gd_half4 bq[WN][4]; /* bias of the 4 columns of every register quad, loaded once per tile */
+    auto load_bias = [&]() __attribute__((always_inline)) {
+        const bool vec = (reinterpret_cast<uintptr_t>(bias) & 7u) == 0u;
 #pragma unroll
         for (int j = 0; j < WN; ++j) {
-            const uint32_t lc = b_frag_row + j * 32u;
-            const gd_half bh = MODE != GD_HIP_EPI_NONE ? bias[min(n0 + lc, p.N - 1u)] : (gd_half)0.f;
 #pragma unroll
-            for (int i = 0; i < WM; ++i) {
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t gc = n0 + wn * (WN * 32u) + (uint32_t)j * 32u + 8u * (uint32_t)q + 4u * frag_c;
+                if (vec && gc + 4u <= p.N) {
+                    bq[j][q] = *reinterpret_cast<const gd_half4 *>(bias + gc);
+                } else {
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const uint32_t lr = wm * (WM * 32u) + i * 32u + 8u * (e >> 2) + 4u * frag_c + (e & 3);
-                    const float v = acc[i][j][e];
-                    gd_half h;
-                    if (MODE == GD_HIP_EPI_BIAS_F32) h = (gd_half)(v + (float)bh);
-                    else if (MODE == GD_HIP_EPI_BIAS_F16) h = (gd_half)v + bh;
-                    else h = (gd_half)v;
-                    sC[lr * BN + lc] = h;
+                    for (int r = 0; r < 4; ++r) bq[j][q][r] = bias[min(gc + (uint32_t)r, p.N - 1u)];
                 }
             }
         }
     };
-    if (p.epilogue == GD_HIP_EPI_BIAS_F32) round_tiles(std::integral_constant<uint32_t, GD_HIP_EPI_BIAS_F32>{});
-    else if (p.epilogue == GD_HIP_EPI_BIAS_F16) round_tiles(std::integral_constant<uint32_t, GD_HIP_EPI_BIAS_F16>{});
-    else round_tiles(std::integral_constant<uint32_t, GD_HIP_EPI_NONE>{});
-    __syncthreads();
-    constexpr uint32_t CHUNKS = BM * BN / 8u;
-    for (uint32_t idx = tid; idx < CHUNKS; idx += 256u) {
-        const uint32_t lr = idx / (BN / 8u), lc = (idx % (BN / 8u)) * 8u;
-        const uint32_t gr = m0 + lr, gc = n0 + lc;
-        if (gr >= p.M || gc >= p.N) continue;
-        gd_half8 h = *reinterpret_cast<const gd_half8 *>(sC + lr * BN + lc);
-        gd_half *yr = y + (size_t)gr * p.ldy + gc;
-        if (vector_store && gc + 8u <= p.N) {
-            if (p.has_residual) {
-                const gd_half8 r = *reinterpret_cast<const gd_half8 *>(residual + (size_t)gr * p.ldr + gc);
+    auto epilogue_pass = [&](auto pass_tag, auto mode_tag) __attribute__((always_inline)) {
+        constexpr int I = decltype(pass_tag)::value;
+        constexpr uint32_t MODE = decltype(mode_tag)::value;
+        const uint32_t e = wm * 32u + frag_row;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) h[e] = r[e] + h[e];
-            }
-            *reinterpret_cast<gd_half8 *>(yr) = h;
-        } else {
-            for (uint32_t e = 0; e < 8u && gc + e < p.N; ++e) {
-                gd_half v = h[e];
-                if (p.has_residual) v = residual[(size_t)gr * p.ldr + gc + e] + v;
-                yr[e] = v;
+        for (int j = 0; j < WN; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t lc = wn * (WN * 32u) + (uint32_t)j * 32u + 8u * (uint32_t)q + 4u * frag_c;
+                gd_half4 h;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float v = acc[I][j][4 * q + r];
+                    if (MODE == GD_HIP_EPI_NONE) h[r] = (gd_half)v;
+                    else if (MODE == GD_HIP_EPI_BIAS_F32) h[r] = (gd_half)(v + (float)bq[j][q][r]);
+                    else h[r] = (gd_half)v + bq[j][q][r];
+                }
+                *reinterpret_cast<gd_half4 *>(epi + (e * EU + ((lc >> 2) ^ (e & 31u))) * 8u) = h;
             }
         }
+        __syncthreads();
+        constexpr uint32_t CPRW = BN / 8u; /* 16-byte chunks per row */
+#pragma unroll
+        for (uint32_t idx0 = 0; idx0 < 64u * CPRW; idx0 += 256u) {
+            const uint32_t idx = idx0 + tid;
+            const uint32_t er = idx / CPRW, v = idx % CPRW;
+            const uint32_t gr = m0 + (er >> 5) * (WM * 32u) + (uint32_t)I * 32u + (er & 31u), gc = n0 + v * 8u;
+            if (gr >= p.M || gc >= p.N) continue;
+            const uint32_t xr = er & 31u;
+            const gd_half8 raw = *reinterpret_cast<const gd_half8 *>(epi + (er * EU + 2u * (v ^ (xr >> 1))) * 8u);
+            gd_half8 h = raw;
+            if (xr & 1u) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    h[t] = raw[4 + t];
+                    h[4 + t] = raw[t];
+                }
+            }
+            gd_half *yr = y + (size_t)gr * p.ldy + gc;
+            if (vector_store && gc + 8u <= p.N) {
+                if (p.has_residual) {
+                    const gd_half8 r = *reinterpret_cast<const gd_half8 *>(residual + (size_t)gr * p.ldr + gc);
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) h[t] = r[t] + h[t];
+                }
+                *reinterpret_cast<gd_half8 *>(yr) = h;
+            } else {
+                for (uint32_t t = 0; t < 8u && gc + t < p.N; ++t) {
+                    gd_half v1 = h[t];
+                    if (p.has_residual) v1 = residual[(size_t)gr * p.ldr + gc + t] + v1;
+                    yr[t] = v1;
+                }
+            }
+        }
+        if (I + 1 < WM) __syncthreads(); /* the next pass overwrites the buffer; after the last pass the barriers
+                                            of the next tile's main loop come first */
+    };
+    auto epilogue = [&](auto mode_tag) __attribute__((always_inline)) {
+        if (decltype(mode_tag)::value != GD_HIP_EPI_NONE) load_bias();
+        epilogue_pass(std::integral_constant<int, 0>{}, mode_tag);
+        epilogue_pass(std::integral_constant<int, 1>{}, mode_tag);
+        if (WM > 2) {
+            epilogue_pass(std::integral_constant<int, (WM > 2 ? 2 : 0)>{}, mode_tag);
+            epilogue_pass(std::integral_constant<int, (WM > 2 ? 3 : 0)>{}, mode_tag);
+        }
+    };
+
+        /* interior tile: every staged chunk is in range, so the main loop carries no guards */
+        const bool interior = m0 + BM <= p.M && n0 + BN <= p.N && (p.K % GD_TILE_BK) == 0u;
+
+        if (PRO == GD_HIP_PRO_RMS_NORM) {
+            __syncthreads(); /* the previous tile's epilogue has left the buffer that holds the row factors */
+            for (uint32_t r = wave; r < BM; r += 4u) {
+                const uint32_t row = min(m0 + r, p.M - 1u);
+                const gd_half *xr = x + (size_t)row * p.ldx;
+                float ss = 0.f;
+                for (uint32_t k = lane * 8u; k < p.K; k += 512u) {
+                    const gd_half8 v = *reinterpret_cast<const gd_half8 *>(xr + k);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) ss = fmaf((float)v[e], (float)v[e], ss);
+                }
+                ss = gd_wave_sum(ss);
+                if (lane == 0u) s_inv[r] = rsqrtf(ss / (float)p.K + p.eps);
+            }
+            __syncthreads();
+        }
+
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+            for (int j = 0; j < WN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+        if (direct_ok(m0, n0)) {
+            const uint32_t dtiles = p.K / 64u; /* >= 2 */
+            if (!prefetched) {
+                direct_loads(m0, n0, 0u);
+                direct_loads(m0, n0, 1u);
+            }
+            /* at most PER_TILE vector memory operations outstanding: loads complete in order, so K tile 0 has
+             * landed whatever else (K tile 1, stores of the previous epilogue) is still on its way */
+            __builtin_amdgcn_s_waitcnt(0x0F70 | (PER_TILE & 15) | ((PER_TILE >> 4) << 14));
+            __syncthreads();
+            {
+#pragma unroll
+                for (int i = 0; i < WM; ++i) qa[0][i] = direct_frag_a(dA, 0u, (uint32_t)i);
+#pragma unroll
+                for (int j = 0; j < WN; ++j) qb[0][j] = direct_frag_b(dB, 0u, (uint32_t)j);
+            }
+            uint32_t kt = 0;
+            for (; kt + 2u < dtiles; ++kt) k_tile_direct(kt, std::integral_constant<int, 0>{});
+            k_tile_direct(kt, std::integral_constant<int, 1>{});
+            k_tile_direct(kt + 1u, std::integral_constant<int, 2>{});
+            __syncthreads(); /* every wavefront has read its last fragments: both stages are free */
+            /* request the next output tile's first two K tiles now; they land during the epilogue */
+            prefetched = false;
+            const uint32_t next = tile + gridDim.x;
+            if (next < total) {
+                uint32_t nm0, nn0;
+                locate(next, nm0, nn0);
+                if (direct_ok(nm0, nn0)) {
+                    direct_loads(nm0, nn0, 0u);
+                    direct_loads(nm0, nn0, 1u);
+                    prefetched = true;
+                }
+            }
+        } else {
+            prefetched = false;
+            load_tile(0u, gd_t{});
+            store_tile(0u);
+            __syncthreads();
+            if (interior) {
+                for (uint32_t kt = 0; kt + 1u < ktiles; ++kt) k_tile_regs(kt, gd_f{}, gd_t{});
+                k_tile_regs(ktiles - 1u, gd_f{}, gd_f{});
+            } else {
+                for (uint32_t kt = 0; kt + 1u < ktiles; ++kt) k_tile_regs(kt, gd_t{}, gd_t{});
+                k_tile_regs(ktiles - 1u, gd_t{}, gd_f{});
+            }
+        }
+
+        if (p.epilogue == GD_HIP_EPI_BIAS_F32) epilogue(std::integral_constant<uint32_t, GD_HIP_EPI_BIAS_F32>{});
+        else if (p.epilogue == GD_HIP_EPI_BIAS_F16) epilogue(std::integral_constant<uint32_t, GD_HIP_EPI_BIAS_F16>{});
+        else epilogue(std::integral_constant<uint32_t, GD_HIP_EPI_NONE>{});
     }
 }
 
 template <int WM, int WN, bool W_NK, int PRO>
 static int launch_tile_one(hipStream_t stream, const gd_half *x, const gd_half *w, const gd_half *bias,
                            const gd_half *residual, const gd_half *norm_w, gd_half *y, const gd_hip_linear_params &p,
-                           uint32_t vector_store)
+                           uint32_t vector_store, uint32_t workgroups)
 {
     constexpr uint32_t BM = 64u * WM, BN = 64u * WN;
-    constexpr size_t lds = (size_t)2u * (BM + BN) * 8u * 16u;
-    static_assert(lds >= (size_t)BM * BN * 2u, "the epilogue reuses the staging buffers");
+    constexpr size_t lds = (size_t)2u * (BM + BN) * 8u * 16u + (size_t)64u * BN * 2u; /* stages + epilogue rows */
     static bool configured = false;
     auto kernel = gd_linear_tile_kernel<WM, WN, W_NK, PRO>;
     if (!configured) {
@@ -452,16 +568,18 @@ static int launch_tile_one(hipStream_t stream, const gd_half *x, const gd_half *
         configured = true;
     }
     const uint32_t tiles_m = (p.M + BM - 1u) / BM, tiles_n = (p.N + BN - 1u) / BN;
-    kernel<<<tiles_m * tiles_n, 256, lds, stream>>>(x, w, bias, residual, norm_w, y, p, tiles_m, tiles_n, vector_store);
+    /* persistent workgroups: at most `workgroups` of them (a multiple of 8 keeps the tile -> XCD relation) */
+    const uint32_t grid = tiles_m * tiles_n < workgroups ? tiles_m * tiles_n : workgroups;
+    kernel<<<grid, 256, lds, stream>>>(x, w, bias, residual, norm_w, y, p, tiles_m, tiles_n, vector_store);
     return (int)hipGetLastError();
 }
 
 template <int WM, int WN>
 static int launch_tile(hipStream_t stream, const gd_half *x, const gd_half *w, const gd_half *bias,
                        const gd_half *residual, const gd_half *norm_w, gd_half *y, const gd_hip_linear_params &p,
-                       uint32_t vector_store)
+                       uint32_t vector_store, uint32_t workgroups)
 {
-#define GD_GO(NK, PRO) return launch_tile_one<WM, WN, NK, PRO>(stream, x, w, bias, residual, norm_w, y, p, vector_store)
+#define GD_GO(NK, PRO) return launch_tile_one<WM, WN, NK, PRO>(stream, x, w, bias, residual, norm_w, y, p, vector_store, workgroups)
     if (p.w_is_nk) {
         if (p.prologue == GD_HIP_PRO_SWIGLU) GD_GO(true, GD_HIP_PRO_SWIGLU);
         if (p.prologue == GD_HIP_PRO_RMS_NORM) GD_GO(true, GD_HIP_PRO_RMS_NORM);
@@ -474,15 +592,18 @@ static int launch_tile(hipStream_t stream, const gd_half *x, const gd_half *w, c
 }
 
 /* Requires: K % 8 == 0, 16-byte aligned x rows (and gate half), w rows (for [K,N]: N % 8 == 0 too) and
- * norm weight; M >= 1.  big_tiles: use the 256 x 256 tile. */
+ * norm weight; M >= 1.  big_tiles: use the 256 x 256 tile (one workgroup per compute unit; the 128 x 128 tile
+ * fits two). */
 extern "C" int gd_hip_launch_linear_tile(hipStream_t stream, const void *x, const void *w, const void *bias,
                                          const void *residual, const void *norm_w, void *y,
-                                         const gd_hip_linear_params *params, int big_tiles, int vector_store)
+                                         const gd_hip_linear_params *params, int big_tiles, int vector_store,
+                                         int compute_units)
 {
     const gd_hip_linear_params &p = *params;
+    const uint32_t units = ((uint32_t)(compute_units > 0 ? compute_units : 256) + 7u) & ~7u;
     if (big_tiles)
         return launch_tile<4, 4>(stream, (const gd_half *)x, (const gd_half *)w, (const gd_half *)bias,
-                                 (const gd_half *)residual, (const gd_half *)norm_w, (gd_half *)y, p, (uint32_t)vector_store);
+                                 (const gd_half *)residual, (const gd_half *)norm_w, (gd_half *)y, p, (uint32_t)vector_store, units);
     return launch_tile<2, 2>(stream, (const gd_half *)x, (const gd_half *)w, (const gd_half *)bias,
-                             (const gd_half *)residual, (const gd_half *)norm_w, (gd_half *)y, p, (uint32_t)vector_store);
+                             (const gd_half *)residual, (const gd_half *)norm_w, (gd_half *)y, p, (uint32_t)vector_store, 2u * units);
 }
