@@ -81,7 +81,7 @@ def sdpa_roofline(dec, D, pkg, iters=200):
     algo_bytes = B * keys * H * Dh * 2 * 2 + 2 * B * H * Dh * 2 + 4 * B
     sec = ms / 1e3 / iters
     gbs = algo_bytes / sec / 1e9
-    return {"bound": "hbm", "kernel": "gd_sdpa_decode_split_kernel<64,1,8,4>", "achieved": round(gbs, 1),
+    return {"bound": "hbm", "kernel": "gd_sdpa_decode_split_kernel<64,1,4,2>", "achieved": round(gbs, 1),
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": SDPA_TRAFFIC_BYTES,
             "algorithmic_bytes_per_launch": algo_bytes, "us_per_launch": round(sec * 1e6, 3), "launches": iters}
 

@@ -94,7 +94,7 @@ gd_status gd_backend_create_default(gd_backend **out_backend)
     b->host_visible_buffers = hv != NULL && hv[0] == '1' && hv[1] == '\0';
     b->sdpa_chunk = env_int("GD_HIP_SDPA_CHUNK", 0, 32, 1 << 20);
     b->sdpa_waves = env_int("GD_HIP_SDPA_WAVES", 0, 4, 8);
-    b->sdpa_unroll = env_int("GD_HIP_SDPA_UNROLL", 0, 4, 8);
+    b->sdpa_unroll = env_int("GD_HIP_SDPA_UNROLL", 0, 2, 8);
     b->sdpa_nontemporal = env_int("GD_HIP_SDPA_NONTEMPORAL", 0, 0, 1);
     b->linear_tiles = env_int("GD_HIP_LINEAR_TILES", 0, 1, 4);
     b->linear_waves = env_int("GD_HIP_LINEAR_WAVES", 0, 4, 8);
@@ -156,7 +156,7 @@ gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t 
         return GD_OK;
     }
     if (strcmp(name, "sdpa_waves") == 0 || strcmp(name, "sdpa_unroll") == 0) {
-        if (value != 0 && value != 4 && value != 8) return GD_ERR_INVALID_ARGUMENT;
+        if (value != 0 && value != 4 && value != 8 && !(value == 2 && name[5] == 'u')) return GD_ERR_INVALID_ARGUMENT;
         if (name[5] == 'w') backend->sdpa_waves = (int)value;
         else backend->sdpa_unroll = (int)value;
         return GD_OK;

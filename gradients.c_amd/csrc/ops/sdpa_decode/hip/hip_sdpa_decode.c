@@ -62,14 +62,18 @@ static gd_status dispatch(gd_backend *backend, const gd_backend_tensor_view *q, 
     p.dtype = q->dtype;
     p.chunk = 0u;
     p.nsplit = 1u;
-    p.waves = backend->sdpa_waves == 4 ? 4u : 8u;
-    /* measured on MI355X: 8 rows in flight suit 128-byte rows (D = 64), 4 suit 256-byte rows (D = 128) */
-    p.unroll = backend->sdpa_unroll != 0 ? (uint32_t)backend->sdpa_unroll : 4u; /* 4: every workgroup of a 512-item launch is resident at once */
+    /* measured on MI355X (512 keys, 64 rows x 8 heads): 4 wavefronts with trips of 2 row loads beat 8 wavefronts
+     * with trips of 4 by 7 %: what is left to do when the last rows arrive is one short trip and a merge of 4 */
+    p.waves = backend->sdpa_waves == 8 ? 8u : 4u;
+    p.unroll = backend->sdpa_unroll != 0 ? (uint32_t)backend->sdpa_unroll : 2u;
     p.nontemporal = backend->sdpa_nontemporal != 0 ? 1u : 0u;
     group = p.hq / p.hkv;
     if (q->dtype == GD_BACKEND_DTYPE_F16 && p.tq == 1u && (p.dh == 64u || p.dh == 128u) && p.prefix_len == 0u &&
         (group == 1u || group == 2u || group == 4u || group == 8u) &&
-        ((q->offset | k->offset | v->offset | out->offset) & 15u) == 0u && p.batch <= 65535u) {
+        ((q->offset | k->offset | v->offset | out->offset) & 15u) == 0u && p.batch <= 65535u &&
+        /* the kernel addresses the rows of one (batch row, kv head) with 24-bit factors and 32-bit byte offsets */
+        p.tmax < (1u << 24) && (uint64_t)p.hkv * p.dh * 2u < (1u << 24) &&
+        (uint64_t)p.tmax * p.hkv * p.dh * 2u < 0xffffffffull) {
         /* longest key range a row can have */
         uint32_t span = p.window > 0u && p.window < p.tmax ? p.window : p.tmax;
         uint32_t chunk = (uint32_t)backend->sdpa_chunk;

@@ -76,6 +76,33 @@ __device__ __forceinline__ float gd_row_group_sum(float x)
     return x;
 }
 
+/* Reductions over the 64 / N row slots of a wavefront: lanes i, i + N, i + 2N, ... (N = 8 or 16) are combined
+ * and every lane receives the result.  Distance 8: rotation by 8 inside the 16-lane row (DPP).  Distances 16
+ * and 32: v_permlane16_swap / v_permlane32_swap on two copies of the value, which leave one copy holding the
+ * even (lower) partner's value in both places and the other the odd (upper) partner's. */
+template <int N, typename OP>
+__device__ __forceinline__ float gd_slot_reduce(float x, OP op)
+{
+    typedef unsigned gd_uint2 __attribute__((ext_vector_type(2)));
+    if (N == 8) x = op(x, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x128, 0xf, 0xf, false)));
+    gd_uint2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = op(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return op(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+template <int N>
+__device__ __forceinline__ float gd_slot_sum(float x)
+{
+    return gd_slot_reduce<N>(x, [](float a, float b) { return a + b; });
+}
+
+template <int N>
+__device__ __forceinline__ float gd_slot_max(float x)
+{
+    return gd_slot_reduce<N>(x, [](float a, float b) { return fmaxf(a, b); });
+}
+
 template <int D, int G, int WAVES, int UNROLL, bool NT>
 __global__ void __launch_bounds__(WAVES * 64)
 gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__restrict__ kc,
@@ -85,8 +112,13 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
     constexpr int LPK = D / 8;      /* lanes per key row */
     constexpr int KPW = 64 / LPK;   /* key rows per wavefront load */
     constexpr int KPB = KPW * WAVES;
+    /* Every kernel argument this path reads is requested from the argument segment here, in one batch with
+     * one wait.  Left to the compiler, each load sits in front of its first use behind the early exits, and
+     * a wavefront goes through five dependent round trips before its first K/V load. */
+    asm volatile("" ::"s"(q), "s"(kc), "s"(vc), "s"(pos_ptr), "s"(out), "s"(ws), "s"(p.tmax), "s"(p.hq), "s"(p.hkv),
+                 "s"(p.window), "s"(p.pos_mode), "s"(p.cache_pos), "s"(p.scale), "s"(p.chunk), "s"(p.nsplit));
     const int split = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int slot = lane / LPK, sub = lane % LPK;
 
     const int pos = gd_decode_pos(pos_ptr, p, b);
@@ -110,6 +142,47 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
         return;
     }
 
+    /* Addresses: one scalar base per cache for this (batch row, kv head), plus a 32-bit byte offset per lane
+     * made by one 24-bit multiply-add (the host checks that tmax, the row pitch and their product fit).  The
+     * four wavefronts of a SIMD start together and share its issue slots, so every vector instruction in
+     * front of the first row loads delays all of them. */
+    const uint32_t pitch = p.hkv * (uint32_t)(D * 2); /* bytes between consecutive keys */
+    const size_t slab = ((size_t)b * p.tmax * p.hkv + (size_t)hkv) * (size_t)(D * 2);
+    const unsigned char *kslab = reinterpret_cast<const unsigned char *>(kc) + slab;
+    const unsigned char *vslab = reinterpret_cast<const unsigned char *>(vc) + slab;
+    const uint32_t lane_off = (uint32_t)sub * 16u;
+
+    /* Row loads of trip t+1 are issued before the arithmetic of trip t (two register buffers), so
+     * the memory pipe stays busy while the wavefront computes.  All K rows of a trip are requested before
+     * its V rows: the scores need every K row, the accumulation takes the V rows one by one.  s0: the
+     * wavefront's first row of the trip (scalar); rows past the range re-read the last row and are masked
+     * in the arithmetic. */
+    auto load_trip = [&](gd_half8 (&kv)[UNROLL], gd_half8 (&vv)[UNROLL], int s0) __attribute__((always_inline)) {
+        uint32_t off[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+            off[u] = __umul24((uint32_t)min(s0 + u * KPB + slot, r1 - 1), pitch) + lane_off;
+        /* every cache row is read exactly once per launch: optionally mark the loads streaming */
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const gd_half8 *kp = reinterpret_cast<const gd_half8 *>(kslab + off[u]);
+            kv[u] = NT ? __builtin_nontemporal_load(kp) : *kp;
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const gd_half8 *vp = reinterpret_cast<const gd_half8 *>(vslab + off[u]);
+            vv[u] = NT ? __builtin_nontemporal_load(vp) : *vp;
+        }
+    };
+
+    constexpr int STEP = KPB * UNROLL;
+    /* trips are decided per wavefront (scalar branches), rows past the range are masked per lane */
+    const int jw = r0 + wave * KPW;
+    const bool any_rows = jw < r1;
+    gd_half8 kA[UNROLL], vA[UNROLL], kB[UNROLL], vB[UNROLL];
+    if (any_rows) load_trip(kA, vA, jw);
+    __builtin_amdgcn_sched_barrier(0); /* nothing below moves in front of the first loads */
+
     /* query rows of the G heads that share this kv head stay in F16: products of two halfs are
      * exact in F32, so v_dot2_f32_f16 loses nothing; the softmax scale (exp2 domain) is applied
      * to the reduced dot product */
@@ -131,26 +204,8 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
         for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
     }
 
-    const size_t row_stride = (size_t)p.hkv * D; /* elements between consecutive keys */
-    const gd_half *kbase = kc + ((size_t)b * p.tmax * p.hkv + hkv) * D + sub * 8;
-    const gd_half *vbase = vc + ((size_t)b * p.tmax * p.hkv + hkv) * D + sub * 8;
-
-    /* Row loads of trip t+1 are issued before the arithmetic of trip t (two register buffers), so
-     * the memory pipe stays busy while the wavefront computes. */
-    auto load_trip = [&](gd_half8 (&kv)[UNROLL], gd_half8 (&vv)[UNROLL], bool (&ok)[UNROLL], int j0) {
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const int j = j0 + u * KPB;
-            ok[u] = j < r1;
-            const int jj = ok[u] ? j : (r1 - 1);
-            const gd_half8 *kp = reinterpret_cast<const gd_half8 *>(kbase + (size_t)jj * row_stride);
-            const gd_half8 *vp = reinterpret_cast<const gd_half8 *>(vbase + (size_t)jj * row_stride);
-            /* every cache row is read exactly once per launch: optionally mark the loads streaming */
-            kv[u] = NT ? __builtin_nontemporal_load(kp) : *kp;
-            vv[u] = NT ? __builtin_nontemporal_load(vp) : *vp;
-        }
-    };
-    auto compute_trip = [&](const gd_half8 (&kv)[UNROLL], const gd_half8 (&vv)[UNROLL], const bool (&ok)[UNROLL]) {
+    auto compute_trip = [&](const gd_half8 (&kv)[UNROLL], const gd_half8 (&vv)[UNROLL], int s0)
+        __attribute__((always_inline)) {
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             /* scores of the UNROLL rows, then one rescale of the running state for all of them */
@@ -163,10 +218,13 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
                 for (int e = 0; e < 4; ++e)
                     d = __builtin_amdgcn_fdot2(qh[g][e], (gd_half2){kv[u][2 * e], kv[u][2 * e + 1]}, d, false);
                 d = gd_row_group_sum<LPK>(d);
-                sc[u] = ok[u] ? d * qscale : GD_NEG_INF;
+                sc[u] = (s0 + u * KPB + slot < r1) ? d * qscale : GD_NEG_INF;
                 mt = fmaxf(mt, sc[u]);
             }
-            const float mn = fmaxf(m[g], mt); /* finite: the first row of a trip is always live */
+            /* a lane whose rows of this and all earlier trips lie past the range has mt = m = -inf: the
+             * reference point 0 then makes every factor below exp2(-inf) = 0 instead of exp2(nan) */
+            const float mx = fmaxf(m[g], mt);
+            const float mn = mx == GD_NEG_INF ? 0.f : mx;
             const float corr = exp2f(m[g] - mn); /* exp2(-inf) = 0 on the first trip */
             float lsum = l[g] * corr;
 #pragma unroll
@@ -179,48 +237,46 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
                 for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(pr, (float)vv[u][e], acc[g][e]);
             }
             l[g] = lsum;
-            m[g] = mn;
+            m[g] = mx;
         }
     };
 
-    constexpr int STEP = KPB * UNROLL;
-    int ja = r0 + wave * KPW + slot;
-    if (ja < r1) {
-        gd_half8 kA[UNROLL], vA[UNROLL], kB[UNROLL], vB[UNROLL];
-        bool okA[UNROLL], okB[UNROLL];
-        load_trip(kA, vA, okA, ja);
+    if (any_rows) {
+        int sa = jw; /* first row of the wavefront's trip, the same in every lane */
+        /* The arithmetic of a trip is written once per branch on purpose: where the two paths (a further trip
+         * was requested / was not) meet in front of shared code, the compiler has to wait for ALL outstanding
+         * loads there, and every wavefront would start computing only after its last row has arrived. */
         while (true) {
-            const int jb = ja + STEP;
-            const bool has_b = jb < r1;
-            if (has_b) load_trip(kB, vB, okB, jb);
-            compute_trip(kA, vA, okA);
-            if (!has_b) break;
-            ja = jb + STEP;
-            const bool has_a = ja < r1;
-            if (has_a) load_trip(kA, vA, okA, ja);
-            compute_trip(kB, vB, okB);
-            if (!has_a) break;
+            const int sb = sa + STEP;
+            if (sb < r1) {
+                load_trip(kB, vB, sb);
+                compute_trip(kA, vA, sa);
+            } else {
+                compute_trip(kA, vA, sa);
+                break;
+            }
+            sa = sb + STEP;
+            if (sa < r1) {
+                load_trip(kA, vA, sa);
+                compute_trip(kB, vB, sb);
+            } else {
+                compute_trip(kB, vB, sb);
+                break;
+            }
         }
     }
 
-    /* merge the KPW row slots of the wavefront */
+    /* merge the KPW row slots of the wavefront: common maximum first, one rescale, then plain sums; every
+     * lane of the wavefront ends up with the totals.  Exchanges stay in the vector unit: a rotation inside
+     * the 16-lane row (distance 8) and the row / half swaps of gfx950 (distances 16 and 32). */
 #pragma unroll
     for (int g = 0; g < G; ++g) {
+        const float mw = gd_slot_max<LPK>(m[g]);
+        const float c = (m[g] == GD_NEG_INF) ? 0.f : exp2f(m[g] - mw);
+        l[g] = gd_slot_sum<LPK>(l[g] * c);
 #pragma unroll
-        for (int off = LPK; off < 64; off <<= 1) {
-            const float mo = __shfl_xor(m[g], off, 64);
-            const float lo = __shfl_xor(l[g], off, 64);
-            const float mn = fmaxf(m[g], mo);
-            const float c1 = (m[g] == GD_NEG_INF) ? 0.f : exp2f(m[g] - mn);
-            const float c2 = (mo == GD_NEG_INF) ? 0.f : exp2f(mo - mn);
-            l[g] = l[g] * c1 + lo * c2;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float ao = __shfl_xor(acc[g][e], off, 64);
-                acc[g][e] = acc[g][e] * c1 + ao * c2;
-            }
-            m[g] = mn;
-        }
+        for (int e = 0; e < 8; ++e) acc[g][e] = gd_slot_sum<LPK>(acc[g][e] * c);
+        m[g] = mw;
     }
 
     /* merge the wavefronts through LDS */
@@ -371,8 +427,10 @@ static int launch_split(hipStream_t stream, const void *q, const void *k, const 
     } while (0)
     if constexpr (G == 1) {
         if (p.waves == 8u && p.unroll == 8u) GD_GO(8, 8);
+        else if (p.waves == 8u && p.unroll == 2u) GD_GO(8, 2);
         else if (p.waves == 8u) GD_GO(8, 4);
         else if (p.unroll == 8u) GD_GO(4, 8);
+        else if (p.unroll == 2u) GD_GO(4, 2);
         else GD_GO(4, 4);
     } else {
         GD_GO(4, 4);

@@ -446,8 +446,8 @@ gd_status gd_backend_device_info(const gd_backend *backend, char *name, size_t n
 
 /* Kernel tunables, normally left at 0 = automatic.  name "sdpa_chunk": keys per workgroup of
  * the split-KV decode kernel (also read once from the environment variable
- * GD_HIP_SDPA_CHUNK); "sdpa_waves" (4 or 8 wavefronts per workgroup) and "sdpa_unroll" (4 or 8
- * key-row loads in flight per lane) of the same kernel.  "linear_tiles" (1, 2 or 4 column tiles of 16
+ * GD_HIP_SDPA_CHUNK); "sdpa_waves" (4 or 8 wavefronts per workgroup) and "sdpa_unroll" (2, 4 or 8
+ * key-row loads per lane and trip) of the same kernel.  "linear_tiles" (1, 2 or 4 column tiles of 16
  * per workgroup) and "linear_waves" (4 or 8 wavefronts sharing the K range) of the few-row projection
  * kernel (environment: GD_HIP_LINEAR_TILES, GD_HIP_LINEAR_WAVES).  Unknown name -> GD_ERR_INVALID_ARGUMENT. */
 gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t value);
