@@ -55,7 +55,12 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
     __shared__ float s_part[WAVES][16];
     /* w stored [K,N]: a 32(k) x COLS(n) tile per wavefront, turned by the transposing LDS read */
     __shared__ __align__(16) gd_half s_tr[W_NK ? 1 : WAVES][W_NK ? 8 : 32 * COLS];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    /* every kernel argument the kernel reads, requested in one batch with one wait (left alone, the compiler puts
+     * each load in front of its first use, one dependent round trip after the other) */
+    asm volatile("" ::"s"(x), "s"(w), "s"(bias), "s"(residual), "s"(norm_w), "s"(y), "s"(p.M), "s"(p.N), "s"(p.K),
+                 "s"(p.ldx), "s"(p.ldw), "s"(p.ldy), "s"(p.epilogue), "s"(p.has_residual), "s"(p.ldr), "s"(p.eps),
+                 "s"(p.swiglu_cols), "s"(p.rope_head_dim), "s"(n_tiles));
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int li = lane & 15, lg = lane >> 4;
     /* XCD-aware tile order: workgroup ids are dealt round-robin to the 8 XCDs, so give each XCD a
      * contiguous run of column tiles (neighbouring tiles share weight cache lines when w is [K,N]) */
@@ -86,11 +91,51 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
     const gd_half8 zero8 = (gd_half8)(gd_half)0.f;
     const gd_half *xrow = x + (size_t)mrow * p.ldx;
 
+    /* Fast path (whole steps of 32, byte offsets that fit 32 bits, all columns of a [K,N] tile in range): the
+     * loads carry no guards and take a scalar base that advances with the step plus one per-lane offset computed
+     * once, so a register set is requested by a run of load instructions with nothing in between.  The four to
+     * eight wavefronts of a workgroup share the issue slots of their SIMDs: what sits in front of the first loads
+     * is paid by every one of them before the memory round trip even starts. */
+    const bool off32 = (W_NK ? (uint64_t)(p.N + pair_offset) * p.ldw : (uint64_t)p.K * p.ldw) < 0x7fffffffull &&
+                       (uint64_t)p.M * p.ldx + 2u * (uint64_t)p.K < 0x7fffffffull;
+    const bool fast = (p.K & 31u) == 0u && off32 && (W_NK || n0 + COLS <= p.N);
+    const unsigned char *wb = reinterpret_cast<const unsigned char *>(w);
+    const unsigned char *xb = reinterpret_cast<const unsigned char *>(x);
+    const unsigned char *nb = reinterpret_cast<const unsigned char *>(norm_w);
+    uint32_t woff[NT]; /* bytes from w to the lane's fragment of step 0 */
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        if (W_NK) {
+            const uint32_t n = (gated && j >= NT / 2)
+                                   ? pair_offset + min(n0 + 16u * (uint32_t)(j - NT / 2) + (uint32_t)li, p.N - 1u)
+                                   : min(n0 + 16u * (uint32_t)j + (uint32_t)li, p.N - 1u);
+            woff[j] = (n * p.ldw + (uint32_t)lg * 8u) * 2u;
+        } else {
+            woff[j] = (((uint32_t)j * (32u / NT) + (uint32_t)lane / (2u * NT)) * p.ldw + n0 + ((uint32_t)lane % (2u * NT)) * 8u) * 2u;
+        }
+    }
+    const uint32_t xoff = (mrow * p.ldx + (uint32_t)lg * 8u) * 2u;
+    const uint32_t wstep = W_NK ? 64u : 64u * p.ldw; /* bytes per step of 32 k */
+
     /* requests the operands of steps s0 .. s0+U-1 into register set `set` */
-    auto load_set = [&](auto set_tag, uint32_t s0) __attribute__((always_inline)) {
+    auto load_set_impl = [&](auto set_tag, auto full_tag, uint32_t s0) __attribute__((always_inline)) {
         constexpr int set = decltype(set_tag)::value;
+        constexpr bool FULL = decltype(full_tag)::value;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
+            if (FULL) {
+                const unsigned char *ws = wb + (size_t)(s0 + u) * wstep;
+#pragma unroll
+                for (int j = 0; j < NT; ++j) bf[set][u][j] = *reinterpret_cast<const gd_half8 *>(ws + woff[j]);
+                if (!RES) {
+                    const unsigned char *xs = xb + (size_t)(s0 + u) * 64u;
+                    af[set][u] = *reinterpret_cast<const gd_half8 *>(xs + xoff);
+                    if (PRO == GD_HIP_PRO_SWIGLU) zf[set][u] = *reinterpret_cast<const gd_half8 *>(xs + (size_t)p.K * 2u + xoff);
+                    if (PRO == GD_HIP_PRO_RMS_NORM)
+                        nf[set][u] = *reinterpret_cast<const gd_half8 *>(nb + (size_t)(s0 + u) * 64u + (uint32_t)lg * 16u);
+                }
+                continue;
+            }
             const bool sok = (s0 + u) < s_end;
             const uint32_t k = (s0 + u) * 32u + lg * 8u; /* K % 8 == 0: a fragment is all-valid or all-out */
             const bool kok = sok && k < p.K;
@@ -117,6 +162,10 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
                 if (PRO == GD_HIP_PRO_RMS_NORM) nf[set][u] = kok ? *reinterpret_cast<const gd_half8 *>(norm_w + k) : zero8;
             }
         }
+    };
+    auto load_set = [&](auto set_tag, uint32_t s0) __attribute__((always_inline)) {
+        if (fast && s0 + (uint32_t)U <= s_end) load_set_impl(set_tag, std::true_type{}, s0);
+        else load_set_impl(set_tag, std::false_type{}, s0);
     };
 
     gd_float4 acc[NT];
@@ -173,13 +222,25 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
         /* the wavefront's whole activation slice (at most RES_STEPS steps): one batch of loads, and the row's sum of
          * squares comes from these registers instead of a second pass over x */
         float ss = 0.f;
+        if (fast && s_begin + (uint32_t)RES_STEPS <= s_end) {
 #pragma unroll
-        for (int r = 0; r < RES_STEPS; ++r) {
-            const uint32_t k = (s_begin + r) * 32u + lg * 8u;
-            const bool kok = (s_begin + r) < s_end && k < p.K;
-            ar[r] = kok ? *reinterpret_cast<const gd_half8 *>(xrow + k) : zero8;
-            if (PRO == GD_HIP_PRO_RMS_NORM) nr[r] = kok ? *reinterpret_cast<const gd_half8 *>(norm_w + k) : zero8;
+            for (int r = 0; r < RES_STEPS; ++r) {
+                ar[r] = *reinterpret_cast<const gd_half8 *>(xb + (size_t)(s_begin + r) * 64u + xoff);
+                if (PRO == GD_HIP_PRO_RMS_NORM)
+                    nr[r] = *reinterpret_cast<const gd_half8 *>(nb + (size_t)(s_begin + r) * 64u + (uint32_t)lg * 16u);
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < RES_STEPS; ++r) {
+                const uint32_t k = (s_begin + r) * 32u + lg * 8u;
+                const bool kok = (s_begin + r) < s_end && k < p.K;
+                ar[r] = kok ? *reinterpret_cast<const gd_half8 *>(xrow + k) : zero8;
+                if (PRO == GD_HIP_PRO_RMS_NORM) nr[r] = kok ? *reinterpret_cast<const gd_half8 *>(norm_w + k) : zero8;
+            }
         }
+        /* the second register set is requested here too: behind the barrier of the row norms its round trip would
+         * start only when the first one has ended */
+        load_set(gd_s1{}, s_begin + U);
         if (PRO == GD_HIP_PRO_RMS_NORM) {
 #pragma unroll
             for (int r = 0; r < RES_STEPS; ++r)
@@ -215,7 +276,6 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
     /* two register sets alternate: the next U steps are in flight while the current ones are multiplied */
     if (RES) {
         /* at most RES_STEPS steps: fully unrolled so that the resident fragments are indexed statically */
-        load_set(gd_s1{}, s_begin + U);
         compute_set(gd_s0{}, std::integral_constant<int, 0>{});
         if (2 * U < RES_STEPS) {
             load_set(gd_s0{}, s_begin + 2u * U);
