@@ -247,6 +247,28 @@ static gd_status linear_forward(gd_context *ctx, const gpt_linear *l, const gd_t
     return gd_linear(ctx, x, &l->weight, &l->bias, out);
 }
 
+static gd_status fused_project_rows(gd_gpt_decoder *d, int64_t B, const gd_tensor *x, int64_t x_cols,
+                                    const gpt_linear *lin, const gd_tensor *w_override, const gd_tensor *bias,
+                                    const gd_tensor *residual, const gd_tensor *norm_w, uint32_t prologue,
+                                    uint32_t epilogue, int64_t n_out, gd_tensor *y);
+
+/* attention input -> block output of the packed prefill: the two residual additions ride in the epilogues of the
+ * projections in front of them (same F16 rounding points as the separate gd_add), everything else as block_tail */
+static gd_status block_tail_prefill(gd_gpt_decoder *d, const gpt_block *b, const gd_tensor *residual,
+                                    const gd_tensor *attn_flat, gd_tensor *out)
+{
+    gd_context *ctx = d->ctx;
+    const int64_t rows = attn_flat->shape[0], Dm = d->cfg.d_model, Hm = d->cfg.mlp_hidden;
+    gd_tensor attn_resid, mlp_normed, up_gate, gated;
+    TRY(fused_project_rows(d, rows, attn_flat, Dm, &b->attn_proj, NULL, &b->attn_proj.bias, residual, NULL, 0U, 0U, Dm,
+                           &attn_resid));
+    TRY(gd_rms_norm(ctx, &attn_resid, &b->mlp_norm_w, d->cfg.rms_eps, &mlp_normed));
+    TRY(linear_forward(ctx, &b->up_gate, &mlp_normed, &up_gate));
+    TRY(gd_swiglu_split(ctx, &up_gate, &gated));
+    return fused_project_rows(d, rows, &gated, Hm, &b->down_proj, NULL, &b->down_proj.bias, &attn_resid, NULL, 0U, 0U,
+                              Dm, out);
+}
+
 /* attention input -> block output, shared by decode and prefill (reference :1052-1070, 941-958) */
 static gd_status block_tail(gd_gpt_decoder *d, const gpt_block *b, const gd_tensor *residual, const gd_tensor *attn_flat,
                             gd_tensor *out)
@@ -300,6 +322,7 @@ static gd_status block_prefill(gd_gpt_decoder *d, int32_t l, const gd_tensor *x,
     TRY(gd_kv_cache_append_packed(ctx, &d->k_cache[l], &d->v_cache[l], cache_positions, cu, &k, &v));
     TRY(gd_sdpa_varlen(ctx, &q, &k, &v, cu, &sdpa, &attn));
     TRY(gd_reshape(ctx, &attn, gd_shape_make(2U, flat_shape), &attn_flat));
+    if (x->shape[0] >= 128) return block_tail_prefill(d, b, x, &attn_flat, out);
     return block_tail(d, b, x, &attn_flat, out);
 }
 
@@ -466,15 +489,15 @@ static gd_status scratch_f16(gd_context *ctx, int64_t rows, int64_t cols, gd_ten
 }
 
 /* y = [residual +] bias_mode(prologue(x) @ w) through gd_backend_fused_linear */
-static gd_status fused_project(gd_gpt_decoder *d, const gd_tensor *x, int64_t x_cols, const gpt_linear *lin,
-                               const gd_tensor *w_override, const gd_tensor *bias, const gd_tensor *residual,
-                               const gd_tensor *norm_w, uint32_t prologue, uint32_t epilogue, int64_t n_out, gd_tensor *y)
+static gd_status fused_project_rows(gd_gpt_decoder *d, int64_t B, const gd_tensor *x, int64_t x_cols,
+                                    const gpt_linear *lin, const gd_tensor *w_override, const gd_tensor *bias,
+                                    const gd_tensor *residual, const gd_tensor *norm_w, uint32_t prologue,
+                                    uint32_t epilogue, int64_t n_out, gd_tensor *y)
 {
     gd_backend_matrix_view xm, wm, rm, ym;
     gd_backend_vector_view bv, nv;
     gd_backend_fused_linear_args a;
     const gd_tensor *w = w_override != NULL ? w_override : &lin->weight;
-    const int64_t B = d->cfg.batch;
     gd_status st;
     TRY(scratch_f16(d->ctx, B, n_out, y));
     mview(x, B, x_cols, &xm);
@@ -491,6 +514,14 @@ static gd_status fused_project(gd_gpt_decoder *d, const gd_tensor *x, int64_t x_
     st = gd_backend_fused_linear(gd_context_backend(d->ctx), &xm, &wm, &bv, residual != NULL ? &rm : NULL,
                                  norm_w != NULL ? &nv : NULL, &ym, &a);
     return st;
+}
+
+static gd_status fused_project(gd_gpt_decoder *d, const gd_tensor *x, int64_t x_cols, const gpt_linear *lin,
+                               const gd_tensor *w_override, const gd_tensor *bias, const gd_tensor *residual,
+                               const gd_tensor *norm_w, uint32_t prologue, uint32_t epilogue, int64_t n_out, gd_tensor *y)
+{
+    return fused_project_rows(d, d->cfg.batch, x, x_cols, lin, w_override, bias, residual, norm_w, prologue, epilogue,
+                              n_out, y);
 }
 
 /* The decode step with the fused backend entry points: same operators, same rounding points as
