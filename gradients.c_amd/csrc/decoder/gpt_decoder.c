@@ -263,8 +263,14 @@ static gd_status block_tail_prefill(gd_gpt_decoder *d, const gpt_block *b, const
     TRY(fused_project_rows(d, rows, attn_flat, Dm, &b->attn_proj, NULL, &b->attn_proj.bias, residual, NULL, 0U, 0U, Dm,
                            &attn_resid));
     TRY(gd_rms_norm(ctx, &attn_resid, &b->mlp_norm_w, d->cfg.rms_eps, &mlp_normed));
-    TRY(linear_forward(ctx, &b->up_gate, &mlp_normed, &up_gate));
-    TRY(gd_swiglu_split(ctx, &up_gate, &gated));
+    if (b->up_gate.transposed && (Dm % 8) == 0) {
+        /* swiglu in the epilogue of the up/gate projection: the [rows, 2H] intermediate is never written */
+        TRY(fused_project_rows(d, rows, &mlp_normed, Dm, &b->up_gate, NULL, &b->up_gate.bias, NULL, NULL, 0U, 1U, Hm,
+                               &gated));
+    } else {
+        TRY(linear_forward(ctx, &b->up_gate, &mlp_normed, &up_gate));
+        TRY(gd_swiglu_split(ctx, &up_gate, &gated));
+    }
     return fused_project_rows(d, rows, &gated, Hm, &b->down_proj, NULL, &b->down_proj.bias, &attn_resid, NULL, 0U, 0U,
                               Dm, out);
 }

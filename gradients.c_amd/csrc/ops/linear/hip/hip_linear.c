@@ -34,11 +34,10 @@ static gd_status project_full(gd_backend *backend, const gd_backend_matrix_view 
         K = x->cols;
     }
     if (gated) {
-        /* swiglu epilogue: w [2H,K], bias [2H], y [M,H]; only the few-row kernel implements it */
+        /* swiglu epilogue: w [2H,K], bias [2H], y [M,H] */
         if (!w_is_nk || residual != NULL) return GD_ERR_UNSUPPORTED;
         if (w->cols != K || (w->rows & 1u) != 0u || w->rows / 2u != y->cols || (bias != NULL && bias->length != w->rows))
             return GD_ERR_INVALID_ARGUMENT;
-        if (y->rows >= 128u) return GD_ERR_UNSUPPORTED;
     } else if (w_is_nk ? (w->cols != K || w->rows != y->cols) : (w->rows != K || w->cols != y->cols)) {
         return GD_ERR_INVALID_ARGUMENT;
     }

@@ -454,10 +454,11 @@ extern "C" int gd_hip_launch_linear(hipStream_t stream, const void *x, const voi
     if (!vector_ok || p.K == 0 || (!p.w_is_nk && !kn_vector_ok)) {
         const uint64_t total = (uint64_t)p.M * p.N;
         gd_linear_scalar_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(xp, wp, bp, rp, np, yp, p);
-    } else if (p.M >= 128u && (p.w_is_nk || kn_vector_ok) && p.swiglu_cols == 0u && p.rope_head_dim == 0u) {
+    } else if (p.M >= 128u && (p.w_is_nk || kn_vector_ok) && p.rope_head_dim == 0u) {
         /* matrix-core bound: LDS-tiled kernel; the 256 x 256 tile once it still gives every compute unit
          * a workgroup, the 128 x 128 tile below that */
-        const uint64_t big = (uint64_t)((p.M + 255u) / 256u) * ((p.N + 255u) / 256u);
+        const uint32_t out_cols = p.swiglu_cols != 0u ? 128u : 256u; /* output columns of a 256-wide weight tile */
+        const uint64_t big = (uint64_t)((p.M + 255u) / 256u) * ((p.N + out_cols - 1u) / out_cols);
         const uint32_t units = min_workgroups > 0 ? (uint32_t)min_workgroups / 2u : 256u;
         return gd_hip_launch_linear_tile(stream, x, w, bias, residual, norm_w, y, params, big >= units, store_vector_ok, (int)units);
     } else {

@@ -92,7 +92,17 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
 
     const uint32_t total = tiles_m * tiles_n;
     constexpr bool DIRECT = PRO == GD_HIP_PRO_NONE;
-    uint32_t m0 = 0u, n0 = 0u; /* origin of the current tile */
+    uint32_t m0 = 0u, n0 = 0u; /* origin of the current tile (rows, output columns) */
+    /* swiglu epilogue ([N,K] weights of 2H rows, H = p.N output columns): the first BN/2 weight rows of a tile are
+     * value rows n0 .., the others the gate rows H + n0 ..; the tile then owns BN/2 output columns */
+    const bool gated = p.swiglu_cols != 0u;
+    const uint32_t out_bn = gated ? BN / 2u : BN;
+    auto wrow = [&](uint32_t tn0, uint32_t r) __attribute__((always_inline)) {
+        return gated ? (r < BN / 2u ? tn0 + r : p.swiglu_cols + tn0 + (r - BN / 2u)) : tn0 + r;
+    };
+    auto wrow_ok = [&](uint32_t tn0, uint32_t r) __attribute__((always_inline)) {
+        return tn0 + (gated && r >= BN / 2u ? r - BN / 2u : r) < p.N;
+    };
     auto locate = [&](uint32_t t, uint32_t &tm0, uint32_t &tn0) __attribute__((always_inline)) {
         uint32_t pid = t;
         if ((total & 7u) == 0u) pid = (pid & 7u) * (total >> 3) + (pid >> 3);
@@ -100,10 +110,10 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
         const uint32_t first_m = (pid / width) * 8u;
         const uint32_t gsz = min(tiles_m - first_m, 8u);
         tm0 = (first_m + (pid % width) % gsz) * BM;
-        tn0 = ((pid % width) / gsz) * BN;
+        tn0 = ((pid % width) / gsz) * out_bn;
     };
     auto direct_ok = [&](uint32_t tm0, uint32_t tn0) __attribute__((always_inline)) {
-        return DIRECT && tm0 + BM <= p.M && tn0 + BN <= p.N && (p.K % 64u) == 0u && p.K >= 128u;
+        return DIRECT && tm0 + BM <= p.M && tn0 + out_bn <= p.N && (p.K % 64u) == 0u && p.K >= 128u;
     };
 
     uint32_t tid_opaque = threadIdx.x;
@@ -150,9 +160,10 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
         if (W_NK) {
 #pragma unroll
             for (int i = 0; i < B_PER; ++i) {
-                const uint32_t gn = n0 + a_r + 32u * i;
+                const uint32_t gn = wrow(n0, a_r + 32u * (uint32_t)i);
                 if (GUARDED) rb[i] = zero8;
-                if (!GUARDED || (kok && gn < p.N)) rb[i] = *reinterpret_cast<const gd_half8 *>(w + (size_t)gn * p.ldw + k);
+                if (!GUARDED || (kok && wrow_ok(n0, a_r + 32u * (uint32_t)i)))
+                    rb[i] = *reinterpret_cast<const gd_half8 *>(w + (size_t)gn * p.ldw + k);
             }
         } else {
             const uint32_t gn = n0 + kb_nc * 8u;
@@ -234,7 +245,7 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
         } else if (W_NK) {
             const uint32_t tb = t - (uint32_t)A_DIRECT;
             const uint32_t row0 = wave_u * (BN / 4u) + tb * RW;
-            gd_tile_load_lds16(w + (size_t)(tn0 + row0) * p.ldw + kt * DBK, (tb & 1u) ? d_off_b1 : d_off_b,
+            gd_tile_load_lds16(w + (size_t)wrow(tn0, row0) * p.ldw + kt * DBK, (tb & 1u) ? d_off_b1 : d_off_b,
                                lds_base + ((2u * BM + stage * BN) * CH + row0 * CH) * 16u);
         } else {
             /* k-rows kr0 .. kr0+RPL-1 of the tile; lane L fills position L%CPR of row kr0 + L/CPR */
@@ -395,12 +406,14 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
         for (int j = 0; j < WN; ++j) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const uint32_t gc = n0 + wn * (WN * 32u) + (uint32_t)j * 32u + 8u * (uint32_t)q + 4u * frag_c;
-                if (vec && gc + 4u <= p.N) {
+                const uint32_t lc = wn * (WN * 32u) + (uint32_t)j * 32u + 8u * (uint32_t)q + 4u * frag_c;
+                const uint32_t gc = wrow(n0, lc); /* the four columns of a quad lie in the same half of a gated tile */
+                if (vec && (gc & 3u) == 0u && wrow_ok(n0, lc + 3u)) {
                     bq[j][q] = *reinterpret_cast<const gd_half4 *>(bias + gc);
                 } else {
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) bq[j][q][r] = bias[min(gc + (uint32_t)r, p.N - 1u)];
+                    for (int r = 0; r < 4; ++r)
+                        bq[j][q][r] = wrow_ok(n0, lc + (uint32_t)r) ? bias[gc + (uint32_t)r] : (gd_half)0.f;
                 }
             }
         }
@@ -427,12 +440,7 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
         }
         __syncthreads();
         constexpr uint32_t CPRW = BN / 8u; /* 16-byte chunks per row */
-#pragma unroll
-        for (uint32_t idx0 = 0; idx0 < 64u * CPRW; idx0 += 256u) {
-            const uint32_t idx = idx0 + tid;
-            const uint32_t er = idx / CPRW, v = idx % CPRW;
-            const uint32_t gr = m0 + (er >> 5) * (WM * 32u) + (uint32_t)I * 32u + (er & 31u), gc = n0 + v * 8u;
-            if (gr >= p.M || gc >= p.N) continue;
+        auto read_chunk = [&](uint32_t er, uint32_t v) __attribute__((always_inline)) {
             const uint32_t xr = er & 31u;
             const gd_half8 raw = *reinterpret_cast<const gd_half8 *>(epi + (er * EU + 2u * (v ^ (xr >> 1))) * 8u);
             gd_half8 h = raw;
@@ -443,6 +451,35 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
                     h[4 + t] = raw[t];
                 }
             }
+            return h;
+        };
+        if (gated) {
+            /* value chunk v and gate chunk v + CPRW/2 of the same row make output chunk v */
+#pragma unroll
+            for (uint32_t idx0 = 0; idx0 < 32u * CPRW; idx0 += 256u) {
+                const uint32_t idx = idx0 + tid;
+                const uint32_t er = idx / (CPRW / 2u), v = idx % (CPRW / 2u);
+                const uint32_t gr = m0 + (er >> 5) * (WM * 32u) + (uint32_t)I * 32u + (er & 31u), gc = n0 + v * 8u;
+                if (gr >= p.M || gc >= p.N) continue;
+                const gd_half8 hv = read_chunk(er, v), hg = read_chunk(er, v + CPRW / 2u);
+                gd_half8 h;
+#pragma unroll
+                for (int t = 0; t < 8; ++t) h[t] = (gd_half)((float)hv[t] * gd_tile_silu((float)hg[t]));
+                gd_half *yr = y + (size_t)gr * p.ldy + gc;
+                if (vector_store && gc + 8u <= p.N) {
+                    *reinterpret_cast<gd_half8 *>(yr) = h;
+                } else {
+                    for (uint32_t t = 0; t < 8u && gc + t < p.N; ++t) yr[t] = h[t];
+                }
+            }
+        } else {
+#pragma unroll
+        for (uint32_t idx0 = 0; idx0 < 64u * CPRW; idx0 += 256u) {
+            const uint32_t idx = idx0 + tid;
+            const uint32_t er = idx / CPRW, v = idx % CPRW;
+            const uint32_t gr = m0 + (er >> 5) * (WM * 32u) + (uint32_t)I * 32u + (er & 31u), gc = n0 + v * 8u;
+            if (gr >= p.M || gc >= p.N) continue;
+            gd_half8 h = read_chunk(er, v);
             gd_half *yr = y + (size_t)gr * p.ldy + gc;
             if (vector_store && gc + 8u <= p.N) {
                 if (p.has_residual) {
@@ -450,7 +487,9 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
 #pragma unroll
                     for (int t = 0; t < 8; ++t) h[t] = r[t] + h[t];
                 }
-                *reinterpret_cast<gd_half8 *>(yr) = h;
+                /* long K: the output is not read again soon and would only push operand panels out of L2 */
+                if (p.K >= 1024u) __builtin_nontemporal_store(h, reinterpret_cast<gd_half8 *>(yr));
+                else *reinterpret_cast<gd_half8 *>(yr) = h;
             } else {
                 for (uint32_t t = 0; t < 8u && gc + t < p.N; ++t) {
                     gd_half v1 = h[t];
@@ -458,6 +497,7 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
                     yr[t] = v1;
                 }
             }
+        }
         }
         if (I + 1 < WM) __syncthreads(); /* the next pass overwrites the buffer; after the last pass the barriers
                                             of the next tile's main loop come first */
@@ -473,7 +513,7 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
     };
 
         /* interior tile: every staged chunk is in range, so the main loop carries no guards */
-        const bool interior = m0 + BM <= p.M && n0 + BN <= p.N && (p.K % GD_TILE_BK) == 0u;
+        const bool interior = m0 + BM <= p.M && n0 + out_bn <= p.N && (p.K % GD_TILE_BK) == 0u;
 
         if (PRO == GD_HIP_PRO_RMS_NORM) {
             __syncthreads(); /* the previous tile's epilogue has left the buffer that holds the row factors */
@@ -567,7 +607,8 @@ static int launch_tile_one(hipStream_t stream, const gd_half *x, const gd_half *
         if (e != hipSuccess) return (int)e;
         configured = true;
     }
-    const uint32_t tiles_m = (p.M + BM - 1u) / BM, tiles_n = (p.N + BN - 1u) / BN;
+    const uint32_t out_bn = p.swiglu_cols != 0u ? BN / 2u : BN; /* output columns per tile */
+    const uint32_t tiles_m = (p.M + BM - 1u) / BM, tiles_n = (p.N + out_bn - 1u) / out_bn;
     /* persistent workgroups: at most `workgroups` of them (a multiple of 8 keeps the tile -> XCD relation) */
     const uint32_t grid = tiles_m * tiles_n < workgroups ? tiles_m * tiles_n : workgroups;
     kernel<<<grid, 256, lds, stream>>>(x, w, bias, residual, norm_w, y, p, tiles_m, tiles_n, vector_store);

@@ -340,7 +340,7 @@ gd_status gd_backend_linear_nt(gd_backend *backend, const gd_backend_matrix_view
  *     | half(half(t) + bias)                         bias_mode 2 (gd_linear_transposed_weight)
  *   y = u, or half(residual + u) when residual != NULL (gd_add)                      epilogue 0
  *     | half(u[:, :H] * silu(u[:, H:])), w [2H,K], bias [2H], y [M,H]                epilogue 1 (the gd_swiglu_split
- *       that follows the up/gate projection; w_is_nk only, no residual, fewer than 128 rows, else UNSUPPORTED) */
+ *       that follows the up/gate projection; w_is_nk only, no residual, else UNSUPPORTED) */
 typedef struct gd_backend_fused_linear_args {
     uint32_t w_is_nk;
     uint32_t bias_mode;
