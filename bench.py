@@ -28,7 +28,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per sdpa_decode launch at this shape from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
 # profiles/sdpa_decode_config2_pmc.md (fetch scaled by the factor a 64 MiB device copy shows in the same run)
-SDPA_TRAFFIC_BYTES = 67327400
+SDPA_TRAFFIC_BYTES = 67300600
 
 
 def _package():
