@@ -98,6 +98,51 @@ def test_batched_ragged_prefill_and_steps(gda, oracle, window, tie):
         dev.close()
 
 
+def test_scaled_architecture_prefill_and_steps(gda, oracle):
+    """The layer shapes of BASELINE configs 3 and 4 (d_model 2048, 16 heads of 128, SwiGLU hidden 5632) at two layers
+    and a 4096-token vocabulary: a ragged packed prefill long enough for the many-row kernels (336 rows: one full and
+    one ragged 256-row tile, attention over several 64-key blocks), then cached steps through the public-operator
+    loop and through the fused resident loop, all against the CPU oracle decoder."""
+    from gradients_c_amd import decoder as D
+    V, Dm, L, H, Dh, Hm, T, B = 4096, 2048, 2, 16, 128, 5632, 256, 4
+    cfg = D.gpt_config(V, Dm, L, H, Dh, Hm, T, B, 0, False, 4242)
+    dev = D.GptDecoder(cfg, max_prefill_tokens=512)
+    ref = oracle.Decoder(V, Dm, L, H, Dh, Hm, T, B, 0, 4242, False)
+    try:
+        lens = np.array([150, 40, 129, 17], np.int32)
+        cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        prompt = oracle.uniform_i32(int(cu[-1]), 4243, 0, V - 1)
+        lg_d, nx_d, gp_d = dev.prefill(prompt, cu)
+        lg_r, nx_r, gp_r = ref.prefill(prompt, cu)
+        worst = np.abs(lg_d.astype(np.float32) - lg_r.astype(np.float32)).max()
+        print("prefill logits: worst difference", worst, "largest logit", np.abs(lg_r.astype(np.float32)).max())
+        assert worst < 8e-3
+        _assert_ids(nx_d, nx_r, gp_d, gp_r, "prefill")
+        for l in range(L):
+            for b in range(B):
+                kd, kr = dev.read_tensor("k_cache", l)[b, :lens[b]], ref.tensor("k_cache", l)[b, :lens[b]]
+                vd, vr = dev.read_tensor("v_cache", l)[b, :lens[b]], ref.tensor("v_cache", l)[b, :lens[b]]
+                assert np.abs(kd.astype(np.float32) - kr.astype(np.float32)).max() < 8e-3, (l, b)
+                assert np.abs(vd.astype(np.float32) - vr.astype(np.float32)).max() < 8e-3, (l, b)
+        tok = nx_r.copy()
+        for step in range(4):
+            lg_d, nx_d, gp_d = dev.step(tok)
+            lg_r, nx_r, gp_r = ref.step(tok)
+            assert np.abs(lg_d.astype(np.float32) - lg_r.astype(np.float32)).max() < 8e-3, step
+            _assert_ids(nx_d, nx_r, gp_d, gp_r, f"step {step}")
+            tok = nx_r.copy()
+        # fused resident loop from the same state: every step against the oracle following the device's tokens
+        ids, gaps, _ = dev.run_resident(tok, 6)
+        for s in range(6):
+            _, nx_r, gp_r = ref.step(tok)
+            bad = [i for i in np.nonzero(ids[s] != nx_r)[0] if min(gaps[s][i], gp_r[i]) >= 1e-3]
+            assert not bad, (s, bad)
+            tok = ids[s].copy()
+        assert np.array_equal(dev.positions, lens + 10) and np.array_equal(ref.positions, lens + 10)
+    finally:
+        dev.close()
+
+
 def _resident_pair(D, oracle, seed):
     cfg = D.gpt_config(2048, 512, 3, 8, 64, 1536, 96, 8, 0, True, seed)
     a, b = D.GptDecoder(cfg, max_prefill_tokens=8 * 32), D.GptDecoder(cfg, max_prefill_tokens=8 * 32)

@@ -256,6 +256,42 @@ def test_decode_isolated_config_shape(backend, arena, oracle, chunk):
     _close(out.read(), oracle.sdpa_decode(q, wk, wv, L, 0.125))
 
 
+def test_decode_full_size_long_context_sampled(backend, oracle):
+    """BASELINE config 3's attention at its full size (B=16, 16 heads of 128, 4096-row caches, live lengths in
+    [1024, 4096]: 537 MB of cache filled on the device), checked on sampled batch rows against a float64 softmax of
+    the downloaded rows, and for independence from the split of the key range (size-independent property)."""
+    B, H, D, T = 16, 16, 128, 4096
+    big = backend.buffer(640 << 20)
+    try:
+        k, v = big.alloc((B, T, H, D), 1), big.alloc((B, T, H, D), 1)
+        backend.rand_uniform(k, 9001, -1.0, 1.0)
+        backend.rand_uniform(v, 9002, -1.0, 1.0)
+        q = oracle.normal_f16((B, 1, H, D), 9003)
+        pos = oracle.uniform_i32(B, 9004, 1023, 4095)
+        tq, tp, out = big.from_numpy(q), big.from_numpy(pos), big.alloc((B, 1, H, D), 1)
+        scale = 1.0 / np.sqrt(D)
+        results = []
+        for chunk in (0, 512, 2048):
+            backend.set_tunable("sdpa_chunk", chunk)
+            try:
+                backend.sdpa_decode_positions(tq, k, v, tp, out, scale)
+            finally:
+                backend.set_tunable("sdpa_chunk", 0)
+            results.append(out.read().astype(np.float32))
+        assert np.abs(results[0] - results[1]).max() < 1e-3 and np.abs(results[0] - results[2]).max() < 1e-3
+        for b in (0, 7, 15):
+            n = int(pos[b]) + 1
+            kb = k.rows(b, 1).read()[0, :n].astype(np.float64)  # [n, H, D]
+            vb = v.rows(b, 1).read()[0, :n].astype(np.float64)
+            sc = np.einsum("hd,nhd->hn", q[b, 0].astype(np.float64), kb) * scale
+            w = np.exp(sc - sc.max(axis=1, keepdims=True))
+            want = np.einsum("hn,nhd->hd", w / w.sum(axis=1, keepdims=True), vb)
+            got = results[0][b, 0]
+            assert np.all(np.abs(got - want) <= 1e-3 + 2e-3 * np.abs(want)), b
+    finally:
+        backend.free(big)
+
+
 @pytest.mark.parametrize("H,Hkv,D", [(8, 8, 64), (16, 16, 128), (8, 2, 64), (8, 1, 128), (6, 3, 64), (6, 2, 64)])
 def test_decode_head_layouts(backend, arena, oracle, H, Hkv, D):
     pos = np.array([0, 1, 63, 64, 200, 299, -1, 31], np.int32)
@@ -693,6 +729,72 @@ def test_many_row_projection_prologues(backend, arena, oracle, M, K, N, nk):
     _close(y.read(), oracle.swiglu_split_linear(x12, w_kn, bias))
     backend.fused_linear(arena.from_numpy(x), tw, tb, None, arena.from_numpy(nw), y, nk, 1, 2, 1e-5)
     _close(y.read(), oracle.linear(oracle.rms_norm(x, nw, 1e-5), w_kn, bias))
+
+
+def test_many_row_projection_full_size_sampled(backend, oracle):
+    """The packed-prefill projections of BASELINE config 4 at full size (30,229 rows): the qkv projection ([N,K]
+    weight, bias added after the F16 rounding) and the down projection ([K,N] weight, F32 bias, residual), operands
+    filled on the device, sampled rows (first, last, both sides of every kind of tile edge) against float64."""
+    M = 30229
+    big = backend.buffer(900 << 20)
+    try:
+        for (K, N, nk) in ((2048, 6144, True), (5632, 2048, False)):
+            big.reset()
+            x, w = big.alloc((M, K), 1), big.alloc((N, K) if nk else (K, N), 1)
+            backend.rand_uniform(x, 9101 + K, -1.0, 1.0)
+            backend.rand_uniform(w, 9102 + K, -0.05, 0.05)
+            bias = oracle.normal_f16((N,), 9103, 0.5)
+            res = big.alloc((M, N), 1)
+            backend.rand_uniform(res, 9104, -1.0, 1.0)
+            y = big.alloc((M, N), 1)
+            backend.fused_linear(x, w, big.from_numpy(bias), None if nk else res, None, y, nk, 2 if nk else 1, 0)
+            wf = w.read().astype(np.float64)
+            wf = wf.T if nk else wf
+            for r in (0, 1, 255, 256, 4095, 4096, 17000, 30207, 30208, 30228):
+                xr = x.rows(r, 1).read()[0].astype(np.float64)
+                t = xr @ wf
+                if nk:
+                    want = (t.astype(np.float16).astype(np.float32) + bias.astype(np.float32)).astype(np.float16)
+                else:
+                    u = (t + bias.astype(np.float64)).astype(np.float16)
+                    want = (res.rows(r, 1).read()[0].astype(np.float32) + u.astype(np.float32)).astype(np.float16)
+                got = y.rows(r, 1).read()[0].astype(np.float32)
+                scale_ = np.abs(t) + np.abs(bias.astype(np.float64)) + 1.0
+                assert np.all(np.abs(got - want.astype(np.float32)) <= 1e-3 + 2e-3 * scale_), (K, N, r)
+    finally:
+        backend.free(big)
+
+
+def test_varlen_full_size_sampled(backend, oracle):
+    """The packed causal prefill attention of BASELINE config 4 at full size: 32 sequences of 64..2048 tokens, 16
+    heads of 128; sampled query rows (first and last of a sequence, both sides of 64-key block edges and of
+    128-row workgroup edges) against a float64 softmax over the visible keys."""
+    H, D = 16, 128
+    lens = oracle.uniform_i32(32, 9201, 64, 2048)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    n = int(cu[-1])
+    big = backend.buffer(640 << 20)
+    try:
+        q, k, v, out = (big.alloc((n, H, D), 1) for _ in range(4))
+        for t, seed in ((q, 9202), (k, 9203), (v, 9204)):
+            backend.rand_uniform(t, seed, -1.0, 1.0)
+        scale = 1.0 / np.sqrt(D)
+        backend.sdpa_varlen(q, k, v, big.from_numpy(cu), out, scale)
+        for s in (0, 5, 17, 31):
+            base, L = int(cu[s]), int(lens[s])
+            ks = k.rows(base, L).read().astype(np.float64)
+            vs = v.rows(base, L).read().astype(np.float64)
+            for i in sorted({0, 1, 63, 64, 127, 128, L // 2, L - 2, L - 1}):
+                if i >= L:
+                    continue
+                qi = q.rows(base + i, 1).read()[0].astype(np.float64)  # [H, D]
+                sc = np.einsum("hd,nhd->hn", qi, ks[:i + 1]) * scale
+                wgt = np.exp(sc - sc.max(axis=1, keepdims=True))
+                want = np.einsum("hn,nhd->hd", wgt / wgt.sum(axis=1, keepdims=True), vs[:i + 1])
+                got = out.rows(base + i, 1).read()[0].astype(np.float32)
+                assert np.all(np.abs(got - want) <= 1e-3 + 2e-3 * np.abs(want)), (s, i)
+    finally:
+        backend.free(big)
 
 
 def test_many_row_projection_row_pitches_and_unaligned_output(backend, arena, oracle, gda):
