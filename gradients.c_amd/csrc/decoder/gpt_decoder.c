@@ -26,6 +26,10 @@ typedef struct gpt_linear {
 typedef struct gpt_block {
     gd_tensor attn_norm_w, mlp_norm_w;
     gpt_linear qkv_proj, attn_proj, up_gate, down_proj;
+    /* the down projection's weight once more as [d_model, hidden] (the reference keeps it [hidden, d_model]): with
+     * few rows the projection streams the weight once, and rows that are contiguous along the summed dimension
+     * come in whole cache lines per workgroup; a 16-column slice of the [K,N] layout uses a quarter of every line */
+    gd_tensor down_t;
 } gpt_block;
 
 struct gd_gpt_decoder {
@@ -64,7 +68,9 @@ static double uniform_open_closed_at(uint64_t seed, uint64_t n)
     return ((double)(mix64(seed + n * UINT64_C(0x9e3779b97f4a7c15)) >> 11) + 1.0) * (1.0 / 9007199254740992.0);
 }
 
-static gd_status init_normal(gd_context *ctx, gd_tensor *t, uint64_t seed, float stddev)
+/* twin != NULL: t is [rows, cols]; the same values also go to twin as [cols, rows] */
+static gd_status init_normal_twin(gd_context *ctx, gd_tensor *t, uint64_t seed, float stddev, gd_tensor *twin,
+                                  int64_t rows, int64_t cols)
 {
     int64_t n, pairs, pi;
     float *values;
@@ -82,8 +88,28 @@ static gd_status init_normal(gd_context *ctx, gd_tensor *t, uint64_t seed, float
         if (2 * pi + 1 < n) values[2 * pi + 1] = (float)(radius * sin(angle) * (double)stddev);
     }
     st = gd_tensor_write_f32(ctx, t, values, (size_t)n);
+    if (st == GD_OK && twin != NULL) {
+        float *turned = (float *)malloc((size_t)n * sizeof(float));
+        int64_t r;
+        if (turned == NULL) {
+            free(values);
+            return GD_ERR_OUT_OF_MEMORY;
+        }
+#pragma omp parallel for schedule(static)
+        for (r = 0; r < cols; ++r) {
+            int64_t c;
+            for (c = 0; c < rows; ++c) turned[r * rows + c] = values[c * cols + r];
+        }
+        st = gd_tensor_write_f32(ctx, twin, turned, (size_t)n);
+        free(turned);
+    }
     free(values);
     return st;
+}
+
+static gd_status init_normal(gd_context *ctx, gd_tensor *t, uint64_t seed, float stddev)
+{
+    return init_normal_twin(ctx, t, seed, stddev, NULL, 0, 0);
 }
 
 static gd_status param(gd_context *ctx, gd_dtype dtype, uint32_t rank, int64_t d0, int64_t d1, gd_tensor *out)
@@ -114,7 +140,7 @@ size_t gd_gpt_params_bytes(const gd_gpt_config *c)
 {
     const size_t Dm = (size_t)c->d_model, Hm = (size_t)c->mlp_hidden, V = (size_t)c->vocab;
     size_t per_layer = 2U * pad256(Dm * 2U) + pad256(3U * Dm * Dm * 2U) + pad256(3U * Dm * 2U) + pad256(Dm * Dm * 2U) +
-                       pad256(Dm * 2U) + pad256(2U * Hm * Dm * 2U) + pad256(2U * Hm * 2U) + pad256(Hm * Dm * 2U) +
+                       pad256(Dm * 2U) + pad256(2U * Hm * Dm * 2U) + pad256(2U * Hm * 2U) + 2U * pad256(Hm * Dm * 2U) +
                        pad256(Dm * 2U);
     size_t total = pad256(V * Dm * 2U) * (c->tie_lm_head ? 1U : 2U) + pad256(V * 2U) + pad256(Dm * 2U);
     return total + per_layer * (size_t)c->n_layers + 4096U;
@@ -179,7 +205,13 @@ gd_status gd_gpt_decoder_create(gd_context *ctx, const gd_gpt_config *cfg, gd_gp
         STEP(linear_init(ctx, &b->qkv_proj, cfg->d_model, 3 * (int64_t)cfg->d_model, true, splitmix64(bs ^ 1U), std));
         STEP(linear_init(ctx, &b->attn_proj, cfg->d_model, cfg->d_model, true, splitmix64(bs ^ 2U), resid));
         STEP(linear_init(ctx, &b->up_gate, cfg->d_model, 2 * (int64_t)cfg->mlp_hidden, true, splitmix64(bs ^ 3U), std));
-        STEP(linear_init(ctx, &b->down_proj, cfg->mlp_hidden, cfg->d_model, false, splitmix64(bs ^ 4U), resid));
+        b->down_proj.transposed = false;
+        STEP(param(ctx, GD_DTYPE_F16, 2U, cfg->mlp_hidden, cfg->d_model, &b->down_proj.weight));
+        STEP(param(ctx, GD_DTYPE_F16, 2U, cfg->d_model, cfg->mlp_hidden, &b->down_t));
+        STEP(init_normal_twin(ctx, &b->down_proj.weight, splitmix64(bs ^ 4U), resid, &b->down_t, cfg->mlp_hidden,
+                              cfg->d_model));
+        STEP(param(ctx, GD_DTYPE_F16, 1U, cfg->d_model, 0, &b->down_proj.bias));
+        STEP(gd_tensor_zero_(ctx, &b->down_proj.bias));
         STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_F16, gd_shape_make(4U, cache_dims), 256U, &d->k_cache[l]));
         STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_F16, gd_shape_make(4U, cache_dims), 256U, &d->v_cache[l]));
     }
@@ -230,6 +262,7 @@ gd_tensor *gd_gpt_decoder_tensor(gd_gpt_decoder *d, const char *name, int32_t la
     if (!strcmp(name, "w_upgate")) return &b->up_gate.weight;
     if (!strcmp(name, "b_upgate")) return &b->up_gate.bias;
     if (!strcmp(name, "w_down")) return &b->down_proj.weight;
+    if (!strcmp(name, "w_down_t")) return &b->down_t;
     if (!strcmp(name, "b_down")) return &b->down_proj.bias;
     if (!strcmp(name, "k_cache")) return &d->k_cache[layer];
     if (!strcmp(name, "v_cache")) return &d->v_cache[layer];
@@ -512,8 +545,9 @@ static gd_status fused_project_rows(gd_gpt_decoder *d, int64_t B, const gd_tenso
     if (residual != NULL) mview(residual, B, n_out, &rm);
     if (norm_w != NULL) vview(norm_w, &nv);
     vview(bias, &bv);
-    a.w_is_nk = lin->transposed ? 1U : 0U;
-    a.bias_mode = lin->transposed ? 2U : 1U; /* [N,K]: matmul_nt + add (two roundings); [K,N]: fused F32 bias */
+    a.w_is_nk = (lin->transposed || w_override != NULL) ? 1U : 0U; /* an override is the [N,K] twin of a [K,N] weight */
+    a.bias_mode = lin->transposed ? 2U : 1U; /* gd_linear_transposed_weight: matmul_nt + add (two roundings);
+                                                gd_linear: F32 bias in front of the single rounding */
     a.prologue = prologue;
     a.eps = d->cfg.rms_eps;
     a.epilogue = epilogue;
@@ -588,10 +622,10 @@ static gd_status enqueue_fused_step(gd_gpt_decoder *d, gd_tensor *logits)
         if (B < 128) {
             /* the gate is applied in the up/gate projection's epilogue: the [B,2Hm] intermediate is never stored */
             TRY(fused_project(d, &x1, Dm, &b->up_gate, NULL, &b->up_gate.bias, NULL, &b->mlp_norm_w, 2U, 1U, Hm, &ug));
-            TRY(fused_project(d, &ug, Hm, &b->down_proj, NULL, &b->down_proj.bias, &x1, NULL, 0U, 0U, Dm, &x2));
+            TRY(fused_project(d, &ug, Hm, &b->down_proj, &b->down_t, &b->down_proj.bias, &x1, NULL, 0U, 0U, Dm, &x2));
         } else {
             TRY(fused_project(d, &x1, Dm, &b->up_gate, NULL, &b->up_gate.bias, NULL, &b->mlp_norm_w, 2U, 0U, 2 * Hm, &ug));
-            TRY(fused_project(d, &ug, 2 * Hm, &b->down_proj, NULL, &b->down_proj.bias, &x1, NULL, 1U, 0U, Dm, &x2));
+            TRY(fused_project(d, &ug, 2 * Hm, &b->down_proj, &b->down_t, &b->down_proj.bias, &x1, NULL, 1U, 0U, Dm, &x2));
         }
         x = x2;
     }
