@@ -7,7 +7,7 @@
  */
 #include "../../_shared/hip_device.h"
 
-#define GD_ARGMAX_THREADS 256
+#define GD_ARGMAX_MAX_THREADS 1024 /* long rows; short rows run with 256 */
 #define GD_NEG_INF (-__builtin_inff())
 
 struct gd_top2 {
@@ -55,18 +55,30 @@ struct gd_hip_advance {
 };
 
 template <typename T, bool ADVANCE>
-__global__ void __launch_bounds__(GD_ARGMAX_THREADS)
+__global__ void __launch_bounds__(GD_ARGMAX_MAX_THREADS)
 gd_argmax_rows_kernel(const T *__restrict__ logits, int32_t *__restrict__ ids, float *__restrict__ gap,
                       uint64_t cols, gd_hip_advance adv)
 {
-    __shared__ gd_top2 sm[GD_ARGMAX_THREADS / 64];
+    __shared__ gd_top2 sm[GD_ARGMAX_MAX_THREADS / 64];
     __shared__ int32_t s_token;
     const T *row = logits + (uint64_t)blockIdx.x * cols;
     gd_top2 t;
     t.best = GD_NEG_INF;
     t.second = GD_NEG_INF;
     t.idx = -1;
-    for (uint64_t c = threadIdx.x; c < cols; c += GD_ARGMAX_THREADS) gd_top2_push(t, (float)row[c], (int32_t)c);
+    const uint32_t threads = blockDim.x;
+    uint64_t done = 0; /* columns covered by the vector part */
+    if (sizeof(T) == 2 && (reinterpret_cast<uintptr_t>(row) & 15u) == 0u) {
+        /* 8 halfs per lane and trip; lane-major order keeps the lowest-index rule: pushes of one lane ascend */
+        const uint64_t whole = cols & ~(uint64_t)7;
+        for (uint64_t c = (uint64_t)threadIdx.x * 8u; c < whole; c += (uint64_t)threads * 8u) {
+            const gd_half8 v = *reinterpret_cast<const gd_half8 *>(row + c);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) gd_top2_push(t, (float)v[e], (int32_t)(c + e));
+        }
+        done = whole;
+    }
+    for (uint64_t c = done + threadIdx.x; c < cols; c += threads) gd_top2_push(t, (float)row[c], (int32_t)c);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         gd_top2 o;
@@ -79,7 +91,7 @@ gd_argmax_rows_kernel(const T *__restrict__ logits, int32_t *__restrict__ ids, f
     __syncthreads();
     if (threadIdx.x == 0) {
         gd_top2 r = sm[0];
-        for (int w = 1; w < GD_ARGMAX_THREADS / 64; ++w) r = gd_top2_merge(r, sm[w]);
+        for (uint32_t w = 1; w < threads / 64u; ++w) r = gd_top2_merge(r, sm[w]);
         const int32_t token = r.idx < 0 ? 0 : r.idx;
         const float g = (r.idx >= 0 && r.second > GD_NEG_INF) ? r.best - r.second : __builtin_inff();
         ids[blockIdx.x] = token;
@@ -99,7 +111,7 @@ gd_argmax_rows_kernel(const T *__restrict__ logits, int32_t *__restrict__ ids, f
         __syncthreads();
         const gd_u128 *src = reinterpret_cast<const gd_u128 *>(adv.table + (size_t)s_token * adv.row_bytes);
         gd_u128 *dst = reinterpret_cast<gd_u128 *>(adv.next_x + (size_t)blockIdx.x * adv.row_bytes);
-        for (uint32_t c = threadIdx.x; c < adv.row_bytes / 16u; c += GD_ARGMAX_THREADS) dst[c] = src[c];
+        for (uint32_t c = threadIdx.x; c < adv.row_bytes / 16u; c += threads) dst[c] = src[c];
     }
 }
 
@@ -109,9 +121,9 @@ extern "C" int gd_hip_launch_argmax_rows(hipStream_t stream, const void *logits,
     const gd_hip_advance none = {nullptr, nullptr, nullptr, nullptr, 0u, 0, nullptr, nullptr, 0u};
     if (rows == 0) return (int)hipSuccess;
     if (is_f16)
-        gd_argmax_rows_kernel<gd_half, false><<<(unsigned)rows, GD_ARGMAX_THREADS, 0, stream>>>((const gd_half *)logits, ids, gap, cols, none);
+        gd_argmax_rows_kernel<gd_half, false><<<(unsigned)rows, cols >= 8192u ? GD_ARGMAX_MAX_THREADS : 256, 0, stream>>>((const gd_half *)logits, ids, gap, cols, none);
     else
-        gd_argmax_rows_kernel<float, false><<<(unsigned)rows, GD_ARGMAX_THREADS, 0, stream>>>((const float *)logits, ids, gap, cols, none);
+        gd_argmax_rows_kernel<float, false><<<(unsigned)rows, cols >= 8192u ? GD_ARGMAX_MAX_THREADS : 256, 0, stream>>>((const float *)logits, ids, gap, cols, none);
     return (int)hipGetLastError();
 }
 
@@ -124,8 +136,8 @@ extern "C" int gd_hip_launch_argmax_advance(hipStream_t stream, const void *logi
                                 (const unsigned char *)table, (unsigned char *)next_x, row_bytes};
     if (rows == 0) return (int)hipSuccess;
     if (is_f16)
-        gd_argmax_rows_kernel<gd_half, true><<<(unsigned)rows, GD_ARGMAX_THREADS, 0, stream>>>((const gd_half *)logits, ids, nullptr, cols, adv);
+        gd_argmax_rows_kernel<gd_half, true><<<(unsigned)rows, cols >= 8192u ? GD_ARGMAX_MAX_THREADS : 256, 0, stream>>>((const gd_half *)logits, ids, nullptr, cols, adv);
     else
-        gd_argmax_rows_kernel<float, true><<<(unsigned)rows, GD_ARGMAX_THREADS, 0, stream>>>((const float *)logits, ids, nullptr, cols, adv);
+        gd_argmax_rows_kernel<float, true><<<(unsigned)rows, cols >= 8192u ? GD_ARGMAX_MAX_THREADS : 256, 0, stream>>>((const float *)logits, ids, nullptr, cols, adv);
     return (int)hipGetLastError();
 }
