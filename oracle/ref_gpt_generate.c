@@ -11,6 +11,10 @@
  * Output file:         int32 ids[new_tokens][batch], then float logits[new_tokens][batch][GPT_VOCAB_SIZE]
  * (row 0 of both comes from the prefill, row s > 0 from decode step s).
  * Seed: argv[3] (decimal), the weight seed handed to gpt_lm_init.
+ * Optional argv[4]: the freshly initialised model is also written there by the reference's own
+ * gd_module_save_state (src/nn/module_io.c:700-800), which gives the loader tests a checkpoint that the
+ * reference itself produced.  The model dimensions are the example's compile-time macros
+ * (gpt_lm_shared.h:10-28); the Makefile also builds a small-dimension variant for that fixture.
  */
 #include "gpt_lm_shared.c"
 
@@ -34,7 +38,7 @@ int main(int argc, char **argv)
     uint64_t rng = 1U;
     int batch, steps, total = 0, b, i, s;
     gd_status st;
-    if (argc != 4) die("usage: ref_gpt_generate <in> <out> <seed>");
+    if (argc != 4 && argc != 5) die("usage: ref_gpt_generate <in> <out> <seed> [checkpoint to write]");
     f = fopen(argv[1], "rb");
     if (f == NULL || fread(head, sizeof(head[0]), 3U, f) != 3U) die("cannot read the input header");
     batch = head[0];
@@ -83,6 +87,13 @@ int main(int argc, char **argv)
     }
     if (st != GD_OK) gpt_fail_status(ctx, st, "gd_context_create", __LINE__);
     gpt_lm_init(ctx, &model, &config);
+    if (argc == 5) {
+        static const char meta[] = "{\"writer\":\"gd_module_save_state\",\"model\":\"gpt_lm\"}";
+        gd_module_save_options save = gd_module_save_options_default();
+        save.metadata = meta;
+        save.metadata_len = sizeof(meta) - 1U;
+        TRY(ctx, gd_module_save_state(ctx, &model.mod, argv[4], &save));
+    }
     TRY(ctx, gd_context_seal_params(ctx));
     TRY(ctx, gpt_lm_prepare_generation_cache(ctx, &model, &config, batch, GPT_CONTEXT_LENGTH, &cache));
     gd_module_set_training(&model.mod, false);
