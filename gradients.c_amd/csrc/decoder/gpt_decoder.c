@@ -10,6 +10,9 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <stdio.h>
+
+#include "gd_checkpoint.h"
 #include "gd_gpt_decoder.h"
 
 #define TRY(expr)                       \
@@ -270,6 +273,130 @@ gd_tensor *gd_gpt_decoder_tensor(gd_gpt_decoder *d, const char *name, int32_t la
 }
 
 int32_t *gd_gpt_decoder_positions(gd_gpt_decoder *d) { return d != NULL ? d->pos : NULL; }
+
+/* ---- weights from a checkpoint of the reference ------------------------------------------ */
+
+typedef struct ckpt_slot {
+    char path[GD_CHECKPOINT_PATH_MAX];
+    gd_tensor *dst, *second; /* second: another tensor that receives the same values (untied LM head) */
+    gd_tensor *turned;       /* [cols, rows] copy of a [rows, cols] weight */
+    const gd_checkpoint_entry *entry;
+} ckpt_slot;
+
+static void slot_set(ckpt_slot *s, gd_tensor *dst, const char *fmt, int32_t layer)
+{
+    memset(s, 0, sizeof(*s));
+    (void)snprintf(s->path, sizeof(s->path), fmt, (int)layer);
+    s->dst = dst;
+}
+
+/* same test as the reference's gd_ckpt_file_entry_matches_tensor (src/nn/module_io.c:809-824) */
+static bool entry_fits(const gd_checkpoint_entry *e, const gd_tensor *t)
+{
+    size_t nbytes = 0U;
+    uint32_t i;
+    if (gd_tensor_logical_nbytes(t, &nbytes) != GD_OK || e->dtype != t->dtype || e->rank != t->rank ||
+        e->nbytes != (uint64_t)nbytes)
+        return false;
+    for (i = 0U; i < t->rank; ++i) {
+        if (e->shape[i] != t->shape[i]) return false;
+    }
+    return true;
+}
+
+gd_status gd_gpt_decoder_load_checkpoint(gd_gpt_decoder *d, const char *path, int32_t strict)
+{
+    gd_checkpoint *ck = NULL;
+    ckpt_slot *slots;
+    unsigned char *bytes = NULL, *flipped = NULL;
+    size_t n_slots, capacity = 0U, si;
+    uint32_t fi;
+    int32_t l;
+    gd_status st;
+    if (d == NULL || path == NULL || path[0] == '\0') return GD_ERR_INVALID_ARGUMENT;
+    if (d->resident_open) return GD_ERR_BUSY;
+    /* the names gpt_lm_init gives its parameters (gpt_lm_shared.c:272-279, 303-338, 382-413) */
+    n_slots = 3U + 10U * (size_t)d->cfg.n_layers;
+    slots = (ckpt_slot *)calloc(n_slots, sizeof(*slots));
+    if (slots == NULL) return GD_ERR_OUT_OF_MEMORY;
+    slot_set(&slots[0], &d->token_embedding, "gpt_lm.token_embedding", 0);
+    if (!d->cfg.tie_lm_head) slots[0].second = &d->lm_head; /* the reference's head is the embedding table */
+    slot_set(&slots[1], &d->lm_head_bias, "gpt_lm.lm_head_bias", 0);
+    slot_set(&slots[2], &d->final_norm_w, "gpt_lm.final_norm_w", 0);
+    for (l = 0; l < d->cfg.n_layers; ++l) {
+        gpt_block *b = &d->blocks[l];
+        ckpt_slot *s = &slots[3U + 10U * (size_t)l];
+        slot_set(&s[0], &b->attn_norm_w, "gpt_lm.blocks.%d.attn_norm_w", l);
+        slot_set(&s[1], &b->mlp_norm_w, "gpt_lm.blocks.%d.mlp_norm_w", l);
+        slot_set(&s[2], &b->qkv_proj.weight, "gpt_lm.blocks.%d.qkv_proj.weight", l);
+        slot_set(&s[3], &b->qkv_proj.bias, "gpt_lm.blocks.%d.qkv_proj.bias", l);
+        slot_set(&s[4], &b->attn_proj.weight, "gpt_lm.blocks.%d.attn_proj.weight", l);
+        slot_set(&s[5], &b->attn_proj.bias, "gpt_lm.blocks.%d.attn_proj.bias", l);
+        slot_set(&s[6], &b->up_gate.weight, "gpt_lm.blocks.%d.up_gate.weight", l);
+        slot_set(&s[7], &b->up_gate.bias, "gpt_lm.blocks.%d.up_gate.bias", l);
+        slot_set(&s[8], &b->down_proj.weight, "gpt_lm.blocks.%d.down_proj.weight", l);
+        s[8].turned = &b->down_t;
+        slot_set(&s[9], &b->down_proj.bias, "gpt_lm.blocks.%d.down_proj.bias", l);
+    }
+    st = gd_checkpoint_open(path, &ck);
+    /* everything is checked before the first byte is written (module_io.c:868-899): a refused file leaves the
+     * decoder's weights as they were */
+    for (fi = 0U; st == GD_OK && fi < gd_checkpoint_count(ck); ++fi) {
+        const gd_checkpoint_entry *e = gd_checkpoint_entry_at(ck, fi);
+        ckpt_slot *hit = NULL;
+        if (e->flags == GD_CHECKPOINT_ENTRY_BUFFER) continue; /* the decoder registers no buffers */
+        for (si = 0U; si < n_slots; ++si) {
+            if (strcmp(slots[si].path, e->path) == 0) {
+                hit = &slots[si];
+                break;
+            }
+        }
+        if (hit == NULL) {
+            if (strict) st = GD_ERR_BAD_STATE; /* unexpected tensor */
+            continue;
+        }
+        if (!entry_fits(e, hit->dst)) {
+            st = GD_ERR_BAD_STATE; /* dtype, rank, shape or size differ */
+            break;
+        }
+        hit->entry = e;
+        if ((size_t)e->nbytes > capacity) capacity = (size_t)e->nbytes;
+    }
+    for (si = 0U; st == GD_OK && strict && si < n_slots; ++si) {
+        if (slots[si].entry == NULL) st = GD_ERR_BAD_STATE; /* missing tensor */
+    }
+    if (st == GD_OK && capacity > 0U) {
+        bytes = (unsigned char *)malloc(capacity);
+        flipped = (unsigned char *)malloc(capacity);
+        if (bytes == NULL || flipped == NULL) st = GD_ERR_OUT_OF_MEMORY;
+    }
+    for (si = 0U; st == GD_OK && si < n_slots; ++si) {
+        const ckpt_slot *s = &slots[si];
+        size_t nbytes;
+        if (s->entry == NULL) continue;
+        nbytes = (size_t)s->entry->nbytes;
+        st = gd_checkpoint_read(ck, s->entry, 0U, bytes, nbytes);
+        if (st == GD_OK) st = gd_tensor_write(d->ctx, s->dst, bytes, nbytes);
+        if (st == GD_OK && s->second != NULL) st = gd_tensor_write(d->ctx, s->second, bytes, nbytes);
+        if (st == GD_OK && s->turned != NULL) {
+            const int64_t rows = s->dst->shape[0], cols = s->dst->shape[1];
+            const uint16_t *src = (const uint16_t *)bytes;
+            uint16_t *out = (uint16_t *)flipped;
+            int64_t c;
+#pragma omp parallel for schedule(static)
+            for (c = 0; c < cols; ++c) {
+                int64_t r;
+                for (r = 0; r < rows; ++r) out[c * rows + r] = src[r * cols + c];
+            }
+            st = gd_tensor_write(d->ctx, s->turned, flipped, nbytes);
+        }
+    }
+    free(bytes);
+    free(flipped);
+    gd_checkpoint_close(ck);
+    free(slots);
+    return st;
+}
 
 /* ---- forward pieces -------------------------------------------------------------------- */
 

@@ -1,5 +1,6 @@
 """ctypes binding of the host core (gradients_infer.h) and the decoder (gd_gpt_decoder.h)."""
 import ctypes as C
+import os
 
 import numpy as np
 
@@ -46,6 +47,11 @@ def make_shape(dims):
 
 
 _T = C.POINTER(GdTensor)
+
+
+class CheckpointEntry(C.Structure):  # gd_checkpoint_entry
+    _fields_ = [("path", C.c_char * 256), ("flags", C.c_uint32), ("dtype", C.c_int), ("rank", C.c_uint32),
+                ("shape", C.c_int64 * 8), ("data_offset", C.c_uint64), ("nbytes", C.c_uint64)]
 _declared = False
 
 
@@ -122,6 +128,18 @@ def lib():
         l.gd_gpt_decoder_resident_run.argtypes = [_vp, C.c_int32]
         l.gd_gpt_decoder_resident_sync.argtypes = [_vp]
         l.gd_gpt_decoder_resident_end.argtypes = [_vp, _vp, _vp, C.POINTER(C.c_int32)]
+        l.gd_gpt_decoder_load_checkpoint.argtypes = [_vp, C.c_char_p, C.c_int32]
+        l.gd_checkpoint_read_metadata.argtypes = [C.c_char_p, C.POINTER(_vp), C.POINTER(C.c_size_t)]
+        l.gd_checkpoint_open.argtypes = [C.c_char_p, C.POINTER(_vp)]
+        l.gd_checkpoint_close.argtypes = [_vp]
+        l.gd_checkpoint_close.restype = None
+        l.gd_checkpoint_count.argtypes = [_vp]
+        l.gd_checkpoint_count.restype = C.c_uint32
+        l.gd_checkpoint_entry_at.argtypes = [_vp, C.c_uint32]
+        l.gd_checkpoint_entry_at.restype = C.POINTER(CheckpointEntry)
+        l.gd_checkpoint_find.argtypes = [_vp, C.c_char_p]
+        l.gd_checkpoint_find.restype = C.POINTER(CheckpointEntry)
+        l.gd_checkpoint_read.argtypes = [_vp, C.POINTER(CheckpointEntry), C.c_uint64, _vp, C.c_size_t]
         _declared = True
     return l
 
@@ -232,6 +250,12 @@ class GptDecoder:
         self.ctx.check(st, "gd_tensor_read")
         return a
 
+    def load_checkpoint(self, path, strict=True):
+        """Weights from a .gdckpt file the reference wrote for its gpt_lm example (strict as in the reference's
+        gd_module_load_options)."""
+        self.ctx.check(lib().gd_gpt_decoder_load_checkpoint(self.handle, os.fsencode(path), 1 if strict else 0),
+                       "gd_gpt_decoder_load_checkpoint")
+
     def write_tensor(self, name, layer, array):
         self.ctx.check(self.ctx.write(self.tensor(name, layer), array), "gd_tensor_write")
 
@@ -306,3 +330,70 @@ def view_of(t):
         st *= t.shape[d]
     v.count = st
     return v
+
+
+_CKPT_NUMPY = {1: np.float16, 3: np.float32, 4: np.int32, 5: np.uint8, 6: np.uint16}
+
+
+class Checkpoint:
+    """Read-only view of a .gdckpt file (gd_checkpoint_*): directory entries, metadata, raw tensor bytes."""
+
+    def __init__(self, path):
+        self.handle = _vp()
+        st = lib().gd_checkpoint_open(os.fsencode(path), C.byref(self.handle))
+        if st != GD_OK:
+            self.handle = None
+            raise GdError(st, f"gd_checkpoint_open({path})")
+        self.path = path
+
+    def close(self):
+        if getattr(self, "handle", None):
+            lib().gd_checkpoint_close(self.handle)
+            self.handle = None
+
+    __del__ = close
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def __len__(self):
+        return lib().gd_checkpoint_count(self.handle)
+
+    def entries(self):
+        return [lib().gd_checkpoint_entry_at(self.handle, i).contents for i in range(len(self))]
+
+    def paths(self):
+        return [e.path.decode() for e in self.entries()]
+
+    def metadata(self):
+        blob, n = _vp(), C.c_size_t()
+        st = lib().gd_checkpoint_read_metadata(os.fsencode(self.path), C.byref(blob), C.byref(n))
+        if st != GD_OK:
+            raise GdError(st, "gd_checkpoint_read_metadata")
+        try:
+            return C.string_at(blob, n.value)
+        finally:
+            _libc_free(blob)
+
+    def read(self, path):
+        """The tensor stored under `path` as a numpy array (BF16 comes back as its uint16 bits)."""
+        p = lib().gd_checkpoint_find(self.handle, path.encode())
+        if not p:
+            raise KeyError(path)
+        e = p.contents
+        raw = np.empty(e.nbytes, np.uint8)
+        st = lib().gd_checkpoint_read(self.handle, p, 0, raw.ctypes.data_as(_vp), e.nbytes)
+        if st != GD_OK:
+            raise GdError(st, f"gd_checkpoint_read({path})")
+        dtype = np.uint16 if e.dtype == 2 else _CKPT_NUMPY[e.dtype]
+        return raw.view(dtype).reshape([e.shape[i] for i in range(e.rank)])
+
+
+def _libc_free(ptr):
+    libc = C.CDLL(None)
+    libc.free.argtypes = [_vp]
+    libc.free.restype = None
+    libc.free(ptr)

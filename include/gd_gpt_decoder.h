@@ -52,6 +52,23 @@ void gd_gpt_decoder_destroy(gd_gpt_decoder *dec);
  * b_qkv, w_attn, b_attn, w_upgate, b_upgate, w_down, b_down, k_cache, v_cache); NULL if unknown. */
 gd_tensor *gd_gpt_decoder_tensor(gd_gpt_decoder *dec, const char *name, int32_t layer);
 
+/* Replaces the weights with those of a checkpoint the reference wrote with gd_module_save_state for its
+ * gpt_lm example (".gdckpt"; container described in gd_checkpoint.h).  The counterpart of the
+ * reference's gd_module_load_state(ctx, &model.mod, path, {strict, load_buffers}) as its inference
+ * programs call it (examples/gpt_lm/infer.c:514-516; src/nn/module_io.c:826-940): tensors are matched
+ * by the paths gpt_lm_init registers ("gpt_lm.token_embedding", "gpt_lm.lm_head_bias",
+ * "gpt_lm.final_norm_w", "gpt_lm.blocks.<l>.{attn_norm_w, mlp_norm_w, qkv_proj.weight, qkv_proj.bias,
+ * attn_proj.weight, attn_proj.bias, up_gate.weight, up_gate.bias, down_proj.weight, down_proj.bias}")
+ * and every match must agree in dtype, rank, shape and byte count (GD_ERR_BAD_STATE otherwise).
+ * strict != 0: a parameter in the file the decoder does not have, or one the decoder has and the file
+ * lacks, is GD_ERR_BAD_STATE; strict == 0: both are skipped.  Buffer entries are ignored (the decoder
+ * registers none).  All checks run before the first byte is written, so a refused file leaves the
+ * weights untouched.  The reference ties the LM head to the embedding table; a decoder created with
+ * tie_lm_head = 0 receives the table in both places.  The [d_model, hidden] copy of each down
+ * projection is rebuilt from the loaded [hidden, d_model] weight.  GD_ERR_BUSY while a resident
+ * session is open; file errors as in gd_checkpoint_open.  Caches and positions are not touched. */
+gd_status gd_gpt_decoder_load_checkpoint(gd_gpt_decoder *dec, const char *path, int32_t strict);
+
 /* Host copy of the live length of every sequence ([batch]); writable (e.g. after filling caches). */
 int32_t *gd_gpt_decoder_positions(gd_gpt_decoder *dec);
 
@@ -78,7 +95,7 @@ gd_status gd_gpt_decoder_step(gd_gpt_decoder *dec, const int32_t *ids, int32_t *
  *   GD_GPT_RESIDENT_UNFUSED         issue the step through the public operators exactly like
  *                                   gd_gpt_decoder_step (about 40 launches for 3 layers).  Without
  *                                   it the step uses the fused backend entry points
- *                                   (gd_backend_fused_linear, gd_backend_qkv_rope_append: 6 launches
+ *                                   (gd_backend_fused_linear, gd_backend_qkv_rope_append: 5 launches
  *                                   per layer), which keep every rounding point of the separate
  *                                   operators. */
 #define GD_GPT_RESIDENT_HOLD_POSITIONS 1

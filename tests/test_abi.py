@@ -34,6 +34,23 @@ def test_library_exports_every_declared_symbol(gda):
     assert not missing, missing
 
 
+def test_library_exports_the_host_core_decoder_and_checkpoint_symbols(gda):
+    """Every function the other public headers declare (host core, decoder, checkpoint reader) is exported too;
+    functions defined in a header (static inline) are not library symbols."""
+    lib = ctypes.CDLL(gda.LIB_PATH)
+    for header in ("gradients_infer.h", "gd_gpt_decoder.h", "gd_checkpoint.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        text = re.sub(r"static inline[^{;]*\{.*?\n\}", "", text, flags=re.S)
+        text = "\n".join(l for l in text.splitlines() if not l.lstrip().startswith("#"))
+        names = sorted(set(re.findall(r"\b(gd_\w+)\s*\(", text)))
+        assert len(names) >= 7, header
+        missing = [n for n in names if not hasattr(lib, n)]
+        assert not missing, (header, missing)
+    for must in ("gd_gpt_decoder_load_checkpoint", "gd_checkpoint_read_metadata", "gd_checkpoint_open"):
+        assert hasattr(lib, must)
+
+
 def test_python_binding_covers_the_header(gda):
     assert set(_declared_symbols()) == set(gda.EXPORTED_SYMBOLS)
 

@@ -235,3 +235,63 @@ def test_decode_step_matches_packed_forward(gda, oracle):
     finally:
         a.close()
         b.close()
+
+
+def test_checkpoint_written_by_the_reference_reproduces_its_generation(gda):
+    """tests/golden/gpt_small_seed777.gdckpt was saved by the reference's gd_module_save_state from the model its
+    own generation code then ran (tests/golden/make_gdckpt_fixture.py; vocabulary 64, width 64, 2 heads of 32, MLP
+    128, context 64, 2 layers, window 0): a decoder created from ANOTHER seed, after loading the file, must give the
+    reference's logits (F16 read back as F32, absolute 4e-3 as for the reference-program tests) and its token ids
+    (near-ties excepted), stepwise and through the fused resident path; and every weight must hold the file's bytes."""
+    import os
+    from gradients_c_amd import decoder as D
+    golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    ckpt = os.path.join(golden, "gpt_small_seed777.gdckpt")
+    head = np.fromfile(os.path.join(golden, "gpt_small_seed777_in.bin"), np.int32)
+    B, new_tokens, layers = (int(v) for v in head[:3])
+    lens = head[3:3 + B]
+    prompt = head[3 + B:]
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    assert prompt.size == cu[-1]
+    out = np.fromfile(os.path.join(golden, "gpt_small_seed777_out.bin"), np.uint8)
+    ref_ids = out[:4 * new_tokens * B].view(np.int32).reshape(new_tokens, B)
+    ref_logits = out[4 * new_tokens * B:].view(np.float32).reshape(new_tokens, B, 64)
+
+    dev = D.GptDecoder(D.gpt_config(64, 64, layers, 2, 32, 128, 64, B, 0, True, 31337), max_prefill_tokens=int(cu[-1]))
+    try:
+        lg0, _, _ = dev.prefill(prompt, cu)
+        assert np.abs(ref_logits[0] - lg0.astype(np.float32)).max() > 0.05, "other seed, other model"
+        dev.positions[:] = 0
+        dev.load_checkpoint(ckpt)
+        with D.Checkpoint(ckpt) as ck:
+            for path, name, layer in (("gpt_lm.token_embedding", "embed", 0), ("gpt_lm.token_embedding", "lm_head", 0),
+                                      ("gpt_lm.blocks.1.up_gate.weight", "w_upgate", 1),
+                                      ("gpt_lm.blocks.0.qkv_proj.weight", "w_qkv", 0)):
+                assert np.array_equal(dev.read_tensor(name, layer).view(np.uint16).ravel(),
+                                      ck.read(path).view(np.uint16).ravel()), path
+            down = ck.read("gpt_lm.blocks.1.down_proj.weight")
+            assert np.array_equal(dev.read_tensor("w_down_t", 1).reshape(64, 128).view(np.uint16), down.T.view(np.uint16))
+        near = 0
+        for s in range(new_tokens):
+            lg, nx, gp = dev.prefill(prompt, cu) if s == 0 else dev.step(ref_ids[s - 1])
+            assert np.abs(ref_logits[s] - lg.astype(np.float32)).max() < 4e-3, s
+            for b in np.nonzero(nx != ref_ids[s])[0]:
+                assert gp[b] < 1e-3, f"step {s} row {b}: token differs and is not a near-tie"
+                near += 1
+        print("near-ties:", near)
+        # the fused resident path on the loaded weights (it reads the [d_model, hidden] copy of the down weight)
+        dev.positions[:] = 0
+        _, nx, _ = dev.prefill(prompt, cu)
+        ids, gaps, _ = dev.run_resident(ref_ids[0], new_tokens - 1)
+        for s in range(1, new_tokens):
+            for b in np.nonzero(ids[s - 1] != ref_ids[s])[0]:
+                assert gaps[s - 1][b] < 1e-3, f"resident step {s} row {b}"
+            if not np.array_equal(ids[s - 1], ref_ids[s]):
+                break  # after a near-tie the sequences legitimately part
+        # a load while a resident session is open is refused
+        dev.resident_begin(ref_ids[0], 2)
+        st = D.lib().gd_gpt_decoder_load_checkpoint(dev.handle, ckpt.encode(), 1)
+        dev.resident_end()
+        assert st == -4
+    finally:
+        dev.close()
