@@ -398,6 +398,88 @@ gd_status gd_gpt_decoder_load_checkpoint(gd_gpt_decoder *d, const char *path, in
     return st;
 }
 
+/* value of "key=value" on a line of its own in the metadata blob, as the reference's inference programs look it
+ * up (examples/gpt_lm/infer.c:344-376); false if absent or not a whole non-negative number that fits an int32 */
+static bool metadata_i32(const char *blob, size_t len, const char *key, int32_t *out)
+{
+    const size_t key_len = strlen(key);
+    size_t at = 0U;
+    while (at < len) {
+        size_t end = at;
+        while (end < len && blob[end] != '\n') ++end;
+        if (end > at + key_len && strncmp(blob + at, key, key_len) == 0 && blob[at + key_len] == '=') {
+            int64_t v = 0;
+            size_t i = at + key_len + 1U;
+            if (i == end) return false;
+            for (; i < end; ++i) {
+                if (blob[i] < '0' || blob[i] > '9') return false;
+                v = v * 10 + (blob[i] - '0');
+                if (v > INT32_MAX) return false;
+            }
+            *out = (int32_t)v;
+            return true;
+        }
+        at = end < len ? end + 1U : end;
+    }
+    return false;
+}
+
+gd_status gd_gpt_config_from_checkpoint(const char *path, gd_gpt_config *cfg)
+{
+    gd_checkpoint *ck = NULL;
+    const gd_checkpoint_entry *embed, *down;
+    char *blob = NULL;
+    size_t blob_len = 0U;
+    int32_t layers = 0, v;
+    uint32_t i;
+    gd_status st;
+    if (path == NULL || cfg == NULL) return GD_ERR_INVALID_ARGUMENT;
+    st = gd_checkpoint_open(path, &ck);
+    if (st != GD_OK) return st;
+    /* the directory fixes vocabulary, width, MLP width and depth */
+    embed = gd_checkpoint_find(ck, "gpt_lm.token_embedding");
+    down = gd_checkpoint_find(ck, "gpt_lm.blocks.0.down_proj.weight");
+    for (i = 0U; i < gd_checkpoint_count(ck); ++i) {
+        const char *p = gd_checkpoint_entry_at(ck, i)->path;
+        int n = -1, used = 0;
+        if (sscanf(p, "gpt_lm.blocks.%d.attn_norm_w%n", &n, &used) == 1 && used > 0 && p[used] == '\0' && n >= layers)
+            layers = n + 1;
+    }
+    if (embed == NULL || down == NULL || embed->rank != 2U || down->rank != 2U || layers <= 0 ||
+        embed->shape[0] > INT32_MAX || embed->shape[1] > INT32_MAX || down->shape[0] > INT32_MAX ||
+        down->shape[1] != embed->shape[1]) {
+        gd_checkpoint_close(ck);
+        return GD_ERR_BAD_STATE;
+    }
+    gd_checkpoint_close(ck);
+    cfg->vocab = (int32_t)embed->shape[0];
+    cfg->d_model = (int32_t)embed->shape[1];
+    cfg->mlp_hidden = (int32_t)down->shape[0];
+    cfg->n_layers = layers;
+    cfg->tie_lm_head = 1;
+    /* the metadata the reference's trainer writes (examples/gpt_lm/main.c:1836-1864) carries what shapes cannot
+     * tell; where it repeats what the directory fixes, the two must agree */
+    st = gd_checkpoint_read_metadata(path, &blob, &blob_len);
+    if (st != GD_OK) return st;
+    if ((metadata_i32(blob, blob_len, "vocab_size", &v) && v != cfg->vocab) ||
+        (metadata_i32(blob, blob_len, "d_model", &v) && v != cfg->d_model) ||
+        (metadata_i32(blob, blob_len, "mlp_hidden", &v) && v != cfg->mlp_hidden) ||
+        (metadata_i32(blob, blob_len, "n_layers", &v) && v != cfg->n_layers)) {
+        free(blob);
+        return GD_ERR_BAD_STATE;
+    }
+    if (metadata_i32(blob, blob_len, "n_heads", &v)) cfg->n_heads = v;
+    if (metadata_i32(blob, blob_len, "head_dim", &v)) cfg->head_dim = v;
+    if (metadata_i32(blob, blob_len, "sdpa_window", &v)) cfg->sdpa_window = v;
+    if (cfg->max_seq <= 0 && metadata_i32(blob, blob_len, "context_length", &v)) cfg->max_seq = v;
+    free(blob);
+    if (cfg->n_heads > 0 && cfg->head_dim <= 0 && cfg->d_model % cfg->n_heads == 0) cfg->head_dim = cfg->d_model / cfg->n_heads;
+    if (cfg->head_dim > 0 && cfg->n_heads <= 0 && cfg->d_model % cfg->head_dim == 0) cfg->n_heads = cfg->d_model / cfg->head_dim;
+    if (cfg->n_heads <= 0 || cfg->head_dim <= 0 || (int64_t)cfg->n_heads * cfg->head_dim != cfg->d_model)
+        return GD_ERR_BAD_STATE;
+    return GD_OK;
+}
+
 /* ---- forward pieces -------------------------------------------------------------------- */
 
 /* reference src/nn/module.c:1012-1028 */

@@ -129,6 +129,7 @@ def lib():
         l.gd_gpt_decoder_resident_sync.argtypes = [_vp]
         l.gd_gpt_decoder_resident_end.argtypes = [_vp, _vp, _vp, C.POINTER(C.c_int32)]
         l.gd_gpt_decoder_load_checkpoint.argtypes = [_vp, C.c_char_p, C.c_int32]
+        l.gd_gpt_config_from_checkpoint.argtypes = [C.c_char_p, C.POINTER(GptConfig)]
         l.gd_checkpoint_read_metadata.argtypes = [C.c_char_p, C.POINTER(_vp), C.POINTER(C.c_size_t)]
         l.gd_checkpoint_open.argtypes = [C.c_char_p, C.POINTER(_vp)]
         l.gd_checkpoint_close.argtypes = [_vp]
@@ -205,6 +206,15 @@ def gpt_config(vocab, d_model, n_layers, n_heads, head_dim, mlp_hidden, max_seq,
                seed=1000):
     return GptConfig(vocab, d_model, n_layers, n_heads, head_dim, mlp_hidden, max_seq, batch, window,
                      int(tie_lm_head), 1e-5, 10000.0, seed)
+
+
+def config_from_checkpoint(path, batch, max_seq=0, n_heads=0, head_dim=0, window=0, seed=1000):
+    """gd_gpt_config for the model stored in a .gdckpt file; the keyword values are used where the file is silent."""
+    cfg = GptConfig(0, 0, 0, n_heads, head_dim, 0, max_seq, batch, window, 1, 1e-5, 10000.0, seed)
+    st = lib().gd_gpt_config_from_checkpoint(os.fsencode(path), C.byref(cfg))
+    if st != GD_OK:
+        raise GdError(st, f"gd_gpt_config_from_checkpoint({path})")
+    return cfg
 
 
 class GptDecoder:

@@ -320,3 +320,65 @@ def test_loader_strictness_and_untouched_weights_on_refusal(host, raw, tmp_path)
         expect_refused(dev, bf16)
     finally:
         dev.close()
+
+
+# ---- model dimensions from the file ------------------------------------------------------------------------------
+
+def with_metadata(raw, blob):
+    """The fixture with another metadata blob: the data section moves, so every directory entry's offset and the
+    header's data offset move with it (test-side rewrite of the container, independent of the C reader)."""
+    info = parse(raw)
+    data = bytearray(raw[:info["meta_off"]]) + blob
+    new_data_off = (len(data) + 255) // 256 * 256
+    data += bytes(new_data_off - len(data)) + raw[info["data_off"]:]
+    delta = new_data_off - info["data_off"]
+    struct.pack_into("<Q", data, 48, len(blob))
+    struct.pack_into("<Q", data, 56, new_data_off)
+    for e in info["entries"]:
+        struct.pack_into("<Q", data, e["at"] + 80, e["offset"] + delta)
+    return bytes(data)
+
+
+TRAINER_METADATA = (b"model=gpt_lm\nvocab_size=64\ncontext_length=64\nd_model=64\nn_layers=2\nn_heads=2\nhead_dim=32\n"
+                    b"mlp_hidden=128\nffn_activation=swiglu\narchitecture=gpt\nsdpa_window=16\ndropout=0.1\n"
+                    b"logits_softcap=20\ntokenizer_path=data/tokenizer-v2048.json\n")
+
+
+def test_config_from_checkpoint(host, raw, tmp_path):
+    pkg, D = host
+    # the fixture's own metadata has no key=value lines: heads come from the caller
+    cfg = D.config_from_checkpoint(CKPT, batch=2, max_seq=48, n_heads=2)
+    assert (cfg.vocab, cfg.d_model, cfg.n_layers, cfg.n_heads, cfg.head_dim, cfg.mlp_hidden) == (64, 64, 2, 2, 32, 128)
+    assert (cfg.max_seq, cfg.batch, cfg.sdpa_window, cfg.tie_lm_head) == (48, 2, 0, 1)
+    assert D.config_from_checkpoint(CKPT, batch=1, max_seq=8, head_dim=16).n_heads == 4
+    for bad in (dict(), dict(n_heads=3), dict(n_heads=2, head_dim=16)):
+        with pytest.raises(pkg.GdError) as err:
+            D.config_from_checkpoint(CKPT, batch=2, max_seq=48, **bad)
+        assert err.value.status == GD_ERR_BAD_STATE
+    # with the metadata the reference's trainer writes, the file alone is enough
+    p = tmp_path / "trainer.gdckpt"
+    p.write_bytes(with_metadata(raw, TRAINER_METADATA))
+    with D.Checkpoint(str(p)) as ck:
+        assert ck.metadata() == TRAINER_METADATA
+        assert ck.read("gpt_lm.blocks.1.down_proj.bias").tobytes() == D.Checkpoint(CKPT).read(
+            "gpt_lm.blocks.1.down_proj.bias").tobytes()
+    cfg = D.config_from_checkpoint(str(p), batch=3)
+    assert (cfg.vocab, cfg.d_model, cfg.n_layers, cfg.n_heads, cfg.head_dim, cfg.mlp_hidden) == (64, 64, 2, 2, 32, 128)
+    assert (cfg.max_seq, cfg.batch, cfg.sdpa_window) == (64, 3, 16)
+    assert D.config_from_checkpoint(str(p), batch=3, max_seq=32).max_seq == 32
+    dev = D.GptDecoder(cfg)
+    try:
+        dev.load_checkpoint(str(p))
+    finally:
+        dev.close()
+    # metadata that contradicts the directory
+    for key, value in ((b"d_model=64", b"d_model=96"), (b"n_layers=2", b"n_layers=3"), (b"vocab_size=64", b"vocab_size=65"),
+                       (b"mlp_hidden=128", b"mlp_hidden=64"), (b"n_heads=2", b"n_heads=3")):
+        q = tmp_path / "contradiction.gdckpt"
+        q.write_bytes(with_metadata(raw, TRAINER_METADATA.replace(key, value)))
+        with pytest.raises(pkg.GdError) as err:
+            D.config_from_checkpoint(str(q), batch=1)
+        assert err.value.status == GD_ERR_BAD_STATE, key
+    with pytest.raises(pkg.GdError) as err:
+        D.config_from_checkpoint(str(tmp_path / "absent.gdckpt"), batch=1)
+    assert err.value.status == GD_ERR_IO
