@@ -79,6 +79,17 @@ class FusedLinearArgs(C.Structure):
                 ("epilogue", C.c_uint32)]
 
 
+class SampleArgs(C.Structure):  # gd_backend_sample_args
+    _fields_ = [("temperature", C.c_float), ("min_p", C.c_float), ("repetition_penalty", C.c_float),
+                ("logits_softcap", C.c_float), ("stop_token", C.c_int32), ("pos_delta", C.c_int32)]
+
+
+class SampleTensors(C.Structure):  # gd_backend_sample_tensors
+    _names = ("history", "hist_len", "finished", "state", "work", "ids", "positions", "step_counters", "out_ids",
+              "table", "next_x")
+    _fields_ = [(n, C.POINTER(TensorView)) for n in _names]
+
+
 class ConcatArgs(C.Structure):
     _fields_ = [("count", C.c_uint64), ("inner", C.c_uint64), ("slice_axis", C.c_uint64), ("full_axis", C.c_uint64),
                 ("axis_offset", C.c_uint64)]
@@ -142,6 +153,7 @@ _SIGNATURES = {
     "gd_backend_fused_qkv_rope_append": [_vp, _MV, _MV, _VV, _VV, _TV, _TV, _TV, _TV, _TV, C.c_uint32, C.c_uint32,
                                          C.POINTER(RopeArgs), C.POINTER(FusedLinearArgs)],
     "gd_backend_argmax_advance": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, C.c_int32, _TV, _TV],
+    "gd_backend_sample_advance": [_vp, _TV, C.POINTER(SampleTensors), C.POINTER(SampleArgs)],
     "gd_backend_copy": [_vp, _vp, C.c_size_t, _vp, C.c_size_t, C.c_size_t],
     "gd_backend_timer_create": [_vp, C.POINTER(_vp)],
     "gd_backend_timer_start": [_vp],
@@ -165,6 +177,7 @@ _OTHER_RESTYPE = {
     "gd_backend_fence_destroy": (None, [C.POINTER(Fence)]),
     "gd_backend_fence_is_complete": (C.c_bool, [C.POINTER(Fence)]),
     "gd_backend_timer_destroy": (None, [_vp]),
+    "gd_backend_sample_state_count": (C.c_size_t, [C.c_uint32]),
     "gd_backend_graph_destroy": (None, [_vp]),
 }
 EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + list(_OTHER_RESTYPE))
@@ -482,6 +495,15 @@ class Backend:
     def argmax_rows(self, logits, ids, gap=None):
         _check(self.call("gd_backend_argmax_rows", logits.view(), ids.view(), gap.view() if gap else None),
                "gd_backend_argmax_rows")
+
+    def sample_advance(self, logits, tensors, temperature, min_p=0.0, repetition_penalty=1.0, logits_softcap=0.0,
+                       stop_token=-1, pos_delta=1):
+        """tensors: dict of Tensor by the field names of gd_backend_sample_tensors (table / next_x optional)."""
+        views = {n: tensors[n].view() for n in SampleTensors._names if tensors.get(n) is not None}
+        t = SampleTensors(**{n: C.pointer(v) for n, v in views.items()})
+        a = SampleArgs(temperature, min_p, repetition_penalty, logits_softcap, stop_token, pos_delta)
+        st = self.call("gd_backend_sample_advance", logits.view(), C.byref(t), C.byref(a))
+        _check(st, "gd_backend_sample_advance")
 
     def gather_rows(self, src, rows, out):
         _check(self.call("gd_backend_gather_rows", src.view(), rows.view(), out.view()), "gd_backend_gather_rows")

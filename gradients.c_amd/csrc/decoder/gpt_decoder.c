@@ -51,6 +51,12 @@ struct gd_gpt_decoder {
     int32_t resident_max_steps, resident_steps, resident_hold, resident_unfused;
     gd_backend_graph *resident_graph;
     gd_tensor resident_out_ids, resident_out_gaps;
+    /* sampling front end (state arena): what the reference's generation loop keeps on the host */
+    gd_tensor last_logits;                 /* [B, V] F16: logits of the last packed prefill */
+    gd_tensor history, hist_len, finished; /* [B, max_seq], [B], [B] I32 */
+    gd_tensor sample_state, sample_work;   /* generator + per-row records; [B*V] F32 */
+    bool resident_sampling;
+    gd_gpt_sampling sampling;
 };
 
 /* ---- deterministic initialisation (reference :32-48, 196-218) ----------------------- */
@@ -152,8 +158,11 @@ size_t gd_gpt_params_bytes(const gd_gpt_config *c)
 size_t gd_gpt_state_bytes(const gd_gpt_config *c)
 {
     const size_t cache = pad256((size_t)c->batch * (size_t)c->max_seq * (size_t)c->n_heads * (size_t)c->head_dim * 2U);
+    const size_t B = (size_t)c->batch, V = (size_t)c->vocab;
+    const size_t sampling = pad256(B * V * 2U) + pad256(B * V * 4U) + pad256(B * (size_t)c->max_seq * 4U) +
+                            2U * pad256(B * 4U) + pad256((8U + 8U * B) * 4U);
     return cache * 2U * (size_t)c->n_layers + 4U * pad256((size_t)c->batch * 4U) +
-           pad256((size_t)c->batch * (size_t)c->d_model * 2U) + 4096U;
+           pad256((size_t)c->batch * (size_t)c->d_model * 2U) + sampling + 4096U;
 }
 
 gd_status gd_gpt_decoder_create(gd_context *ctx, const gd_gpt_config *cfg, gd_gpt_decoder **out)
@@ -226,6 +235,16 @@ gd_status gd_gpt_decoder_create(gd_context *ctx, const gd_gpt_config *cfg, gd_gp
     {
         int64_t xdim[2] = {cfg->batch, cfg->d_model};
         STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_F16, gd_shape_make(2U, xdim), 256U, &d->x0_dev));
+    }
+    {
+        int64_t ldim[2] = {cfg->batch, cfg->vocab}, hdim[2] = {cfg->batch, cfg->max_seq};
+        int64_t sdim[1] = {8 + 8 * (int64_t)cfg->batch}, wdim[1] = {(int64_t)cfg->batch * cfg->vocab};
+        STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_F16, gd_shape_make(2U, ldim), 256U, &d->last_logits));
+        STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_I32, gd_shape_make(2U, hdim), 256U, &d->history));
+        STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_I32, gd_shape_make(1U, bdim), 256U, &d->hist_len));
+        STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_I32, gd_shape_make(1U, bdim), 256U, &d->finished));
+        STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_I32, gd_shape_make(1U, sdim), 256U, &d->sample_state));
+        STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_F32, gd_shape_make(1U, wdim), 256U, &d->sample_work));
     }
 #undef STEP
     if (st != GD_OK) {
@@ -667,6 +686,12 @@ gd_status gd_gpt_decoder_prefill(gd_gpt_decoder *d, const int32_t *ids, const in
         }
         if (st == GD_OK) st = gd_gather_rows(ctx, &x, &t_last, &last_hidden);
         if (st == GD_OK) st = head(d, &last_hidden, &t_logits, &t_next, &t_gaps);
+        /* the sampling front end starts from these logits without a round trip through the host */
+        if (st == GD_OK)
+            st = gd_backend_copy(gd_context_backend(ctx), (gd_backend_buffer *)d->last_logits.storage.buffer,
+                                 d->last_logits.storage.offset + d->last_logits.view_offset,
+                                 (gd_backend_buffer *)t_logits.storage.buffer,
+                                 t_logits.storage.offset + t_logits.view_offset, (size_t)B * (size_t)d->cfg.vocab * 2U);
         if (st == GD_OK) {
             for (b = 0; b < B; ++b) d->pos[b] = cu[b + 1] - cu[b];
             st = gd_end_step(ctx);
@@ -848,12 +873,66 @@ static gd_status enqueue_fused_step(gd_gpt_decoder *d, gd_tensor *logits)
     return GD_OK;
 }
 
+/* sampled pick instead of the greedy one: token, history, finished flags, feedback and records in two launches */
+static gd_status enqueue_sample(gd_gpt_decoder *d, const gd_tensor *logits, int32_t pos_delta)
+{
+    gd_backend_tensor_view vl, vh, vhl, vf, vst, vw, vi, vp, vs, vo, vt, vx;
+    gd_backend_sample_tensors t;
+    gd_backend_sample_args a;
+    tview(logits, &vl);
+    tview(&d->history, &vh);
+    view1(&d->hist_len, &vhl);
+    view1(&d->finished, &vf);
+    view1(&d->sample_state, &vst);
+    view1(&d->sample_work, &vw);
+    view1(&d->ids_dev, &vi);
+    view1(&d->pos_dev, &vp);
+    view1(&d->step_rows_dev, &vs);
+    view1(&d->resident_out_ids, &vo);
+    memset(&t, 0, sizeof(t));
+    t.history = &vh;
+    t.hist_len = &vhl;
+    t.finished = &vf;
+    t.state = &vst;
+    t.work = &vw;
+    t.ids = &vi;
+    t.positions = &vp;
+    t.step_counters = &vs;
+    t.out_ids = &vo;
+    if (d->resident_x0) {
+        tview(&d->token_embedding, &vt);
+        tview(&d->x0_dev, &vx);
+        t.table = &vt;
+        t.next_x = &vx;
+    }
+    a.temperature = d->sampling.temperature;
+    a.min_p = d->sampling.min_p;
+    a.repetition_penalty = d->sampling.repetition_penalty;
+    a.logits_softcap = d->sampling.logits_softcap;
+    a.stop_token = d->sampling.stop_token;
+    a.pos_delta = pos_delta;
+    return gd_backend_sample_advance(gd_context_backend(d->ctx), &vl, &t, &a);
+}
+
 static gd_status enqueue_resident_step(gd_gpt_decoder *d)
 {
     gd_context *ctx = d->ctx;
     gd_tensor x, y, logits, next, gaps;
     gd_backend_tensor_view vn, vg, vi, vp, vs, vo, vog;
     int32_t l;
+    if (d->resident_sampling) {
+        if (d->resident_unfused) {
+            TRY(gd_embedding(ctx, &d->token_embedding, &d->ids_dev, &x));
+            for (l = 0; l < d->cfg.n_layers; ++l) {
+                TRY(block_decode(d, l, &x, &d->pos_dev, &d->pos_dev, &y));
+                x = y;
+            }
+            TRY(head(d, &x, &logits, &next, &gaps));
+        } else {
+            TRY(enqueue_fused_step(d, &logits));
+        }
+        return enqueue_sample(d, &logits, 1);
+    }
     if (d->resident_unfused) {
         TRY(gd_embedding(ctx, &d->token_embedding, &d->ids_dev, &x));
         for (l = 0; l < d->cfg.n_layers; ++l) {
@@ -898,10 +977,14 @@ static void resident_abort(gd_gpt_decoder *d)
     if (d->resident_graph != NULL) gd_backend_graph_destroy(d->resident_graph);
     d->resident_graph = NULL;
     d->resident_open = false;
+    d->resident_sampling = false;
 }
 
-gd_status gd_gpt_decoder_resident_begin(gd_gpt_decoder *d, const int32_t *first_ids, int32_t max_steps,
-                                        int32_t flags)
+/* sampling == NULL: greedy session that starts from first_ids.  Otherwise: the session starts from the logits the
+ * last prefill left in last_logits; max_steps counts picks (the one on those logits included), so at most
+ * max_steps - 1 decode steps run; history / hist_len / finished / sample_state were set by the caller. */
+static gd_status resident_begin_impl(gd_gpt_decoder *d, const int32_t *first_ids, int32_t max_steps, int32_t flags,
+                                     const gd_gpt_sampling *sampling)
 {
     const int32_t hold_positions = flags & GD_GPT_RESIDENT_HOLD_POSITIONS;
     gd_context *ctx;
@@ -909,14 +992,17 @@ gd_status gd_gpt_decoder_resident_begin(gd_gpt_decoder *d, const int32_t *first_
     gd_status st;
     int64_t dims[1];
     int32_t b, zero = 0;
-    if (d == NULL || first_ids == NULL || max_steps <= 0) return GD_ERR_INVALID_ARGUMENT;
+    if (d == NULL || (first_ids == NULL && sampling == NULL) || max_steps <= 0) return GD_ERR_INVALID_ARGUMENT;
     if (d->resident_open) return GD_ERR_BAD_STATE;
     ctx = d->ctx;
     be = gd_context_backend(ctx);
     for (b = 0; b < d->cfg.batch; ++b) {
-        if (d->pos[b] < 0 || d->pos[b] + (hold_positions ? 1 : max_steps) > d->cfg.max_seq) return GD_ERR_INVALID_ARGUMENT;
+        /* a sampled session may run past the end of a cache: such rows have ended (their history is full), their
+         * appends are skipped and their results ignored, as in the reference's loop */
+        if (d->pos[b] < 0 || (sampling == NULL && d->pos[b] + (hold_positions ? 1 : max_steps) > d->cfg.max_seq))
+            return GD_ERR_INVALID_ARGUMENT;
     }
-    TRY(gd_tensor_write(ctx, &d->ids_dev, first_ids, (size_t)d->cfg.batch * sizeof(int32_t)));
+    if (sampling == NULL) TRY(gd_tensor_write(ctx, &d->ids_dev, first_ids, (size_t)d->cfg.batch * sizeof(int32_t)));
     TRY(gd_tensor_write(ctx, &d->pos_dev, d->pos, (size_t)d->cfg.batch * sizeof(int32_t)));
     TRY(gd_tensor_write(ctx, &d->step_dev, &zero, sizeof(zero)));
     TRY(gd_tensor_zero_(ctx, &d->step_rows_dev));
@@ -926,14 +1012,20 @@ gd_status gd_gpt_decoder_resident_begin(gd_gpt_decoder *d, const int32_t *first_
     d->resident_max_steps = max_steps;
     d->resident_steps = 0;
     d->resident_hold = hold_positions != 0;
+    d->resident_sampling = sampling != NULL;
+    if (sampling != NULL) d->sampling = *sampling;
     /* the fused rope + append kernel needs NeoX pairs of a head size that is a multiple of 16 */
     d->resident_unfused = (flags & GD_GPT_RESIDENT_UNFUSED) != 0 || (d->cfg.head_dim % 16) != 0;
     dims[0] = (int64_t)max_steps * d->cfg.batch;
     st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_I32, gd_shape_make(1U, dims), 256U, &d->resident_out_ids);
     if (st == GD_OK) st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F32, gd_shape_make(1U, dims), 256U, &d->resident_out_gaps);
-    /* fused step: the greedy-pick kernel leaves the next input rows in x0_dev; the first ones are gathered here */
+    /* fused step: the pick kernel leaves the next input rows in x0_dev; the first ones are gathered here */
     d->resident_x0 = !d->resident_unfused && (d->cfg.d_model % 8) == 0;
-    if (st == GD_OK && d->resident_x0) {
+    if (sampling != NULL) {
+        /* pick number 0, on the prefill's logits: positions stay, the token becomes the first step's input */
+        if (st == GD_OK) st = enqueue_sample(d, &d->last_logits, 0);
+        max_steps -= 1; /* decode steps from here on */
+    } else if (st == GD_OK && d->resident_x0) {
         gd_backend_tensor_view vt, vi, vx;
         gd_backend_embedding_args ea;
         tview(&d->token_embedding, &vt);
@@ -945,8 +1037,10 @@ gd_status gd_gpt_decoder_resident_begin(gd_gpt_decoder *d, const int32_t *first_
         st = gd_backend_embedding_forward(be, &vt, &vi, &vx, &ea);
     }
     /* the first step runs eagerly (it also sizes the attention workspace); later steps replay a graph */
-    if (st == GD_OK) st = enqueue_resident_step(d);
-    if (st == GD_OK) d->resident_steps = 1;
+    if (st == GD_OK && max_steps > 0) {
+        st = enqueue_resident_step(d);
+        if (st == GD_OK) d->resident_steps = 1;
+    }
     if (st == GD_OK && max_steps > 1) {
         st = gd_backend_graph_begin_capture(be);
         if (st == GD_OK) {
@@ -959,13 +1053,21 @@ gd_status gd_gpt_decoder_resident_begin(gd_gpt_decoder *d, const int32_t *first_
     return st;
 }
 
+gd_status gd_gpt_decoder_resident_begin(gd_gpt_decoder *d, const int32_t *first_ids, int32_t max_steps,
+                                        int32_t flags)
+{
+    if (first_ids == NULL) return GD_ERR_INVALID_ARGUMENT;
+    return resident_begin_impl(d, first_ids, max_steps, flags, NULL);
+}
+
 gd_status gd_gpt_decoder_resident_run(gd_gpt_decoder *d, int32_t n_steps)
 {
     gd_backend *be;
     int32_t s;
     if (d == NULL || n_steps < 0) return GD_ERR_INVALID_ARGUMENT;
     if (!d->resident_open) return GD_ERR_BAD_STATE;
-    if (d->resident_steps + n_steps > d->resident_max_steps) return GD_ERR_INVALID_ARGUMENT;
+    if (d->resident_steps + n_steps > d->resident_max_steps - (d->resident_sampling ? 1 : 0)) return GD_ERR_INVALID_ARGUMENT;
+    if (n_steps > 0 && d->resident_graph == NULL) return GD_ERR_BAD_STATE;
     be = gd_context_backend(d->ctx);
     for (s = 0; s < n_steps; ++s) {
         TRY(gd_backend_graph_launch(be, d->resident_graph));
@@ -985,26 +1087,133 @@ gd_status gd_gpt_decoder_resident_end(gd_gpt_decoder *d, int32_t *out_ids, float
     gd_context *ctx;
     gd_status st;
     gd_tensor ids_view, gaps_view;
-    int32_t b;
+    int32_t b, records;
     if (d == NULL) return GD_ERR_INVALID_ARGUMENT;
     if (!d->resident_open) return GD_ERR_BAD_STATE;
     ctx = d->ctx;
     st = gd_end_step(ctx);
+    /* a sampled session has one record more than decode steps: the pick on the prefill's logits */
+    records = d->resident_steps + (d->resident_sampling ? 1 : 0);
     if (st == GD_OK && out_ids != NULL) {
-        st = gd_tensor_slice(ctx, &d->resident_out_ids, 0U, 0, (int64_t)d->resident_steps * d->cfg.batch, &ids_view);
-        if (st == GD_OK) st = gd_tensor_read(ctx, &ids_view, out_ids, (size_t)d->resident_steps * (size_t)d->cfg.batch * sizeof(int32_t));
+        st = gd_tensor_slice(ctx, &d->resident_out_ids, 0U, 0, (int64_t)records * d->cfg.batch, &ids_view);
+        if (st == GD_OK) st = gd_tensor_read(ctx, &ids_view, out_ids, (size_t)records * (size_t)d->cfg.batch * sizeof(int32_t));
     }
-    if (st == GD_OK && out_gaps != NULL) {
+    if (st == GD_OK && out_gaps != NULL && !d->resident_sampling) {
         st = gd_tensor_slice(ctx, &d->resident_out_gaps, 0U, 0, (int64_t)d->resident_steps * d->cfg.batch, &gaps_view);
         if (st == GD_OK) st = gd_tensor_read(ctx, &gaps_view, out_gaps, (size_t)d->resident_steps * (size_t)d->cfg.batch * sizeof(float));
     }
     if (d->resident_graph != NULL) gd_backend_graph_destroy(d->resident_graph);
     d->resident_graph = NULL;
     d->resident_open = false;
-    if (steps_done != NULL) *steps_done = d->resident_steps;
+    d->resident_sampling = false;
+    if (steps_done != NULL) *steps_done = records;
     if (st == GD_OK && !d->resident_hold) {
         for (b = 0; b < d->cfg.batch; ++b) d->pos[b] += d->resident_steps;
     }
+    return st;
+}
+
+/* ---- generation with the sampling front end ---------------------------------------------- */
+
+uint64_t gd_gpt_generation_rng(uint64_t seed, int32_t n_prompts, uint64_t step)
+{
+    return splitmix64(seed ^ UINT64_C(0xdec0de1234567890) ^ (uint64_t)n_prompts ^ step);
+}
+
+gd_status gd_gpt_decoder_generate(gd_gpt_decoder *d, const int32_t *ids, const int32_t *cu, int32_t max_new,
+                                  const gd_gpt_sampling *sampling, int32_t *out_tokens, int32_t *out_counts)
+{
+    const int32_t check_every = 32; /* decode steps between two looks at the finished flags */
+    gd_context *ctx;
+    int32_t *packed = NULL, *pcu = NULL, *hist = NULL, *lens = NULL, *records = NULL, *flags = NULL;
+    int32_t state_words[8];
+    int32_t B, ctx_len, room, b, total = 0, done = 0, decode_steps;
+    gd_status st;
+    if (d == NULL || ids == NULL || cu == NULL || sampling == NULL || out_tokens == NULL || out_counts == NULL ||
+        max_new <= 0)
+        return GD_ERR_INVALID_ARGUMENT;
+    if (d->resident_open) return GD_ERR_BUSY;
+    ctx = d->ctx;
+    B = d->cfg.batch;
+    ctx_len = d->cfg.max_seq;
+    if (sampling->stop_token >= d->cfg.vocab || cu[0] != 0) return GD_ERR_INVALID_ARGUMENT;
+    /* reference :1514-1518: the prompt may use what the new tokens leave of the context, at least one row short of it */
+    room = max_new >= ctx_len ? ctx_len - 1 : ctx_len - max_new;
+    if (room <= 0) return GD_ERR_INVALID_ARGUMENT;
+    for (b = 0; b < B; ++b) {
+        if (cu[b + 1] <= cu[b]) return GD_ERR_INVALID_ARGUMENT; /* empty prompt (:1520-1522) */
+    }
+    pcu = (int32_t *)calloc((size_t)B + 1U, sizeof(int32_t));
+    lens = (int32_t *)calloc((size_t)B, sizeof(int32_t));
+    hist = (int32_t *)calloc((size_t)B * (size_t)ctx_len, sizeof(int32_t));
+    flags = (int32_t *)calloc((size_t)B, sizeof(int32_t));
+    records = (int32_t *)malloc((size_t)max_new * (size_t)B * sizeof(int32_t));
+    if (pcu == NULL || lens == NULL || hist == NULL || flags == NULL || records == NULL) {
+        st = GD_ERR_OUT_OF_MEMORY;
+        goto out;
+    }
+    /* a prompt longer than the room keeps its last tokens (:1523-1533) */
+    for (b = 0; b < B; ++b) {
+        const int32_t n = cu[b + 1] - cu[b];
+        lens[b] = n > room ? room : n;
+        pcu[b + 1] = pcu[b] + lens[b];
+    }
+    total = pcu[B];
+    packed = (int32_t *)malloc((size_t)total * sizeof(int32_t));
+    if (packed == NULL) {
+        st = GD_ERR_OUT_OF_MEMORY;
+        goto out;
+    }
+    for (b = 0; b < B; ++b) {
+        const int32_t *src = ids + cu[b + 1] - lens[b];
+        memcpy(packed + pcu[b], src, (size_t)lens[b] * sizeof(int32_t));
+        memcpy(hist + (size_t)b * (size_t)ctx_len, src, (size_t)lens[b] * sizeof(int32_t));
+    }
+    st = gd_gpt_decoder_prefill(d, packed, pcu, NULL, NULL, NULL); /* leaves the logits in last_logits */
+    if (st != GD_OK) goto out;
+    memset(state_words, 0, sizeof(state_words));
+    memcpy(&state_words[0], &sampling->rng_state, sizeof(uint64_t));
+    memcpy(&state_words[2], &sampling->rng_state, sizeof(uint64_t));
+    {
+        gd_tensor head_words;
+        st = gd_tensor_slice(ctx, &d->sample_state, 0U, 0, 8, &head_words);
+        if (st == GD_OK) st = gd_tensor_write(ctx, &head_words, state_words, sizeof(state_words));
+    }
+    if (st == GD_OK) st = gd_tensor_write(ctx, &d->history, hist, (size_t)B * (size_t)ctx_len * sizeof(int32_t));
+    if (st == GD_OK) st = gd_tensor_write(ctx, &d->hist_len, lens, (size_t)B * sizeof(int32_t));
+    if (st == GD_OK) st = gd_tensor_zero_(ctx, &d->finished);
+    if (st == GD_OK) st = resident_begin_impl(d, NULL, max_new, 0, sampling);
+    if (st != GD_OK) goto out;
+    /* the reference leaves its loop when every row has ended (:1607, 1634-1636): look at the flags now and then */
+    decode_steps = max_new - 1;
+    while (d->resident_steps < decode_steps) {
+        int32_t n = decode_steps - d->resident_steps, alive = 0;
+        if (n > check_every) n = check_every;
+        st = gd_gpt_decoder_resident_run(d, n);
+        if (st == GD_OK && d->resident_steps < decode_steps) {
+            st = gd_tensor_read(ctx, &d->finished, flags, (size_t)B * sizeof(int32_t));
+            for (b = 0; b < B; ++b) alive += flags[b] == 0;
+        } else {
+            alive = 1;
+        }
+        if (st != GD_OK) {
+            resident_abort(d);
+            goto out;
+        }
+        if (alive == 0) break;
+    }
+    st = gd_gpt_decoder_resident_end(d, records, NULL, &done);
+    if (st != GD_OK) goto out;
+    for (b = 0; b < B; ++b) {
+        int32_t s, n = 0;
+        for (s = 0; s < done; ++s) {
+            const int32_t token = records[(size_t)s * (size_t)B + (size_t)b];
+            if (token >= 0) out_tokens[(size_t)b * (size_t)max_new + (size_t)n++] = token;
+        }
+        out_counts[b] = n;
+    }
+out:
+    free(packed); free(pcu); free(hist); free(lens); free(records); free(flags);
     return st;
 }
 

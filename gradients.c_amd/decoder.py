@@ -49,6 +49,11 @@ def make_shape(dims):
 _T = C.POINTER(GdTensor)
 
 
+class GptSampling(C.Structure):  # gd_gpt_sampling
+    _fields_ = [("temperature", C.c_float), ("min_p", C.c_float), ("repetition_penalty", C.c_float),
+                ("logits_softcap", C.c_float), ("stop_token", C.c_int32), ("rng_state", C.c_uint64)]
+
+
 class CheckpointEntry(C.Structure):  # gd_checkpoint_entry
     _fields_ = [("path", C.c_char * 256), ("flags", C.c_uint32), ("dtype", C.c_int), ("rank", C.c_uint32),
                 ("shape", C.c_int64 * 8), ("data_offset", C.c_uint64), ("nbytes", C.c_uint64)]
@@ -129,6 +134,9 @@ def lib():
         l.gd_gpt_decoder_resident_sync.argtypes = [_vp]
         l.gd_gpt_decoder_resident_end.argtypes = [_vp, _vp, _vp, C.POINTER(C.c_int32)]
         l.gd_gpt_decoder_load_checkpoint.argtypes = [_vp, C.c_char_p, C.c_int32]
+        l.gd_gpt_decoder_generate.argtypes = [_vp, _vp, _vp, C.c_int32, C.POINTER(GptSampling), _vp, _vp]
+        l.gd_gpt_generation_rng.argtypes = [C.c_uint64, C.c_int32, C.c_uint64]
+        l.gd_gpt_generation_rng.restype = C.c_uint64
         l.gd_gpt_config_from_checkpoint.argtypes = [C.c_char_p, C.POINTER(GptConfig)]
         l.gd_checkpoint_read_metadata.argtypes = [C.c_char_p, C.POINTER(_vp), C.POINTER(C.c_size_t)]
         l.gd_checkpoint_open.argtypes = [C.c_char_p, C.POINTER(_vp)]
@@ -306,6 +314,18 @@ class GptDecoder:
                                                ids.ctypes.data_as(_vp), gaps.ctypes.data_as(_vp), C.byref(ms))
         self.ctx.check(st, "gd_gpt_decoder_run_resident")
         return ids, gaps, ms.value
+
+    def generate(self, ids, cu, max_new, temperature=0.0, min_p=0.0, repetition_penalty=1.0, logits_softcap=0.0,
+                 stop_token=-1, rng_state=0):
+        """Packed prompts in, new tokens out (list of one int32 array per batch row): gd_gpt_decoder_generate."""
+        ids, cu = np.ascontiguousarray(ids, np.int32), np.ascontiguousarray(cu, np.int32)
+        s = GptSampling(temperature, min_p, repetition_penalty, logits_softcap, stop_token, rng_state)
+        out = np.full((self.cfg.batch, max_new), -1, np.int32)
+        counts = np.zeros(self.cfg.batch, np.int32)
+        st = lib().gd_gpt_decoder_generate(self.handle, ids.ctypes.data_as(_vp), cu.ctypes.data_as(_vp), max_new,
+                                           C.byref(s), out.ctypes.data_as(_vp), counts.ctypes.data_as(_vp))
+        self.ctx.check(st, "gd_gpt_decoder_generate")
+        return [out[b, :counts[b]].copy() for b in range(self.cfg.batch)]
 
     def resident_begin(self, first_ids, max_steps, hold_positions=False, unfused=False):
         first = np.ascontiguousarray(first_ids, np.int32)

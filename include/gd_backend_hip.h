@@ -419,6 +419,56 @@ gd_status gd_backend_argmax_advance(gd_backend *backend, const gd_backend_tensor
                                     int32_t pos_delta, const gd_backend_tensor_view *table,
                                     const gd_backend_tensor_view *next_x);
 
+/* Next-token sampling and the bookkeeping of a generation loop on the device, two launches.  What the
+ * reference's example does on the host with the downloaded logits (examples/gpt_lm/gpt_lm_shared.c):
+ * soft cap (:1322-1331), repetition penalty over the row's history (:1347-1369), the temperature / min-p draw
+ * (:1371-1442) and the loop's handling of the result (:1586-1600, 1606-1680).  Per row b of logits [B, V]
+ * (F16 or F32, V <= 262144), rows whose finished flag is set skipped:
+ *   v = logits; softcap > 0: v = softcap * tanhf(v / softcap) (F32); every distinct token of
+ *   history[b][0 .. hist_len[b]) inside [0, V): v > 0 ? v / penalty : v * penalty, if penalty is finite and > 1;
+ *   leader = first largest finite v (token 0 if none).  temperature finite and > 0: tokens with
+ *   v >= leader + temperature * log(min_p) (all finite ones if min_p <= 0) have mass exp((v - leader) /
+ *   temperature) (F64); the row draws u from the generator and takes the first token whose running mass
+ *   reaches u * total.  Otherwise, or if the total is not a positive finite number, the leader is taken and
+ *   no draw is made.
+ * The generator is the reference's: one 64-bit state for all rows, state = splitmix64(state) per draw, u =
+ * (state >> 11) / 2^53, rows served in ascending order, only rows that draw advance it.
+ * Then, per row: a row that was not finished ends (finished[b] = 1) if the token is stop_token (>= 0) or its
+ * history is full (hist_len[b] == H); else the token is appended to history[b] and hist_len[b] += 1.
+ * ids[b] = the token, or for an ended row stop_token (0 if there is none); positions[b] += pos_delta;
+ * s = step_counters[b]; if s < max_steps (= out_ids count / B): out_ids[s*B + b] = the appended token, or -1
+ * if nothing was appended; step_counters[b] = s + 1.  table / next_x as in gd_backend_argmax_advance (the
+ * row of ids[b]).
+ * state: I32 [>= gd_backend_sample_state_count(B)], 8-byte aligned, owned by the loop: words 0-1 and 2-3
+ * hold the generator state (little-endian 64-bit, write the same start value to both), word 4 a launch
+ * counter (start 0), the rest is scratch.  work: F32 [>= B*V] scratch.  Sums are formed in another order
+ * than the reference's left-to-right loops: the token can differ from the reference's only when u * total
+ * lies within rounding distance (~1e-13 of the total) of the boundary between two tokens.  Calls on one
+ * state must not overlap. */
+typedef struct gd_backend_sample_args {
+    float temperature, min_p, repetition_penalty, logits_softcap;
+    int32_t stop_token; /* < 0: none */
+    int32_t pos_delta;
+} gd_backend_sample_args;
+
+typedef struct gd_backend_sample_tensors {
+    const gd_backend_tensor_view *history;       /* I32 [B, H] */
+    const gd_backend_tensor_view *hist_len;      /* I32 [B] */
+    const gd_backend_tensor_view *finished;      /* I32 [B] */
+    const gd_backend_tensor_view *state;         /* I32, see above */
+    const gd_backend_tensor_view *work;          /* F32 [B*V] */
+    const gd_backend_tensor_view *ids;           /* I32 [B] */
+    const gd_backend_tensor_view *positions;     /* I32 [B] */
+    const gd_backend_tensor_view *step_counters; /* I32 [B] */
+    const gd_backend_tensor_view *out_ids;       /* I32 [max_steps * B] */
+    const gd_backend_tensor_view *table;         /* [V, Dm] or NULL */
+    const gd_backend_tensor_view *next_x;        /* [B, Dm] or NULL */
+} gd_backend_sample_tensors;
+
+size_t gd_backend_sample_state_count(uint32_t rows);
+gd_status gd_backend_sample_advance(gd_backend *backend, const gd_backend_tensor_view *logits,
+                                    const gd_backend_sample_tensors *tensors, const gd_backend_sample_args *args);
+
 /* Device copy between buffers, enqueued like an operator. */
 gd_status gd_backend_copy(gd_backend *backend, gd_backend_buffer *dst, size_t dst_offset,
                           gd_backend_buffer *src, size_t src_offset, size_t nbytes);

@@ -121,6 +121,30 @@ gd_status gd_gpt_decoder_resident_end(gd_gpt_decoder *dec, int32_t *out_ids, flo
 gd_status gd_gpt_decoder_run_resident(gd_gpt_decoder *dec, const int32_t *first_ids, int32_t n_steps,
                                       int32_t *out_ids, float *out_gaps, float *step_ms);
 
+/* Generation with the reference's sampling front end, tokens in and tokens out: what gpt_generate_prompts_loaded
+ * of the reference's example does between its tokenizer calls (examples/gpt_lm/gpt_lm_shared.c:1444-1700), with
+ * the logits never leaving the device (gd_backend_sample_advance after the packed prefill and after every step
+ * of the resident loop).
+ *   ids / cu     packed prompts of the batch rows, cu [batch+1]; a prompt longer than the room the new tokens
+ *                leave (max_seq - max_new, or max_seq - 1 if max_new >= max_seq) keeps its last tokens (:1514-1533)
+ *   max_new      at most this many tokens per row
+ *   sampling     temperature <= 0 picks greedily; min_p, repetition_penalty (> 1 acts, over prompt + generated
+ *                tokens) and logits_softcap (> 0 acts) as in :1322-1442; a row ends when it picks stop_token
+ *                (>= 0; the token is not part of its output) or its sequence reaches max_seq; rng_state is the
+ *                generator state before the first draw: gd_gpt_generation_rng(seed, batch, step) gives the
+ *                reference's (:1565)
+ *   out_tokens   [batch, max_new]: row b's new tokens in its first out_counts[b] places
+ * The caches are rewritten from position 0.  GD_ERR_BUSY while a resident session is open. */
+typedef struct gd_gpt_sampling {
+    float temperature, min_p, repetition_penalty, logits_softcap;
+    int32_t stop_token; /* < 0: none */
+    uint64_t rng_state;
+} gd_gpt_sampling;
+
+uint64_t gd_gpt_generation_rng(uint64_t seed, int32_t n_prompts, uint64_t step);
+gd_status gd_gpt_decoder_generate(gd_gpt_decoder *dec, const int32_t *ids, const int32_t *cu, int32_t max_new,
+                                  const gd_gpt_sampling *sampling, int32_t *out_tokens, int32_t *out_counts);
+
 #pragma GCC visibility pop
 #ifdef __cplusplus
 }

@@ -640,6 +640,81 @@ GDO_API void gdo_argmax_rows_f16(const uint16_t *logits, int64_t rows, int64_t c
     }
 }
 
+/* ---- sampling front end (the step after the logits) ------------------------ */
+
+/* reference examples/gpt_lm/gpt_lm_shared.c:1322-1331 */
+GDO_API void gdo_logits_softcap(float *logits, int64_t n, float cap)
+{
+    if (!(cap > 0.0f)) return;
+    for (int64_t i = 0; i < n; ++i) logits[i] = cap * tanhf(logits[i] / cap);
+}
+
+/* reference :1347-1369: every distinct token of the history is penalised once */
+GDO_API void gdo_repetition_penalty(float *logits, int64_t vocab, const int32_t *history, int64_t len,
+                                    float penalty)
+{
+    if (len <= 0 || !isfinite(penalty) || penalty <= 1.0f) return;
+    for (int64_t i = 0; i < len; ++i) {
+        const int64_t token = history[i];
+        int seen = 0;
+        if (token < 0 || token >= vocab) continue;
+        for (int64_t j = 0; j < i && !seen; ++j) seen = history[j] == token;
+        if (seen) continue;
+        if (logits[token] > 0.0f) logits[token] /= penalty;
+        else logits[token] *= penalty;
+    }
+}
+
+/* reference :1371-1442.  logits are modified in place by the penalty, *rng advances by one
+ * splitmix64 application only when a draw is made.  margin (may be NULL) receives how far the
+ * drawn point lies from the nearest boundary between two tokens' intervals, as a fraction of
+ * the total mass (+inf when no draw was made): an implementation that sums in another order
+ * may pick the neighbouring token only when this is tiny. */
+GDO_API int32_t gdo_sample_next_token(float *logits, int64_t vocab, const int32_t *history, int64_t len,
+                                      float temperature, float min_p, float penalty, uint64_t *rng,
+                                      double *margin)
+{
+    int best = 0, have = 0;
+    double best_value = -HUGE_VAL;
+    if (margin) *margin = HUGE_VAL;
+    gdo_repetition_penalty(logits, vocab, history, len, penalty);
+    for (int64_t i = 0; i < vocab; ++i) {
+        const double value = (double)logits[i];
+        if (!isfinite(value)) continue;
+        if (!have || value > best_value) {
+            best_value = value;
+            best = (int)i;
+            have = 1;
+        }
+    }
+    if (!have || !isfinite(temperature) || temperature <= 0.0f) return best;
+    const double temp = (double)temperature;
+    const double threshold = min_p > 0.0f ? best_value + temp * log((double)min_p) : -HUGE_VAL;
+    double sum = 0.0;
+    for (int64_t i = 0; i < vocab; ++i) {
+        const double value = (double)logits[i];
+        if (!isfinite(value) || value < threshold) continue;
+        const double p = exp((value - best_value) / temp);
+        if (isfinite(p)) sum += p;
+    }
+    if (!(sum > 0.0) || !isfinite(sum)) return best;
+    *rng = gdo_splitmix64(*rng);
+    double target = ((double)(*rng >> 11) * (1.0 / 9007199254740992.0)) * sum;
+    for (int64_t i = 0; i < vocab; ++i) {
+        const double value = (double)logits[i];
+        if (!isfinite(value) || value < threshold) continue;
+        const double p = exp((value - best_value) / temp);
+        if (!isfinite(p)) continue;
+        target -= p;
+        if (target <= 0.0) {
+            if (margin) *margin = fmin(-target, target + p) / sum;
+            return (int32_t)i;
+        }
+    }
+    if (margin) *margin = 0.0;
+    return best;
+}
+
 /* ---- A13: decoder (call sequence of the reference example) ----------------- */
 
 typedef struct gdo_decoder {

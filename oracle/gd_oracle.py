@@ -74,6 +74,8 @@ def _declare(l):
         "gdo_swiglu_split_f16": [_vp, _i64, _i64, _vp],
         "gdo_embedding_f16": [_vp, _vp, _i64, _i64, _i64, _vp],
         "gdo_argmax_rows_f16": [_vp, _i64, _i64, _vp, _vp],
+        "gdo_logits_softcap": [_vp, _i64, _f32],
+        "gdo_repetition_penalty": [_vp, _i64, _vp, _i64, _f32],
         "gdo_decoder_destroy": [_vp],
         "gdo_decoder_untie_lm_head": [_vp, _u64],
         "gdo_decoder_step": [_vp, _vp, _vp, _vp, _vp],
@@ -83,6 +85,8 @@ def _declare(l):
         fn = getattr(l, name)
         fn.restype = None
         fn.argtypes = argtypes
+    l.gdo_sample_next_token.restype = C.c_int32
+    l.gdo_sample_next_token.argtypes = [_vp, _i64, _vp, _i64, _f32, _f32, _f32, C.POINTER(_u64), C.POINTER(C.c_double)]
     l.gdo_decoder_create.restype = _vp
     l.gdo_decoder_create.argtypes = [_i64] * 8 + [C.c_int, _u64]
     l.gdo_decoder_tensor.restype = _vp
@@ -293,6 +297,29 @@ def argmax_rows(logits):
     gap = np.empty(rows, np.float32)
     lib().gdo_argmax_rows_f16(_p(logits), rows, cols, _p(ids), _p(gap))
     return ids, gap
+
+
+def logits_softcap(logits, cap):
+    out = _c(logits, np.float32).copy()
+    lib().gdo_logits_softcap(_p(out), out.size, cap)
+    return out
+
+
+def repetition_penalty(logits, history, penalty):
+    out = _c(logits, np.float32).copy()
+    history = _c(history, np.int32)
+    lib().gdo_repetition_penalty(_p(out), out.size, _p(history), history.size, penalty)
+    return out
+
+
+def sample_next_token(logits, history, temperature, min_p, penalty, rng):
+    """One row.  Returns (token, new rng state, margin, logits after the penalty)."""
+    work = _c(logits, np.float32).copy()
+    history = _c(history, np.int32)
+    state, margin = _u64(rng), C.c_double()
+    token = lib().gdo_sample_next_token(_p(work), work.size, _p(history), history.size, temperature, min_p, penalty,
+                                        C.byref(state), C.byref(margin))
+    return int(token), int(state.value), float(margin.value), work
 
 
 # ---- decoder -------------------------------------------------------------------

@@ -145,6 +145,8 @@ gd_status gd_backend_copy(gd_backend *b, gd_backend_buffer *dst, size_t dst_offs
     return GD_OK;
 }
 
+size_t gd_backend_sample_state_count(uint32_t rows) { return 8u + 8u * (size_t)rows; }
+
 gd_status gd_backend_device_info(const gd_backend *b, char *name, size_t name_bytes, int32_t *compute_units,
                                  uint64_t *global_mem)
 {

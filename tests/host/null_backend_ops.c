@@ -31,6 +31,7 @@ GD_NULL_OP(gd_backend_qkv_rope_append)
 GD_NULL_OP(gd_backend_qkv_split_rope_forward)
 GD_NULL_OP(gd_backend_rand_uniform)
 GD_NULL_OP(gd_backend_rms_norm_forward)
+GD_NULL_OP(gd_backend_sample_advance)
 GD_NULL_OP(gd_backend_sdpa_decode)
 GD_NULL_OP(gd_backend_sdpa_decode_at)
 GD_NULL_OP(gd_backend_sdpa_decode_positions)

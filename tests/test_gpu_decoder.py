@@ -295,3 +295,96 @@ def test_checkpoint_written_by_the_reference_reproduces_its_generation(gda):
         assert st == -4
     finally:
         dev.close()
+
+
+def _reference_generate(oracle, ref, prompts, max_new, p, stop, rng, ctx_len):
+    """The reference's generation loop (examples/gpt_lm/gpt_lm_shared.c:1444-1700 without the tokenizer) over the
+    oracle decoder and the oracle's restatement of its sampler.  Returns the new tokens per row and the smallest
+    margin seen (distance of a draw from a token boundary, or the greedy gap)."""
+    B = len(prompts)
+    room = ctx_len - 1 if max_new >= ctx_len else ctx_len - max_new
+    seqs = [list(q[-room:]) for q in prompts]
+    plen = [len(q) for q in seqs]
+    cu = np.concatenate([[0], np.cumsum(plen)]).astype(np.int32)
+    logits, _, _ = ref.prefill(np.concatenate(seqs).astype(np.int32), cu)
+    finished, nxt, generated, worst = [False] * B, [0] * B, 0, np.inf
+
+    def pick(b, row):
+        nonlocal rng, worst
+        capped = oracle.logits_softcap(row.astype(np.float32), p["softcap"])
+        tok, rng, margin, left = oracle.sample_next_token(capped, seqs[b], p["temperature"], p["min_p"], p["penalty"], rng)
+        if not np.isfinite(margin):
+            top = np.sort(left[np.isfinite(left)])[-2:]
+            margin = float(top[1] - top[0]) if top.size == 2 else np.inf
+        worst = min(worst, margin)
+        return tok
+
+    for b in range(B):
+        nxt[b] = pick(b, logits[b])
+    while generated < max_new and not all(finished):
+        appended = False
+        for b in range(B):
+            if finished[b]:
+                continue
+            if (stop >= 0 and nxt[b] == stop) or len(seqs[b]) >= ctx_len:
+                finished[b] = True
+                continue
+            seqs[b].append(int(nxt[b]))
+            appended = True
+        if not appended:
+            break
+        generated += 1
+        if generated >= max_new or all(finished):
+            break
+        ids = np.array([(stop if stop >= 0 else 0) if finished[b] else nxt[b] for b in range(B)], np.int32)
+        logits, _, _ = ref.step(ids)
+        for b in range(B):
+            if not finished[b]:
+                nxt[b] = pick(b, logits[b])
+    return [np.array(seqs[b][plen[b]:], np.int32) for b in range(B)], worst
+
+
+@pytest.mark.parametrize("params,stop,max_new", [
+    (dict(temperature=0.8, min_p=0.05, penalty=1.3, softcap=20.0), 7, 24),
+    (dict(temperature=1.0, min_p=0.0, penalty=1.0, softcap=0.0), -1, 12),
+    (dict(temperature=0.0, min_p=0.0, penalty=1.2, softcap=0.0), 3, 40),
+    (dict(temperature=1.5, min_p=0.0, penalty=1.0, softcap=0.0), 1, 70),
+])
+def test_generate_with_the_sampling_front_end(gda, oracle, params, stop, max_new):
+    """gd_gpt_decoder_generate (packed prefill, device sampling, graph-replayed steps) against the reference's loop
+    restated over the oracle: the same tokens row by row, unless a draw fell within 1e-5 of a token boundary (then
+    the sequences may part and only the common prefix is compared).  Small vocabulary so that stop tokens and
+    repeats occur; the last case runs rows into the end of the context."""
+    from gradients_c_amd import decoder as D
+    V, Dm, L, H, Dh, Hm, T, B = 96, 64, 2, 2, 32, 128, 48, 5
+    if max_new == 70:
+        T = 40
+    seed = 4321
+    dev = D.GptDecoder(D.gpt_config(V, Dm, L, H, Dh, Hm, T, B, 0, True, seed), max_prefill_tokens=B * T)
+    ref = oracle.Decoder(V, Dm, L, H, Dh, Hm, T, B, 0, seed, True)
+    try:
+        lens = [9, 1, 30, 4, 17]
+        flat = oracle.uniform_i32(sum(lens), 5, 0, V - 1)
+        cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        prompts = [flat[cu[b]:cu[b + 1]] for b in range(B)]
+        rng0 = D.lib().gd_gpt_generation_rng(seed, B, 0)
+        assert rng0 == oracle.splitmix64(seed ^ 0xdec0de1234567890 ^ B ^ 0)
+        got = dev.generate(flat, cu, max_new, params["temperature"], params["min_p"], params["penalty"],
+                           params["softcap"], stop, rng0)
+        want, worst = _reference_generate(oracle, ref, prompts, max_new, params, stop, rng0, T)
+        exact = all(np.array_equal(g, w) for g, w in zip(got, want))
+        print("rows:", [len(w) for w in want], "worst margin:", worst, "exact:", exact)
+        if not exact:
+            assert worst < 1e-3, (got, want)
+        else:
+            assert all(len(w) <= max_new for w in want)
+        if max_new == 70:
+            room = T - 1
+            assert all(len(w) + min(len(q), room) <= T for w, q in zip(want, prompts))
+        # a second call starts over from its prompts (caches, histories, flags and generator are reset)
+        again = dev.generate(flat, cu, max_new, params["temperature"], params["min_p"], params["penalty"],
+                             params["softcap"], stop, rng0)
+        assert all(np.array_equal(a, g) for a, g in zip(again, got))
+    finally:
+        dev.close()
+        ref.close()

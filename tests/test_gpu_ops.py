@@ -929,3 +929,185 @@ def test_qkv_rope_append_equals_separate_ops(backend, arena, oracle, B, H, D):
     _close(q.read(), wq)
     _close(kc.read(), ok)
     assert np.array_equal(_bits(vc.read()), _bits(ov))
+
+
+# ---- sampling front end -----------------------------------------------------------------------------------------
+
+def _reference_sampling_step(oracle, logits, hist, hist_len, finished, rng, p, stop, H):
+    """One pass of the reference's loop body over the rows (examples/gpt_lm/gpt_lm_shared.c:1606-1680 reordered as
+    sample -> stop / full test -> append), with the oracle's restatement of its sampler.  Returns the new rng, the
+    per-row record (appended token or -1), the next input ids and the margin of every draw."""
+    B = logits.shape[0]
+    rec, ids, margins = np.full(B, -1, np.int32), np.zeros(B, np.int32), np.full(B, np.inf)
+    for b in range(B):
+        if finished[b]:
+            ids[b] = stop if stop >= 0 else 0
+            continue
+        row = oracle.logits_softcap(logits[b].astype(np.float32), p["softcap"])
+        tok, rng, margins[b], after = oracle.sample_next_token(row, hist[b, :hist_len[b]], p["temperature"], p["min_p"],
+                                                               p["penalty"], rng)
+        if not np.isfinite(margins[b]):
+            top = np.sort(after[np.isfinite(after)])[-2:]
+            margins[b] = np.inf if top.size < 2 else float(top[1] - top[0])   # greedy: gap to the runner-up
+        if stop >= 0 and tok == stop:
+            finished[b] = 1
+        elif hist_len[b] >= H:
+            finished[b] = 1
+        else:
+            hist[b, hist_len[b]] = tok
+            hist_len[b] += 1
+            rec[b] = tok
+        ids[b] = (stop if stop >= 0 else 0) if finished[b] else tok
+    return rng, rec, ids, margins
+
+
+@pytest.mark.parametrize("V", [64, 2048, 32003])
+@pytest.mark.parametrize("params", [
+    dict(temperature=0.8, min_p=0.05, penalty=1.3, softcap=20.0),
+    dict(temperature=1.0, min_p=0.0, penalty=1.0, softcap=0.0),
+    dict(temperature=0.0, min_p=0.0, penalty=1.5, softcap=0.0),
+    dict(temperature=2.5, min_p=0.5, penalty=float("inf"), softcap=5.0),
+])
+def test_sample_advance_follows_the_reference_sampler(backend, arena, oracle, gda, V, params):
+    B, H, steps, stop = 9, 24, 4, 5
+    rng_np = np.random.default_rng(V)
+    hist = np.full((B, H), -7, np.int32)
+    hist_len = np.array([5, 0, 24, 23, 9, 3, 12, 1, 7], np.int32)   # row 2 is full, row 3 fills up after one token
+    for b in range(B):
+        hist[b, :hist_len[b]] = rng_np.integers(0, min(V, 40), hist_len[b])   # small range: repeats
+    hist[4, 2] = V + 3                                                         # out of range: ignored
+    finished = np.array([0, 0, 0, 0, 0, 1, 0, 0, 0], np.int32)
+    state0 = 0x0123456789abcdef
+    t = dict(history=arena.from_numpy(hist), hist_len=arena.from_numpy(hist_len), finished=arena.from_numpy(finished),
+             state=arena.alloc((8 + 8 * B,), gda.I32), work=arena.alloc((B * V,), gda.F32),
+             ids=arena.alloc((B,), gda.I32), positions=arena.from_numpy(np.arange(B, dtype=np.int32) * 3),
+             step_counters=arena.from_numpy(np.zeros(B, np.int32)), out_ids=arena.alloc((steps * B,), gda.I32))
+    words = np.zeros(8 + 8 * B, np.int32)
+    words[:4] = np.array([state0, state0], np.uint64).view(np.int32)
+    t["state"].write(words)
+    table = oracle.normal_f16((V, 64), 77)
+    t["table"], t["next_x"] = arena.from_numpy(table), arena.alloc((B, 64), gda.F16)
+    rng = state0
+    for s in range(steps):
+        logits = oracle.normal_f16((B, V), 5000 + 10 * s + V % 7, 4.0)
+        logits[1, 3] = np.nan
+        logits[1, 9] = np.inf
+        logits[6, :] = [np.nan, np.inf, -np.inf][s % 3]            # nothing finite: token 0, no draw
+        logits[7, V // 2] = logits[7, V - 1] = np.float16(30.0)    # tied leaders
+        if s == 1:
+            logits[8, :] = -np.inf
+            logits[8, stop] = 1.0                                  # row 8 must stop here
+        backend.sample_advance(arena.from_numpy(logits), t, params["temperature"], params["min_p"], params["penalty"],
+                               params["softcap"], stop_token=stop, pos_delta=1)
+        rng, rec, ids, margins = _reference_sampling_step(oracle, logits, hist, hist_len, finished, rng, params, stop, H)
+        got_rec = t["out_ids"].read().reshape(steps, B)[s]
+        diff = np.nonzero(got_rec != rec)[0]
+        for b in diff:
+            assert margins[b] < 1e-5, f"step {s} row {b}: {got_rec[b]} vs {rec[b]}, margin {margins[b]}"
+        if diff.size:
+            return   # the histories legitimately part at a near-tie
+        assert np.array_equal(t["ids"].read(), ids), s
+        assert np.array_equal(t["history"].read(), hist) and np.array_equal(t["hist_len"].read(), hist_len), s
+        assert np.array_equal(t["finished"].read(), finished), s
+        assert np.array_equal(t["positions"].read(), np.arange(B) * 3 + s + 1)
+        assert np.array_equal(t["step_counters"].read(), np.full(B, s + 1))
+        assert np.array_equal(_bits(t["next_x"].read()), _bits(table[ids])), s
+        got_state = t["state"].read()[:4].view(np.uint64)
+        assert int(got_state[s % 2]) == rng, (s, hex(int(got_state[s % 2])), hex(rng))
+    assert finished[2] == 1 and finished[3] == 1 and finished[8] == 1 and hist_len[3] == 24
+
+
+def test_sample_advance_frequencies_and_draw_order(backend, arena, oracle, gda):
+    """Every row draws from the same fixed distribution: row b's draw must be number b of the step (the reference
+    serves the rows in order from one generator), and the tokens must follow the softmax."""
+    B, V, steps = 64, 6, 300
+    row = np.array([2.0, 1.0, 0.0, -1.0, 3.0, -4.0], np.float16)
+    logits = arena.from_numpy(np.tile(row, (B, 1)))
+    t = dict(history=arena.alloc((B, 4), gda.I32), hist_len=arena.from_numpy(np.zeros(B, np.int32)),
+             finished=arena.from_numpy(np.zeros(B, np.int32)), state=arena.alloc((8 + 8 * B,), gda.I32),
+             work=arena.alloc((B * V,), gda.F32), ids=arena.alloc((B,), gda.I32),
+             positions=arena.from_numpy(np.zeros(B, np.int32)), step_counters=arena.from_numpy(np.zeros(B, np.int32)),
+             out_ids=arena.alloc((steps * B,), gda.I32))
+    words = np.zeros(8 + 8 * B, np.int32)
+    words[:4] = np.array([42, 42], np.uint64).view(np.int32)
+    t["state"].write(words)
+    zeros = np.zeros(B, np.int32)
+    for s in range(steps):
+        t["hist_len"].write(zeros)          # keep the histories from filling up: every row keeps drawing
+        backend.sample_advance(logits, t, 1.7, 0.0, 1.0, 0.0, stop_token=-1, pos_delta=0)
+    got = t["ids"].read()
+    out = t["out_ids"].read().reshape(steps, B)
+    state, want = 42, np.empty((steps, B), np.int32)
+    for s in range(steps):
+        for b in range(B):
+            want[s, b], state, margin, _ = oracle.sample_next_token(row.astype(np.float32), [], 1.7, 0.0, 1.0, state)
+            assert margin > 1e-9
+    assert np.array_equal(out, want) and np.array_equal(got, want[-1])
+    p = np.exp(row.astype(np.float64) / 1.7)
+    p /= p.sum()
+    counts = np.bincount(out.ravel(), minlength=V)
+    chi2 = float((((counts - out.size * p) ** 2) / (out.size * p)).sum())
+    assert chi2 < 25.0, (chi2, counts / out.size, p)
+
+
+def test_sample_advance_rejects_bad_arguments(backend, arena, gda):
+    B, V = 2, 16
+    ok = dict(history=arena.alloc((B, 4), gda.I32), hist_len=arena.alloc((B,), gda.I32), finished=arena.alloc((B,), gda.I32),
+              state=arena.alloc((8 + 8 * B,), gda.I32), work=arena.alloc((B * V,), gda.F32), ids=arena.alloc((B,), gda.I32),
+              positions=arena.alloc((B,), gda.I32), step_counters=arena.alloc((B,), gda.I32),
+              out_ids=arena.alloc((3 * B,), gda.I32))
+    logits = arena.alloc((B, V), gda.F16)
+    for bad, status in ((dict(state=arena.alloc((8,), gda.I32)), gda.INVALID_ARGUMENT),
+                        (dict(work=arena.alloc((B * V - 1,), gda.F32)), gda.INVALID_ARGUMENT),
+                        (dict(work=arena.alloc((B * V,), gda.F16)), gda.UNSUPPORTED),
+                        (dict(ids=arena.alloc((B + 1,), gda.I32)), gda.INVALID_ARGUMENT),
+                        (dict(history=arena.alloc((B + 1, 4), gda.I32)), gda.INVALID_ARGUMENT),
+                        (dict(out_ids=arena.alloc((3 * B + 1,), gda.I32)), gda.INVALID_ARGUMENT),
+                        (dict(table=arena.alloc((V, 8), gda.F16)), gda.INVALID_ARGUMENT)):
+        with pytest.raises(gda.GdError) as err:
+            backend.sample_advance(logits, dict(ok, **bad), 1.0)
+        assert err.value.status == status, bad.keys()
+    with pytest.raises(gda.GdError) as err:
+        backend.sample_advance(logits, ok, 1.0, stop_token=V)
+    assert err.value.status == gda.INVALID_ARGUMENT
+
+
+def test_sample_advance_on_the_reference_samplers_golden_cases(backend, arena, oracle, gda):
+    """The inputs of tests/golden/sampler_cases.npz through the device kernels: the tokens the reference's own host
+    sampler returned (margins from the oracle: a differing token must lie within 1e-5 of a boundary), its generator
+    after the last row, and the capped + penalised rows it left behind (work buffer; tanhf may differ by an ulp)."""
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sampler_cases.npz"))
+    for c in sorted({k.split("_")[0] for k in z.files}):
+        temperature, min_p, penalty, softcap = (float(v) for v in z[f"{c}_params"])
+        logits, hist_len, history = z[f"{c}_logits"], z[f"{c}_hist_len"], z[f"{c}_history"]
+        B, V = logits.shape
+        H = history.shape[1] + 1                                   # one free place: no row ends by a full history
+        hist = np.zeros((B, H), np.int32)
+        hist[:, :H - 1] = history
+        t = dict(history=arena.from_numpy(hist), hist_len=arena.from_numpy(hist_len),
+                 finished=arena.from_numpy(np.zeros(B, np.int32)), state=arena.alloc((8 + 8 * B,), gda.I32),
+                 work=arena.alloc((B * V,), gda.F32), ids=arena.alloc((B,), gda.I32),
+                 positions=arena.from_numpy(np.zeros(B, np.int32)), step_counters=arena.from_numpy(np.zeros(B, np.int32)),
+                 out_ids=arena.alloc((B,), gda.I32))
+        words = np.zeros(8 + 8 * B, np.int32)
+        words[:2] = words[2:4] = z[f"{c}_rng"].view(np.int32)
+        t["state"].write(words)
+        backend.sample_advance(arena.from_numpy(logits.astype(np.float16)), t, temperature, min_p, penalty, softcap,
+                               stop_token=-1, pos_delta=0)
+        got = t["ids"].read()
+        state = int(z[f"{c}_rng"].view(np.uint64)[0])
+        for r in range(B):
+            tok, state, margin, left = oracle.sample_next_token(oracle.logits_softcap(logits[r], softcap),
+                                                                history[r, :hist_len[r]], temperature, min_p, penalty, state)
+            assert tok == z[f"{c}_tokens"][r]
+            if got[r] != tok:
+                if not np.isfinite(margin):
+                    top = np.sort(left[np.isfinite(left)])[-2:]
+                    margin = float(top[1] - top[0])
+                assert margin < 1e-5, (c, r, got[r], tok, margin)
+        assert int(t["state"].read()[:4].view(np.uint64)[0]) == int(z[f"{c}_rng_after"].view(np.uint64)[-1]), c
+        work = t["work"].read().reshape(B, V)
+        want = z[f"{c}_logits_after"]
+        same = (work == want) | (np.isnan(work) & np.isnan(want))
+        assert np.all(same | (np.abs(work - want) <= 2e-6 * np.abs(want))), c
+        assert np.array_equal(t["hist_len"].read(), hist_len + 1)

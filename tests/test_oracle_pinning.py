@@ -564,3 +564,127 @@ def test_decoder_batch_rows_independent(oracle):
     s2, n2, _ = d2.step(nx2)
     s1, n1, _ = d1.step(nx1)
     assert np.array_equal(s2[1].view(np.uint16), s1[0].view(np.uint16)) and n2[1] == n1[0]
+
+
+# ---- sampling front end (reference examples/gpt_lm/gpt_lm_shared.c:1322-1442) --------------------------------
+
+def test_softcap_against_numpy_and_identity_cases(oracle):
+    rng = np.random.default_rng(3)
+    x = np.concatenate([rng.normal(0, 30, 4000), [0.0, -0.0, 1e-8, 200.0, -200.0, np.inf, -np.inf]]).astype(np.float32)
+    got = oracle.logits_softcap(x, 20.0)
+    want = 20.0 * np.tanh(x.astype(np.float64) / 20.0)
+    assert np.allclose(got, want, rtol=3e-7, atol=1e-12)
+    assert got[-2] == 20.0 and got[-1] == -20.0 and np.all(np.abs(got) <= 20.0)
+    for cap in (0.0, -1.0, float("nan")):
+        assert np.array_equal(oracle.logits_softcap(x, cap), x)
+
+
+def test_repetition_penalty_brute_force(oracle):
+    rng = np.random.default_rng(4)
+    logits = rng.normal(0, 3, 50).astype(np.float32)
+    logits[7] = 0.0
+    history = np.array([3, 7, 3, 49, -1, 50, 12, 12, 12, 0, 3], np.int32)
+    got = oracle.repetition_penalty(logits, history, 1.3)
+    want = logits.copy()
+    for t in set(int(t) for t in history if 0 <= t < 50):   # once per distinct token, however often it occurs
+        want[t] = want[t] / np.float32(1.3) if want[t] > 0 else want[t] * np.float32(1.3)
+    assert np.array_equal(got, want)
+    assert got[3] != logits[3] and got[7] == 0.0 and got[5] == logits[5]
+    for off in (1.0, 0.5, float("nan"), float("inf")):
+        assert np.array_equal(oracle.repetition_penalty(logits, history, off), logits)
+    assert np.array_equal(oracle.repetition_penalty(logits, history[:0], 1.3), logits)
+
+
+def test_sampling_greedy_cases_leave_the_generator_alone(oracle):
+    logits = np.array([1.0, 5.0, np.nan, 5.0, np.inf, -np.inf, 2.0], np.float32)
+    for temperature in (0.0, -1.0, float("nan"), float("inf")):
+        tok, state, margin, _ = oracle.sample_next_token(logits, [], temperature, 0.0, 1.0, 99)
+        assert (tok, state) == (1, 99) and margin == np.inf     # first of the tied finite maxima, no draw
+    bad = np.array([np.nan, np.inf, -np.inf], np.float32)
+    assert oracle.sample_next_token(bad, [], 1.0, 0.0, 1.0, 5)[:2] == (0, 5)
+    # the penalty acts before the pick: the repeated leader loses
+    assert oracle.sample_next_token(np.array([4.0, 3.9], np.float32), [0], 0.0, 0.0, 1.5, 1)[0] == 1
+
+
+def test_sampling_draw_is_the_inverse_cdf_of_the_softmax(oracle):
+    # equal logits: token = floor(u * V) with u the 53-bit fraction of the advanced state
+    state = 0x1234
+    for _ in range(200):
+        tok, new_state, margin, _ = oracle.sample_next_token(np.zeros(8, np.float32), [], 1.0, 0.0, 1.0, state)
+        assert new_state == oracle.splitmix64(state)
+        u = (new_state >> 11) / 2.0 ** 53
+        assert tok == int(np.floor(u * 8)), (tok, u)
+        assert abs(margin - min(u * 8 - tok, tok + 1 - u * 8) / 8) < 1e-12
+        state = new_state
+    # general logits, temperature and min_p against numpy's float64 softmax / cumsum / searchsorted
+    rng = np.random.default_rng(8)
+    for case in range(300):
+        V = int(rng.integers(2, 300))
+        logits = rng.normal(0, 4, V).astype(np.float32)
+        if case % 3 == 0:
+            logits[rng.integers(0, V, 3)] = [np.nan, np.inf, -np.inf]
+        temperature = float(rng.choice([0.3, 0.8, 1.0, 2.5]))
+        min_p = float(rng.choice([0.0, 0.05, 0.3, 1.0]))
+        tok, new_state, margin, _ = oracle.sample_next_token(logits, [], temperature, min_p, 1.0, 1000 + case)
+        finite = np.isfinite(logits)
+        if not finite.any():
+            assert (tok, new_state) == (0, 1000 + case)
+            continue
+        z = np.where(finite, logits.astype(np.float64), -np.inf)
+        p = np.exp((z - z.max()) / temperature)                 # relative to the leader: p.max() == 1
+        keep = finite & (p >= min_p * (1 - 1e-12)) if min_p > 0 else finite
+        mass = np.where(keep, p, 0.0)
+        u = (oracle.splitmix64(1000 + case) >> 11) / 2.0 ** 53
+        want = int(np.searchsorted(np.cumsum(mass), u * mass.sum(), side="left"))
+        if margin > 1e-9:
+            assert tok == want, (case, tok, want, margin)
+        assert keep[tok]
+
+
+def test_sampling_frequencies_follow_the_distribution(oracle):
+    logits = np.array([2.0, 1.0, 0.0, -1.0, 3.0, -4.0], np.float32)
+    temperature, n = 1.7, 40000
+    counts = np.zeros(6)
+    state = 777
+    for _ in range(n):
+        tok, state, _, _ = oracle.sample_next_token(logits, [], temperature, 0.0, 1.0, state)
+        counts[tok] += 1
+    p = np.exp(logits.astype(np.float64) / temperature)
+    p /= p.sum()
+    chi2 = float((((counts - n * p) ** 2) / (n * p)).sum())
+    assert chi2 < 25.0, (chi2, counts / n, p)                   # 5 degrees of freedom: P(chi2 > 25) ~ 1e-4
+    # with min_p the tail is cut and the rest renormalised
+    counts[:] = 0
+    for _ in range(n):
+        tok, state, _, _ = oracle.sample_next_token(logits, [], temperature, 0.2, 1.0, state)
+        counts[tok] += 1
+    keep = p >= 0.2 * p.max()
+    assert counts[~keep].sum() == 0 and 1 < keep.sum() < 6
+    q = np.where(keep, p, 0) / p[keep].sum()
+    chi2 = float((((counts[keep] - n * q[keep]) ** 2) / (n * q[keep])).sum())
+    assert chi2 < 25.0
+
+
+def test_sampler_equals_the_reference_sampler_on_golden_cases(oracle):
+    """tests/golden/sampler_cases.npz holds what the reference's own gpt_apply_logits_softcap +
+    gpt_sample_next_token returned (tests/golden/make_sampler_fixture.py ran them through oracle/_ref/ref_sampler):
+    tokens, the generator after every row and the rows as the sampler left them must be identical."""
+    import os
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sampler_cases.npz"))
+    cases = sorted({k.split("_")[0] for k in z.files})
+    assert len(cases) == 7
+    for c in cases:
+        temperature, min_p, penalty, softcap = (float(v) for v in z[f"{c}_params"])
+        state = int(z[f"{c}_rng"].view(np.uint64)[0])
+        after = z[f"{c}_rng_after"].view(np.uint64)
+        drew = 0
+        for r, row in enumerate(z[f"{c}_logits"]):
+            capped = oracle.logits_softcap(row, softcap)
+            hist = z[f"{c}_history"][r, :z[f"{c}_hist_len"][r]]
+            tok, new_state, _, left = oracle.sample_next_token(capped, hist, temperature, min_p, penalty, state)
+            assert tok == z[f"{c}_tokens"][r], (c, r)
+            assert new_state == int(after[r]), (c, r)
+            assert np.array_equal(left.view(np.uint32), z[f"{c}_logits_after"][r].view(np.uint32)), (c, r)
+            drew += new_state != state
+            state = new_state
+        assert (drew > 0) == (np.isfinite(temperature) and temperature > 0), c
