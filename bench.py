@@ -216,6 +216,43 @@ def long_context_workload(a, pkg, oracle, D, which):
     print(json.dumps(line))
 
 
+def sampled_workload(a, oracle, D):
+    """The headline step (B=64, 511 cached tokens, positions held) with gd_backend_sample_advance after the LM head.
+    Cache rows are allocated for 1024 tokens so that the rows' histories (prompt + sampled tokens, which the
+    repetition penalty scans) can grow for the length of the run; attention still covers 512 keys per step."""
+    B, T, cap = 64, 512, 1024
+    total = a.warmup + a.steps
+    if T - 1 + total + 2 > cap:
+        sys.exit("--sampled: warmup + steps must stay below 510")
+    dec = D.GptDecoder(D.gpt_config(2048, 512, 3, 8, 64, 1536, cap, B, window=0, tie_lm_head=False, seed=1002),
+                       max_prefill_tokens=B * (T - 1))
+    prompt = oracle.uniform_i32(B * (T - 1), 1002, 0, 2047)
+    cu = (np.arange(B + 1) * (T - 1)).astype(np.int32)
+    dec.prefill(prompt, cu, want_logits=False)
+    dec.resident_begin_sampled(prompt, cu, total + 2, temperature=0.8, min_p=0.05, repetition_penalty=1.3,
+                               logits_softcap=20.0, stop_token=-1, rng_state=1002, hold_positions=True)
+    dec.resident_run(a.warmup)
+    dec.resident_sync()
+    t0 = time.perf_counter()
+    dec.resident_run(a.steps)
+    dec.resident_sync()
+    elapsed = time.perf_counter() - t0
+    ids, _ = dec.resident_end()
+    assert ids.shape == (total + 2, B) and ids.min() >= 0 and ids.max() < 2048
+    distinct = len(np.unique(ids))
+    dec.close()
+    print(json.dumps({
+        "metric": "decode tokens/sec at B=64", "value": round(B * a.steps / elapsed, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(elapsed * 1e3 / a.steps, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "configs[2] with the sampling front end: gpt_lm default decoder (V2048 Dm512 L3 H8 Dh64 "
+                               "Hm1536, untied head), B=64, 511 cached tokens, soft cap 20 + repetition penalty 1.3 + "
+                               "temperature 0.8 + min-p 0.05 drawn on the device, device-resident token feedback",
+                   "batch": B, "cache_tokens": T, "sdpa_window": 0, "distinct_tokens_drawn": distinct},
+        "roofline": None, "cpu_baseline": None,
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -227,6 +264,10 @@ def main():
                          "(reported without roofline / cpu_baseline objects)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="with --workload 3 or 4: stop after the packed prefill (for kernel traces of the prefill kernels)")
+    ap.add_argument("--sampled", action="store_true",
+                    help="the headline step with the sampling front end (soft cap 20, repetition penalty 1.3, "
+                         "temperature 0.8, min-p 0.05) in place of the greedy pick; reported without roofline / "
+                         "cpu_baseline objects")
     ap.add_argument("--kernel-only", action="store_true",
                     help="only launch sdpa_decode at the benchmark shape plus calibration copies (for --pmc runs)")
     a = ap.parse_args()
@@ -242,6 +283,10 @@ def main():
     from gradients_c_amd import decoder as D
     if a.workload != 2:
         long_context_workload(a, pkg, oracle, D, a.workload)
+        return
+
+    if a.sampled:
+        sampled_workload(a, oracle, D)
         return
 
     B, T = 64, 512

@@ -178,6 +178,7 @@ _OTHER_RESTYPE = {
     "gd_backend_fence_is_complete": (C.c_bool, [C.POINTER(Fence)]),
     "gd_backend_timer_destroy": (None, [_vp]),
     "gd_backend_sample_state_count": (C.c_size_t, [C.c_uint32]),
+    "gd_backend_sample_work_count": (C.c_size_t, [C.c_uint32, C.c_uint32]),
     "gd_backend_graph_destroy": (None, [_vp]),
 }
 EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + list(_OTHER_RESTYPE))
@@ -504,6 +505,14 @@ class Backend:
         a = SampleArgs(temperature, min_p, repetition_penalty, logits_softcap, stop_token, pos_delta)
         st = self.call("gd_backend_sample_advance", logits.view(), C.byref(t), C.byref(a))
         _check(st, "gd_backend_sample_advance")
+
+    @staticmethod
+    def sample_work_count(rows, cols):
+        return lib().gd_backend_sample_work_count(rows, cols)
+
+    @staticmethod
+    def sample_state_count(rows):
+        return lib().gd_backend_sample_state_count(rows)
 
     def gather_rows(self, src, rows, out):
         _check(self.call("gd_backend_gather_rows", src.view(), rows.view(), out.view()), "gd_backend_gather_rows")

@@ -159,8 +159,9 @@ size_t gd_gpt_state_bytes(const gd_gpt_config *c)
 {
     const size_t cache = pad256((size_t)c->batch * (size_t)c->max_seq * (size_t)c->n_heads * (size_t)c->head_dim * 2U);
     const size_t B = (size_t)c->batch, V = (size_t)c->vocab;
-    const size_t sampling = pad256(B * V * 2U) + pad256(B * V * 4U) + pad256(B * (size_t)c->max_seq * 4U) +
-                            2U * pad256(B * 4U) + pad256((8U + 8U * B) * 4U);
+    const size_t sampling = pad256(B * V * 2U) + pad256(gd_backend_sample_work_count((uint32_t)B, (uint32_t)V) * 4U) +
+                            pad256(B * (size_t)c->max_seq * 4U) +
+                            2U * pad256(B * 4U) + pad256(gd_backend_sample_state_count((uint32_t)B) * 4U);
     return cache * 2U * (size_t)c->n_layers + 4U * pad256((size_t)c->batch * 4U) +
            pad256((size_t)c->batch * (size_t)c->d_model * 2U) + sampling + 4096U;
 }
@@ -238,7 +239,8 @@ gd_status gd_gpt_decoder_create(gd_context *ctx, const gd_gpt_config *cfg, gd_gp
     }
     {
         int64_t ldim[2] = {cfg->batch, cfg->vocab}, hdim[2] = {cfg->batch, cfg->max_seq};
-        int64_t sdim[1] = {8 + 8 * (int64_t)cfg->batch}, wdim[1] = {(int64_t)cfg->batch * cfg->vocab};
+        int64_t sdim[1] = {(int64_t)gd_backend_sample_state_count((uint32_t)cfg->batch)};
+        int64_t wdim[1] = {(int64_t)gd_backend_sample_work_count((uint32_t)cfg->batch, (uint32_t)cfg->vocab)};
         STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_F16, gd_shape_make(2U, ldim), 256U, &d->last_logits));
         STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_I32, gd_shape_make(2U, hdim), 256U, &d->history));
         STEP(gd_tensor_zeros(ctx, GD_ARENA_STATE, GD_DTYPE_I32, gd_shape_make(1U, bdim), 256U, &d->hist_len));
@@ -931,7 +933,7 @@ static gd_status enqueue_resident_step(gd_gpt_decoder *d)
         } else {
             TRY(enqueue_fused_step(d, &logits));
         }
-        return enqueue_sample(d, &logits, 1);
+        return enqueue_sample(d, &logits, d->resident_hold ? 0 : 1);
     }
     if (d->resident_unfused) {
         TRY(gd_embedding(ctx, &d->token_embedding, &d->ids_dev, &x));
@@ -1113,6 +1115,48 @@ gd_status gd_gpt_decoder_resident_end(gd_gpt_decoder *d, int32_t *out_ids, float
     return st;
 }
 
+gd_status gd_gpt_decoder_resident_begin_sampled(gd_gpt_decoder *d, const int32_t *ids, const int32_t *cu,
+                                                int32_t max_picks, int32_t flags, const gd_gpt_sampling *sampling)
+{
+    gd_context *ctx;
+    gd_tensor head_words;
+    int32_t *hist, *lens;
+    int32_t state_words[8];
+    int32_t B, b;
+    gd_status st;
+    if (d == NULL || ids == NULL || cu == NULL || sampling == NULL || max_picks <= 0 || cu[0] != 0 ||
+        sampling->stop_token >= d->cfg.vocab)
+        return GD_ERR_INVALID_ARGUMENT;
+    if (d->resident_open) return GD_ERR_BAD_STATE;
+    ctx = d->ctx;
+    B = d->cfg.batch;
+    if (B <= 0) return GD_ERR_BAD_STATE;
+    for (b = 0; b < B; ++b) {
+        if (cu[b + 1] < cu[b] || cu[b + 1] - cu[b] > d->cfg.max_seq) return GD_ERR_INVALID_ARGUMENT;
+    }
+    hist = (int32_t *)calloc((size_t)B * (size_t)d->cfg.max_seq, sizeof(int32_t));
+    lens = (int32_t *)calloc((size_t)B, sizeof(int32_t));
+    if (hist == NULL || lens == NULL) {
+        free(hist); free(lens);
+        return GD_ERR_OUT_OF_MEMORY;
+    }
+    for (b = 0; b < B; ++b) {
+        lens[b] = cu[b + 1] - cu[b];
+        memcpy(hist + (size_t)b * (size_t)d->cfg.max_seq, ids + cu[b], (size_t)lens[b] * sizeof(int32_t));
+    }
+    memset(state_words, 0, sizeof(state_words));
+    memcpy(&state_words[0], &sampling->rng_state, sizeof(uint64_t));
+    memcpy(&state_words[2], &sampling->rng_state, sizeof(uint64_t));
+    st = gd_tensor_slice(ctx, &d->sample_state, 0U, 0, 8, &head_words);
+    if (st == GD_OK) st = gd_tensor_write(ctx, &head_words, state_words, sizeof(state_words));
+    if (st == GD_OK) st = gd_tensor_write(ctx, &d->history, hist, (size_t)B * (size_t)d->cfg.max_seq * sizeof(int32_t));
+    if (st == GD_OK) st = gd_tensor_write(ctx, &d->hist_len, lens, (size_t)B * sizeof(int32_t));
+    if (st == GD_OK) st = gd_tensor_zero_(ctx, &d->finished);
+    free(hist); free(lens);
+    if (st != GD_OK) return st;
+    return resident_begin_impl(d, NULL, max_picks, flags, sampling);
+}
+
 /* ---- generation with the sampling front end ---------------------------------------------- */
 
 uint64_t gd_gpt_generation_rng(uint64_t seed, int32_t n_prompts, uint64_t step)
@@ -1125,8 +1169,7 @@ gd_status gd_gpt_decoder_generate(gd_gpt_decoder *d, const int32_t *ids, const i
 {
     const int32_t check_every = 32; /* decode steps between two looks at the finished flags */
     gd_context *ctx;
-    int32_t *packed = NULL, *pcu = NULL, *hist = NULL, *lens = NULL, *records = NULL, *flags = NULL;
-    int32_t state_words[8];
+    int32_t *packed = NULL, *pcu = NULL, *lens = NULL, *records = NULL, *flags = NULL;
     int32_t B, ctx_len, room, b, total = 0, done = 0, decode_steps;
     gd_status st;
     if (d == NULL || ids == NULL || cu == NULL || sampling == NULL || out_tokens == NULL || out_counts == NULL ||
@@ -1145,10 +1188,9 @@ gd_status gd_gpt_decoder_generate(gd_gpt_decoder *d, const int32_t *ids, const i
     }
     pcu = (int32_t *)calloc((size_t)B + 1U, sizeof(int32_t));
     lens = (int32_t *)calloc((size_t)B, sizeof(int32_t));
-    hist = (int32_t *)calloc((size_t)B * (size_t)ctx_len, sizeof(int32_t));
     flags = (int32_t *)calloc((size_t)B, sizeof(int32_t));
     records = (int32_t *)malloc((size_t)max_new * (size_t)B * sizeof(int32_t));
-    if (pcu == NULL || lens == NULL || hist == NULL || flags == NULL || records == NULL) {
+    if (pcu == NULL || lens == NULL || flags == NULL || records == NULL) {
         st = GD_ERR_OUT_OF_MEMORY;
         goto out;
     }
@@ -1167,22 +1209,9 @@ gd_status gd_gpt_decoder_generate(gd_gpt_decoder *d, const int32_t *ids, const i
     for (b = 0; b < B; ++b) {
         const int32_t *src = ids + cu[b + 1] - lens[b];
         memcpy(packed + pcu[b], src, (size_t)lens[b] * sizeof(int32_t));
-        memcpy(hist + (size_t)b * (size_t)ctx_len, src, (size_t)lens[b] * sizeof(int32_t));
     }
     st = gd_gpt_decoder_prefill(d, packed, pcu, NULL, NULL, NULL); /* leaves the logits in last_logits */
-    if (st != GD_OK) goto out;
-    memset(state_words, 0, sizeof(state_words));
-    memcpy(&state_words[0], &sampling->rng_state, sizeof(uint64_t));
-    memcpy(&state_words[2], &sampling->rng_state, sizeof(uint64_t));
-    {
-        gd_tensor head_words;
-        st = gd_tensor_slice(ctx, &d->sample_state, 0U, 0, 8, &head_words);
-        if (st == GD_OK) st = gd_tensor_write(ctx, &head_words, state_words, sizeof(state_words));
-    }
-    if (st == GD_OK) st = gd_tensor_write(ctx, &d->history, hist, (size_t)B * (size_t)ctx_len * sizeof(int32_t));
-    if (st == GD_OK) st = gd_tensor_write(ctx, &d->hist_len, lens, (size_t)B * sizeof(int32_t));
-    if (st == GD_OK) st = gd_tensor_zero_(ctx, &d->finished);
-    if (st == GD_OK) st = resident_begin_impl(d, NULL, max_new, 0, sampling);
+    if (st == GD_OK) st = gd_gpt_decoder_resident_begin_sampled(d, packed, pcu, max_new, 0, sampling);
     if (st != GD_OK) goto out;
     /* the reference leaves its loop when every row has ended (:1607, 1634-1636): look at the flags now and then */
     decode_steps = max_new - 1;
@@ -1213,7 +1242,7 @@ gd_status gd_gpt_decoder_generate(gd_gpt_decoder *d, const int32_t *ids, const i
         out_counts[b] = n;
     }
 out:
-    free(packed); free(pcu); free(hist); free(lens); free(records); free(flags);
+    free(packed); free(pcu); free(lens); free(records); free(flags);
     return st;
 }
 

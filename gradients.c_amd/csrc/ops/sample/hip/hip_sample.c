@@ -11,6 +11,7 @@ typedef struct gd_hip_sample_cfg {
     float temperature, min_p, penalty, softcap;
     int32_t stop_token;
     uint32_t cols, hist_cap;
+    uint32_t parts; /* filled in by the launcher */
 } gd_hip_sample_cfg;
 
 typedef struct gd_hip_sample_advance {
@@ -31,7 +32,15 @@ static int i32_rows(const gd_backend_tensor_view *v, uint64_t rows)
     return gd_hip_view_ok(v) && v->dtype == GD_BACKEND_DTYPE_I32 && v->count == (size_t)rows && (v->offset & 3u) == 0u;
 }
 
-size_t gd_backend_sample_state_count(uint32_t rows) { return 8u + 8u * (size_t)rows; }
+size_t gd_backend_sample_state_count(uint32_t rows) { return 8u + 10u * (size_t)rows; }
+
+/* F32 values [rows * cols] (rounded up to an even count), then per row and part of 2048 tokens 258 8-byte cells
+ * (256 segment masses, the part's mass, the part's leader) */
+size_t gd_backend_sample_work_count(uint32_t rows, uint32_t cols)
+{
+    const size_t values = ((size_t)rows * cols + 1u) & ~(size_t)1u, parts = ((size_t)cols + 2047u) / 2048u;
+    return values + 2u * (size_t)rows * parts * 258u;
+}
 
 gd_status gd_backend_sample_advance(gd_backend *backend, const gd_backend_tensor_view *logits,
                                     const gd_backend_sample_tensors *t, const gd_backend_sample_args *args)
@@ -58,7 +67,7 @@ gd_status gd_backend_sample_advance(gd_backend *backend, const gd_backend_tensor
     if (!i32_rows(t->hist_len, rows) || !i32_rows(t->finished, rows) || !i32_rows(t->ids, rows) ||
         !i32_rows(t->positions, rows) || !i32_rows(t->step_counters, rows) ||
         t->state->count < gd_backend_sample_state_count((uint32_t)rows) || (t->state->offset & 7u) != 0u ||
-        t->work->count < (size_t)(rows * cols) || (t->work->offset & 3u) != 0u || (t->out_ids->count % rows) != 0u ||
+        t->work->count < gd_backend_sample_work_count((uint32_t)rows, (uint32_t)cols) || (t->work->offset & 7u) != 0u || (t->out_ids->count % rows) != 0u ||
         (t->out_ids->offset & 3u) != 0u)
         return GD_ERR_INVALID_ARGUMENT;
     max_steps = t->out_ids->count / rows;
@@ -82,6 +91,7 @@ gd_status gd_backend_sample_advance(gd_backend *backend, const gd_backend_tensor
     cfg.stop_token = args->stop_token;
     cfg.cols = (uint32_t)cols;
     cfg.hist_cap = (uint32_t)hist_cap;
+    cfg.parts = 0u;
     adv.history = (int32_t *)gd_hip_view_ptr(t->history);
     adv.hist_len = (int32_t *)gd_hip_view_ptr(t->hist_len);
     adv.finished = (int32_t *)gd_hip_view_ptr(t->finished);

@@ -135,6 +135,7 @@ def lib():
         l.gd_gpt_decoder_resident_end.argtypes = [_vp, _vp, _vp, C.POINTER(C.c_int32)]
         l.gd_gpt_decoder_load_checkpoint.argtypes = [_vp, C.c_char_p, C.c_int32]
         l.gd_gpt_decoder_generate.argtypes = [_vp, _vp, _vp, C.c_int32, C.POINTER(GptSampling), _vp, _vp]
+        l.gd_gpt_decoder_resident_begin_sampled.argtypes = [_vp, _vp, _vp, C.c_int32, C.c_int32, C.POINTER(GptSampling)]
         l.gd_gpt_generation_rng.argtypes = [C.c_uint64, C.c_int32, C.c_uint64]
         l.gd_gpt_generation_rng.restype = C.c_uint64
         l.gd_gpt_config_from_checkpoint.argtypes = [C.c_char_p, C.POINTER(GptConfig)]
@@ -333,6 +334,16 @@ class GptDecoder:
         flags = (1 if hold_positions else 0) | (2 if unfused else 0)
         self.ctx.check(lib().gd_gpt_decoder_resident_begin(self.handle, first.ctypes.data_as(_vp), max_steps, flags),
                        "gd_gpt_decoder_resident_begin")
+
+    def resident_begin_sampled(self, ids, cu, max_picks, temperature, min_p=0.0, repetition_penalty=1.0,
+                               logits_softcap=0.0, stop_token=-1, rng_state=0, hold_positions=False, unfused=False):
+        ids, cu = np.ascontiguousarray(ids, np.int32), np.ascontiguousarray(cu, np.int32)
+        self._resident_max = max_picks
+        s = GptSampling(temperature, min_p, repetition_penalty, logits_softcap, stop_token, rng_state)
+        flags = (1 if hold_positions else 0) | (2 if unfused else 0)
+        self.ctx.check(lib().gd_gpt_decoder_resident_begin_sampled(self.handle, ids.ctypes.data_as(_vp),
+                                                                   cu.ctypes.data_as(_vp), max_picks, flags, C.byref(s)),
+                       "gd_gpt_decoder_resident_begin_sampled")
 
     def resident_run(self, n_steps):
         self.ctx.check(lib().gd_gpt_decoder_resident_run(self.handle, n_steps), "gd_gpt_decoder_resident_run")

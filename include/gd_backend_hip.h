@@ -441,7 +441,8 @@ gd_status gd_backend_argmax_advance(gd_backend *backend, const gd_backend_tensor
  * row of ids[b]).
  * state: I32 [>= gd_backend_sample_state_count(B)], 8-byte aligned, owned by the loop: words 0-1 and 2-3
  * hold the generator state (little-endian 64-bit, write the same start value to both), word 4 a launch
- * counter (start 0), the rest is scratch.  work: F32 [>= B*V] scratch.  Sums are formed in another order
+ * counter (start 0), the rest is scratch.  work: F32 [>= gd_backend_sample_work_count(B, V)], 8-byte aligned,
+ * scratch (the rows after cap and penalty, then masses of runs of consecutive tokens).  Sums are formed in another order
  * than the reference's left-to-right loops: the token can differ from the reference's only when u * total
  * lies within rounding distance (~1e-13 of the total) of the boundary between two tokens.  Calls on one
  * state must not overlap. */
@@ -456,7 +457,7 @@ typedef struct gd_backend_sample_tensors {
     const gd_backend_tensor_view *hist_len;      /* I32 [B] */
     const gd_backend_tensor_view *finished;      /* I32 [B] */
     const gd_backend_tensor_view *state;         /* I32, see above */
-    const gd_backend_tensor_view *work;          /* F32 [B*V] */
+    const gd_backend_tensor_view *work;          /* F32, see above */
     const gd_backend_tensor_view *ids;           /* I32 [B] */
     const gd_backend_tensor_view *positions;     /* I32 [B] */
     const gd_backend_tensor_view *step_counters; /* I32 [B] */
@@ -466,6 +467,7 @@ typedef struct gd_backend_sample_tensors {
 } gd_backend_sample_tensors;
 
 size_t gd_backend_sample_state_count(uint32_t rows);
+size_t gd_backend_sample_work_count(uint32_t rows, uint32_t cols);
 gd_status gd_backend_sample_advance(gd_backend *backend, const gd_backend_tensor_view *logits,
                                     const gd_backend_sample_tensors *tensors, const gd_backend_sample_args *args);
 

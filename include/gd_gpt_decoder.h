@@ -141,6 +141,16 @@ typedef struct gd_gpt_sampling {
     uint64_t rng_state;
 } gd_gpt_sampling;
 
+/* The sampled form of gd_gpt_decoder_resident_begin, for callers that drive the session themselves
+ * (gd_gpt_decoder_generate is prefill + this + run + end).  It starts from the logits the last
+ * gd_gpt_decoder_prefill left on the device: ids / cu are the rows' histories so far (normally that prefill's
+ * prompts; the repetition penalty looks at them), max_picks counts picks, the first of which is made on those
+ * logits, so at most max_picks - 1 decode steps can run.  run / sync / end as for a greedy session; end returns
+ * one record per pick and row: the token appended to the row's history, or -1 for a row that has ended.  flags:
+ * GD_GPT_RESIDENT_HOLD_POSITIONS, GD_GPT_RESIDENT_UNFUSED. */
+gd_status gd_gpt_decoder_resident_begin_sampled(gd_gpt_decoder *dec, const int32_t *ids, const int32_t *cu,
+                                                int32_t max_picks, int32_t flags, const gd_gpt_sampling *sampling);
+
 uint64_t gd_gpt_generation_rng(uint64_t seed, int32_t n_prompts, uint64_t step);
 gd_status gd_gpt_decoder_generate(gd_gpt_decoder *dec, const int32_t *ids, const int32_t *cu, int32_t max_new,
                                   const gd_gpt_sampling *sampling, int32_t *out_tokens, int32_t *out_counts);

@@ -145,7 +145,11 @@ gd_status gd_backend_copy(gd_backend *b, gd_backend_buffer *dst, size_t dst_offs
     return GD_OK;
 }
 
-size_t gd_backend_sample_state_count(uint32_t rows) { return 8u + 8u * (size_t)rows; }
+size_t gd_backend_sample_state_count(uint32_t rows) { return 8u + 10u * (size_t)rows; }
+size_t gd_backend_sample_work_count(uint32_t rows, uint32_t cols)
+{
+    return (((size_t)rows * cols + 1u) & ~(size_t)1u) + 2u * (size_t)rows * (((size_t)cols + 2047u) / 2048u) * 258u;
+}
 
 gd_status gd_backend_device_info(const gd_backend *b, char *name, size_t name_bytes, int32_t *compute_units,
                                  uint64_t *global_mem)

@@ -979,10 +979,10 @@ def test_sample_advance_follows_the_reference_sampler(backend, arena, oracle, gd
     finished = np.array([0, 0, 0, 0, 0, 1, 0, 0, 0], np.int32)
     state0 = 0x0123456789abcdef
     t = dict(history=arena.from_numpy(hist), hist_len=arena.from_numpy(hist_len), finished=arena.from_numpy(finished),
-             state=arena.alloc((8 + 8 * B,), gda.I32), work=arena.alloc((B * V,), gda.F32),
+             state=arena.alloc((8 + 10 * B,), gda.I32), work=arena.alloc((backend.sample_work_count(B, V),), gda.F32),
              ids=arena.alloc((B,), gda.I32), positions=arena.from_numpy(np.arange(B, dtype=np.int32) * 3),
              step_counters=arena.from_numpy(np.zeros(B, np.int32)), out_ids=arena.alloc((steps * B,), gda.I32))
-    words = np.zeros(8 + 8 * B, np.int32)
+    words = np.zeros(8 + 10 * B, np.int32)
     words[:4] = np.array([state0, state0], np.uint64).view(np.int32)
     t["state"].write(words)
     table = oracle.normal_f16((V, 64), 77)
@@ -1024,11 +1024,11 @@ def test_sample_advance_frequencies_and_draw_order(backend, arena, oracle, gda):
     row = np.array([2.0, 1.0, 0.0, -1.0, 3.0, -4.0], np.float16)
     logits = arena.from_numpy(np.tile(row, (B, 1)))
     t = dict(history=arena.alloc((B, 4), gda.I32), hist_len=arena.from_numpy(np.zeros(B, np.int32)),
-             finished=arena.from_numpy(np.zeros(B, np.int32)), state=arena.alloc((8 + 8 * B,), gda.I32),
-             work=arena.alloc((B * V,), gda.F32), ids=arena.alloc((B,), gda.I32),
+             finished=arena.from_numpy(np.zeros(B, np.int32)), state=arena.alloc((8 + 10 * B,), gda.I32),
+             work=arena.alloc((backend.sample_work_count(B, V),), gda.F32), ids=arena.alloc((B,), gda.I32),
              positions=arena.from_numpy(np.zeros(B, np.int32)), step_counters=arena.from_numpy(np.zeros(B, np.int32)),
              out_ids=arena.alloc((steps * B,), gda.I32))
-    words = np.zeros(8 + 8 * B, np.int32)
+    words = np.zeros(8 + 10 * B, np.int32)
     words[:4] = np.array([42, 42], np.uint64).view(np.int32)
     t["state"].write(words)
     zeros = np.zeros(B, np.int32)
@@ -1053,12 +1053,12 @@ def test_sample_advance_frequencies_and_draw_order(backend, arena, oracle, gda):
 def test_sample_advance_rejects_bad_arguments(backend, arena, gda):
     B, V = 2, 16
     ok = dict(history=arena.alloc((B, 4), gda.I32), hist_len=arena.alloc((B,), gda.I32), finished=arena.alloc((B,), gda.I32),
-              state=arena.alloc((8 + 8 * B,), gda.I32), work=arena.alloc((B * V,), gda.F32), ids=arena.alloc((B,), gda.I32),
+              state=arena.alloc((8 + 10 * B,), gda.I32), work=arena.alloc((backend.sample_work_count(B, V),), gda.F32), ids=arena.alloc((B,), gda.I32),
               positions=arena.alloc((B,), gda.I32), step_counters=arena.alloc((B,), gda.I32),
               out_ids=arena.alloc((3 * B,), gda.I32))
     logits = arena.alloc((B, V), gda.F16)
     for bad, status in ((dict(state=arena.alloc((8,), gda.I32)), gda.INVALID_ARGUMENT),
-                        (dict(work=arena.alloc((B * V - 1,), gda.F32)), gda.INVALID_ARGUMENT),
+                        (dict(work=arena.alloc((B * V,), gda.F32)), gda.INVALID_ARGUMENT),
                         (dict(work=arena.alloc((B * V,), gda.F16)), gda.UNSUPPORTED),
                         (dict(ids=arena.alloc((B + 1,), gda.I32)), gda.INVALID_ARGUMENT),
                         (dict(history=arena.alloc((B + 1, 4), gda.I32)), gda.INVALID_ARGUMENT),
@@ -1085,11 +1085,11 @@ def test_sample_advance_on_the_reference_samplers_golden_cases(backend, arena, o
         hist = np.zeros((B, H), np.int32)
         hist[:, :H - 1] = history
         t = dict(history=arena.from_numpy(hist), hist_len=arena.from_numpy(hist_len),
-                 finished=arena.from_numpy(np.zeros(B, np.int32)), state=arena.alloc((8 + 8 * B,), gda.I32),
-                 work=arena.alloc((B * V,), gda.F32), ids=arena.alloc((B,), gda.I32),
+                 finished=arena.from_numpy(np.zeros(B, np.int32)), state=arena.alloc((8 + 10 * B,), gda.I32),
+                 work=arena.alloc((backend.sample_work_count(B, V),), gda.F32), ids=arena.alloc((B,), gda.I32),
                  positions=arena.from_numpy(np.zeros(B, np.int32)), step_counters=arena.from_numpy(np.zeros(B, np.int32)),
                  out_ids=arena.alloc((B,), gda.I32))
-        words = np.zeros(8 + 8 * B, np.int32)
+        words = np.zeros(8 + 10 * B, np.int32)
         words[:2] = words[2:4] = z[f"{c}_rng"].view(np.int32)
         t["state"].write(words)
         backend.sample_advance(arena.from_numpy(logits.astype(np.float16)), t, temperature, min_p, penalty, softcap,
@@ -1106,7 +1106,7 @@ def test_sample_advance_on_the_reference_samplers_golden_cases(backend, arena, o
                     margin = float(top[1] - top[0])
                 assert margin < 1e-5, (c, r, got[r], tok, margin)
         assert int(t["state"].read()[:4].view(np.uint64)[0]) == int(z[f"{c}_rng_after"].view(np.uint64)[-1]), c
-        work = t["work"].read().reshape(B, V)
+        work = t["work"].read()[:B * V].reshape(B, V)
         want = z[f"{c}_logits_after"]
         same = (work == want) | (np.isnan(work) & np.isnan(want))
         assert np.all(same | (np.abs(work - want) <= 2e-6 * np.abs(want))), c
