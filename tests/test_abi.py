@@ -38,7 +38,7 @@ def test_library_exports_the_host_core_decoder_and_checkpoint_symbols(gda):
     """Every function the other public headers declare (host core, decoder, checkpoint reader) is exported too;
     functions defined in a header (static inline) are not library symbols."""
     lib = ctypes.CDLL(gda.LIB_PATH)
-    for header in ("gradients_infer.h", "gd_gpt_decoder.h", "gd_checkpoint.h"):
+    for header in ("gradients_infer.h", "gd_gpt_decoder.h", "gd_checkpoint.h", "gd_tokenizer.h"):
         text = open(os.path.join(ROOT, "include", header)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         text = re.sub(r"static inline[^{;]*\{.*?\n\}", "", text, flags=re.S)
@@ -47,7 +47,8 @@ def test_library_exports_the_host_core_decoder_and_checkpoint_symbols(gda):
         assert len(names) >= 7, header
         missing = [n for n in names if not hasattr(lib, n)]
         assert not missing, (header, missing)
-    for must in ("gd_gpt_decoder_load_checkpoint", "gd_checkpoint_read_metadata", "gd_checkpoint_open"):
+    for must in ("gd_gpt_decoder_load_checkpoint", "gd_checkpoint_read_metadata", "gd_checkpoint_open",
+                 "gd_gpt_decoder_generate", "gd_bpe_tokenizer_load", "gd_tokenizer_encode", "gd_tokenizer_decode"):
         assert hasattr(lib, must)
 
 
