@@ -166,6 +166,18 @@ size_t gd_gpt_state_bytes(const gd_gpt_config *c)
            pad256((size_t)c->batch * (size_t)c->d_model * 2U) + sampling + 4096U;
 }
 
+size_t gd_gpt_scratch_bytes(const gd_gpt_config *c, int32_t max_prefill_tokens)
+{
+    /* every operator output of every layer lives until the step ends (bump allocation): 13 d_model-wide and one
+     * 2 x hidden-wide F16 tensor per layer and row, each padded to 256 bytes; 10 % slack; one transient activation of
+     * the many-row swiglu path; logits, picks and records; 64 MiB for everything small */
+    const size_t rows = (size_t)(max_prefill_tokens > c->batch ? max_prefill_tokens : c->batch);
+    const size_t per_row = 2U * (13U * (size_t)c->d_model + 2U * (size_t)c->mlp_hidden) + 14U * 256U;
+    const size_t layers = rows * per_row * (size_t)c->n_layers;
+    return layers + layers / 10U + rows * ((size_t)c->d_model * 4U + (size_t)c->mlp_hidden * 2U) +
+           (size_t)c->batch * (size_t)c->vocab * 4U + ((size_t)64 << 20);
+}
+
 gd_status gd_gpt_decoder_create(gd_context *ctx, const gd_gpt_config *cfg, gd_gpt_decoder **out)
 {
     gd_gpt_decoder *d;

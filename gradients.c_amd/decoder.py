@@ -68,6 +68,8 @@ def lib():
         l.gd_gpt_params_bytes.argtypes = [C.POINTER(GptConfig)]
         l.gd_gpt_state_bytes.restype = C.c_size_t
         l.gd_gpt_state_bytes.argtypes = [C.POINTER(GptConfig)]
+        l.gd_gpt_scratch_bytes.restype = C.c_size_t
+        l.gd_gpt_scratch_bytes.argtypes = [C.POINTER(GptConfig), C.c_int32]
         l.gd_context_create.argtypes = [C.POINTER(MemoryConfig), C.POINTER(_vp)]
         l.gd_context_destroy.argtypes = [_vp]
         l.gd_context_destroy.restype = None
@@ -234,12 +236,7 @@ class GptDecoder:
         l = lib()
         rows = max(cfg.batch, max_prefill_tokens)
         if scratch_slot_bytes is None:
-            # every operator output of every layer lives until the step ends (bump allocation):
-            # 13 d_model-wide and one 2*hidden-wide F16 tensor per layer and row, 256-byte padded
-            per_row = 2 * (13 * cfg.d_model + 2 * cfg.mlp_hidden) + 14 * 256
-            # + one transient activation of the many-row swiglu path, 10 % slack
-            scratch_slot_bytes = (int(rows * per_row * cfg.n_layers * 1.1) + rows * (cfg.d_model * 4 + cfg.mlp_hidden * 2)
-                                  + cfg.batch * cfg.vocab * 4 + (64 << 20))
+            scratch_slot_bytes = l.gd_gpt_scratch_bytes(C.byref(cfg), rows)
         self.ctx = Context(l.gd_gpt_params_bytes(C.byref(cfg)), l.gd_gpt_state_bytes(C.byref(cfg)),
                            scratch_slot_bytes, data_slot_bytes=max(1 << 20, 16 * rows + (1 << 16)))
         h = _vp()

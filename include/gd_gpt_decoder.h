@@ -41,6 +41,8 @@ typedef struct gd_gpt_decoder gd_gpt_decoder;
 /* Bytes the params and state arenas need for this configuration (for gd_memory_config). */
 size_t gd_gpt_params_bytes(const gd_gpt_config *cfg);
 size_t gd_gpt_state_bytes(const gd_gpt_config *cfg);
+/* Bytes one scratch slot needs for a packed prefill of max_prefill_tokens rows (at least batch rows: a decode step). */
+size_t gd_gpt_scratch_bytes(const gd_gpt_config *cfg, int32_t max_prefill_tokens);
 
 /* Allocates weights in the params arena and caches in the state arena and initialises the weights
  * the way the reference example does (N(0,0.02) from a splitmix64 + Box-Muller stream seeded per

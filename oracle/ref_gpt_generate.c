@@ -13,7 +13,8 @@
  * Seed: argv[3] (decimal), the weight seed handed to gpt_lm_init.
  * Optional argv[4]: the freshly initialised model is also written there by the reference's own
  * gd_module_save_state (src/nn/module_io.c:700-800), which gives the loader tests a checkpoint that the
- * reference itself produced.  The model dimensions are the example's compile-time macros
+ * reference itself produced.  Optional argv[5]: a file whose bytes become the checkpoint's metadata blob
+ * (the tests pass the "key=value" lines the reference's trainer writes, examples/gpt_lm/main.c:1836-1864).  The model dimensions are the example's compile-time macros
  * (gpt_lm_shared.h:10-28); the Makefile also builds a small-dimension variant for that fixture.
  */
 #include "gpt_lm_shared.c"
@@ -38,7 +39,7 @@ int main(int argc, char **argv)
     uint64_t rng = 1U;
     int batch, steps, total = 0, b, i, s;
     gd_status st;
-    if (argc != 4 && argc != 5) die("usage: ref_gpt_generate <in> <out> <seed> [checkpoint to write]");
+    if (argc < 4 || argc > 6) die("usage: ref_gpt_generate <in> <out> <seed> [checkpoint to write [metadata file]]");
     f = fopen(argv[1], "rb");
     if (f == NULL || fread(head, sizeof(head[0]), 3U, f) != 3U) die("cannot read the input header");
     batch = head[0];
@@ -87,12 +88,27 @@ int main(int argc, char **argv)
     }
     if (st != GD_OK) gpt_fail_status(ctx, st, "gd_context_create", __LINE__);
     gpt_lm_init(ctx, &model, &config);
-    if (argc == 5) {
+    if (argc >= 5) {
         static const char meta[] = "{\"writer\":\"gd_module_save_state\",\"model\":\"gpt_lm\"}";
         gd_module_save_options save = gd_module_save_options_default();
+        char *blob = NULL;
         save.metadata = meta;
         save.metadata_len = sizeof(meta) - 1U;
+        if (argc >= 6) {
+            FILE *m = fopen(argv[5], "rb");
+            long n;
+            if (m == NULL) die("cannot open the metadata file");
+            fseek(m, 0, SEEK_END);
+            n = ftell(m);
+            fseek(m, 0, SEEK_SET);
+            blob = (char *)calloc((size_t)n + 1U, 1U);
+            if (n < 0 || blob == NULL || fread(blob, 1U, (size_t)n, m) != (size_t)n) die("cannot read the metadata file");
+            fclose(m);
+            save.metadata = blob;
+            save.metadata_len = (size_t)n;
+        }
         TRY(ctx, gd_module_save_state(ctx, &model.mod, argv[4], &save));
+        free(blob);
     }
     TRY(ctx, gd_context_seal_params(ctx));
     TRY(ctx, gpt_lm_prepare_generation_cache(ctx, &model, &config, batch, GPT_CONTEXT_LENGTH, &cache));
