@@ -68,14 +68,15 @@ static gd_status dispatch(gd_backend *backend, const gd_backend_tensor_view *q, 
     p.unroll = backend->sdpa_unroll != 0 ? (uint32_t)backend->sdpa_unroll : 2u;
     p.nontemporal = backend->sdpa_nontemporal != 0 ? 1u : 0u;
     group = p.hq / p.hkv;
-    if (q->dtype == GD_BACKEND_DTYPE_F16 && p.tq == 1u && (p.dh == 64u || p.dh == 128u) && p.prefix_len == 0u &&
+    if (q->dtype == GD_BACKEND_DTYPE_F16 && p.tq == 1u && (p.dh == 64u || p.dh == 128u) &&
         (group == 1u || group == 2u || group == 4u || group == 8u) &&
         ((q->offset | k->offset | v->offset | out->offset) & 15u) == 0u && p.batch <= 65535u &&
         /* the kernel addresses the rows of one (batch row, kv head) with 24-bit factors and 32-bit byte offsets */
         p.tmax < (1u << 24) && (uint64_t)p.hkv * p.dh * 2u < (1u << 24) &&
         (uint64_t)p.tmax * p.hkv * p.dh * 2u < 0xffffffffull) {
-        /* longest key range a row can have */
+        /* longest run of visible keys a row can have: the window, plus the prefix in front of it */
         uint32_t span = p.window > 0u && p.window < p.tmax ? p.window : p.tmax;
+        if (p.window > 0u && p.prefix_len > 0u) span = span + p.prefix_len < p.tmax ? span + p.prefix_len : p.tmax;
         uint32_t chunk = (uint32_t)backend->sdpa_chunk;
         gd_status st;
         if (chunk == 0u) {

@@ -16,7 +16,7 @@
  *   - slots are merged with shuffles, wavefronts through LDS; with nsplit == 1 the result is
  *     normalised and stored as F16 directly, otherwise (max, sum, acc) partials go to a
  *     workspace and a small combine kernel finishes.
- * Everything else (F32 caches, Tq > 1, prefix masks, other head sizes) takes the generic
+ * Everything else (F32 caches, Tq > 1, other head sizes) takes the generic
  * kernel: one wavefront per query row, lane-per-key scores, lane-per-channel accumulation.
  *
  * Semantics (both kernels): live = min(pos + Tq, Tmax), query position pos + i, mask
@@ -103,7 +103,11 @@ __device__ __forceinline__ float gd_slot_max(float x)
     return gd_slot_reduce<N>(x, [](float a, float b) { return fmaxf(a, b); });
 }
 
-template <int D, int G, int WAVES, int UNROLL, bool NT>
+/* PFX: a prefix of always-visible keys in front of the window (prefix_len > 0).  The visible keys are then two
+ * runs, [0, a_len) and [b0, live); the kernel walks a virtual index over both (v < a_len: key v, else key
+ * v - a_len + b0) and the split of the range counts virtual indices.  Without PFX there is one run and the index is
+ * the key row itself. */
+template <int D, int G, int WAVES, int UNROLL, bool NT, bool PFX = false>
 __global__ void __launch_bounds__(WAVES * 64)
 gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__restrict__ kc,
                             const gd_half *__restrict__ vc, const int32_t *__restrict__ pos_ptr,
@@ -125,8 +129,12 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
     if (pos < 0) return;
     const int live = min(pos + 1, (int)p.tmax);
     const int first = p.window > 0u ? max(0, pos - (int)p.window + 1) : 0;
-    const int r0 = first + split * (int)p.chunk;
-    const int r1 = min(r0 + (int)p.chunk, live);
+    /* reference mask (metal_sdpa_decode.metal:25-52): a query inside the prefix sees the prefix keys that exist; one
+     * behind it sees the whole prefix plus its window (everything up to itself without a window) */
+    const int a_len = PFX ? min((int)p.prefix_len, live) : 0;
+    const int b0 = PFX ? (pos < (int)p.prefix_len ? live : min(max(a_len, first), live)) : first;
+    const int r0 = PFX ? split * (int)p.chunk : first + split * (int)p.chunk;
+    const int r1 = PFX ? min(r0 + (int)p.chunk, a_len + live - b0) : min(r0 + (int)p.chunk, live);
     float *ws_row = ws + (((size_t)b * p.hq + (size_t)hkv * G) * p.nsplit + split) * (D + 2);
     if (r0 >= r1) {
         if (p.nsplit > 1u) {
@@ -160,8 +168,11 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
     auto load_trip = [&](gd_half8 (&kv)[UNROLL], gd_half8 (&vv)[UNROLL], int s0) __attribute__((always_inline)) {
         uint32_t off[UNROLL];
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u)
-            off[u] = __umul24((uint32_t)min(s0 + u * KPB + slot, r1 - 1), pitch) + lane_off;
+        for (int u = 0; u < UNROLL; ++u) {
+            int row = min(s0 + u * KPB + slot, r1 - 1);
+            if (PFX) row = row < a_len ? row : row - a_len + b0;
+            off[u] = __umul24((uint32_t)row, pitch) + lane_off;
+        }
         /* every cache row is read exactly once per launch: optionally mark the loads streaming */
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
@@ -425,7 +436,16 @@ static int launch_split(hipStream_t stream, const void *q, const void *k, const 
             gd_sdpa_decode_split_kernel<D, G, W, U, false><<<grid, W * 64, 0, stream>>>(               \
                 (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, pos, (gd_half *)out, ws, p); \
     } while (0)
-    if constexpr (G == 1) {
+    if (p.prefix_len > 0u) {
+        /* one instantiation per wavefront count: the tunables for trip length and streaming loads do not apply */
+        constexpr int U = G == 1 ? 2 : 4;
+        if (G == 1 && p.waves == 8u)
+            gd_sdpa_decode_split_kernel<D, G, 8, U, false, true><<<grid, 8 * 64, 0, stream>>>(
+                (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, pos, (gd_half *)out, ws, p);
+        else
+            gd_sdpa_decode_split_kernel<D, G, 4, U, false, true><<<grid, 4 * 64, 0, stream>>>(
+                (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, pos, (gd_half *)out, ws, p);
+    } else if constexpr (G == 1) {
         if (p.waves == 8u && p.unroll == 8u) GD_GO(8, 8);
         else if (p.waves == 8u && p.unroll == 2u) GD_GO(8, 2);
         else if (p.waves == 8u) GD_GO(8, 4);

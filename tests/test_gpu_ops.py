@@ -308,8 +308,42 @@ def test_decode_position_past_cache_end_clamps(backend, arena, oracle):
     _decode_case(backend, arena, oracle, 2, 4, 4, 64, 40, np.array([40, 100], np.int32), 0.125, seed=400)
 
 
+@pytest.mark.parametrize("H,Hkv,D", [(8, 8, 64), (4, 1, 128), (6, 3, 64)])
+@pytest.mark.parametrize("window,prefix", [(0, 5), (16, 4), (7, 40), (300, 64), (1, 1), (64, 700)])
+def test_decode_prefix_and_window(backend, arena, oracle, H, Hkv, D, window, prefix):
+    """Always-visible prefix in front of a sliding window (reference mask metal_sdpa_decode.metal:25-52, range helpers
+    :55-84): queries inside the prefix, on its edge, behind it, far behind it (prefix and window apart) and past the
+    end of the cache; head layouts of the split-KV kernel and one of the generic kernel; with and without a split of
+    the visible keys."""
+    Tmax = 700
+    pos = np.array([0, 2, prefix - 1, prefix, prefix + 1, prefix + window, 333, 698, 699, 705, -1], np.int32)
+    pos = np.clip(pos, -1, 705)
+    B = pos.size
+    q = oracle.normal_f16((B, 1, H, D), 4100 + window)
+    k = oracle.normal_f16((B, Tmax, Hkv, D), 4101 + prefix)
+    v = oracle.normal_f16((B, Tmax, Hkv, D), 4102)
+    sentinel = np.full(q.shape, 7.0, np.float16)
+    tq, tk, tv, tp = arena.from_numpy(q), arena.from_numpy(k), arena.from_numpy(v), arena.from_numpy(pos)
+    want = oracle.sdpa_decode(q, k, v, pos, 0.11, window, prefix, out_init=sentinel.astype(np.float32))
+    for chunk in (0, 32, 96):
+        out = arena.from_numpy(sentinel)
+        backend.set_tunable("sdpa_chunk", chunk)
+        try:
+            backend.sdpa_decode_positions(tq, tk, tv, tp, out, 0.11, window, prefix)
+        finally:
+            backend.set_tunable("sdpa_chunk", 0)
+        _close(out.read(), want)
+    # the prefix really is visible: a key inside it with a huge score owns the output of a row far behind it
+    if prefix >= 2 and window > 0 and prefix + window < 333:
+        k2 = k.copy()
+        k2[6, 1] = (q[6, 0, :Hkv] * 40).astype(np.float16) if H == Hkv else k2[6, 1]
+        out = arena.from_numpy(sentinel)
+        backend.sdpa_decode_positions(tq, arena.from_numpy(k2), tv, tp, out, 0.11, window, prefix)
+        _close(out.read(), oracle.sdpa_decode(q, k2, v, pos, 0.11, window, prefix, out_init=sentinel.astype(np.float32)))
+
+
 def test_decode_generic_paths(backend, arena, oracle):
-    """prefix masks, Tq > 1 and odd head sizes take the generic kernel."""
+    """Tq > 1, odd head sizes and F32 caches take the generic kernel (prefix masks too when the head size is odd)."""
     rng_seed = 500
     for (Tq, D, window, prefix) in [(1, 64, 0, 3), (1, 64, 4, 2), (3, 64, 0, 0), (2, 40, 5, 0), (1, 72, 0, 0)]:
         B, H, Hkv, Tmax = 3, 4, 2, 70
