@@ -79,6 +79,11 @@ class FusedLinearArgs(C.Structure):
                 ("epilogue", C.c_uint32)]
 
 
+class MinimaxArgs(C.Structure):  # gd_backend_minimax_m3_sparse_args
+    _fields_ = [("scale", C.c_float), ("block_size", C.c_uint32), ("topk", C.c_uint32), ("init_blocks", C.c_uint32),
+                ("local_blocks", C.c_uint32), ("max_seqlen", C.c_uint32)]
+
+
 class SampleArgs(C.Structure):  # gd_backend_sample_args
     _fields_ = [("temperature", C.c_float), ("min_p", C.c_float), ("repetition_penalty", C.c_float),
                 ("logits_softcap", C.c_float), ("stop_token", C.c_int32), ("pos_delta", C.c_int32)]
@@ -154,6 +159,8 @@ _SIGNATURES = {
                                          C.POINTER(RopeArgs), C.POINTER(FusedLinearArgs)],
     "gd_backend_argmax_advance": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, C.c_int32, _TV, _TV],
     "gd_backend_sample_advance": [_vp, _TV, C.POINTER(SampleTensors), C.POINTER(SampleArgs)],
+    "gd_backend_minimax_m3_index_topk": [_vp, _TV, _TV, _TV, _TV, C.POINTER(MinimaxArgs)],
+    "gd_backend_minimax_m3_sparse_attention": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, C.POINTER(MinimaxArgs)],
     "gd_backend_copy": [_vp, _vp, C.c_size_t, _vp, C.c_size_t, C.c_size_t],
     "gd_backend_timer_create": [_vp, C.POINTER(_vp)],
     "gd_backend_timer_start": [_vp],
@@ -505,6 +512,16 @@ class Backend:
         a = SampleArgs(temperature, min_p, repetition_penalty, logits_softcap, stop_token, pos_delta)
         st = self.call("gd_backend_sample_advance", logits.view(), C.byref(t), C.byref(a))
         _check(st, "gd_backend_sample_advance")
+
+    def minimax_m3_index_topk(self, q, k, cu, topk_idx, block, init_blocks=1, local_blocks=1, max_seqlen=None):
+        a = MinimaxArgs(1.0, block, topk_idx.shape[2], init_blocks, local_blocks, max_seqlen or q.shape[0])
+        _check(self.call("gd_backend_minimax_m3_index_topk", q.view(), k.view(), cu.view(), topk_idx.view(), C.byref(a)),
+               "gd_backend_minimax_m3_index_topk")
+
+    def minimax_m3_sparse_attention(self, q, k, v, cu, topk_idx, out, block, scale, max_seqlen=None):
+        a = MinimaxArgs(scale, block, topk_idx.shape[2], 0, 0, max_seqlen or q.shape[0])
+        _check(self.call("gd_backend_minimax_m3_sparse_attention", q.view(), k.view(), v.view(), cu.view(),
+                         topk_idx.view(), out.view(), C.byref(a)), "gd_backend_minimax_m3_sparse_attention")
 
     @staticmethod
     def sample_work_count(rows, cols):

@@ -2,7 +2,7 @@
  * Entry points of the reference's backend boundary (src/core/backend.h, src/core/backend_generated.h)
  * that are not on the inference decode path: training kernels (backward passes, losses, optimizer,
  * AMP, dropout), unary/binary operators the decoder does not call, batched matmuls, reductions,
- * permute/split, the MiniMax-M3 sparse attention.  The reference's core references all of them, so a
+ * permute/split, the backward pass of the MiniMax-M3 sparse attention.  The reference's core references all of them, so a
  * drop-in backend has to define them; like the reference's null backend
  * (src/backends/null/backend_null.c, src/backends/null/backend_generated.c) each one reports
  * GD_ERR_UNSUPPORTED and touches nothing.
@@ -48,8 +48,6 @@ GD_UNSUPPORTED_ENTRY(gd_backend_lm_cross_entropy_finalize)
 GD_UNSUPPORTED_ENTRY(gd_backend_lm_cross_entropy_online_update)
 GD_UNSUPPORTED_ENTRY(gd_backend_lm_cross_entropy_reduce_normalize)
 GD_UNSUPPORTED_ENTRY(gd_backend_matmul_tn)
-GD_UNSUPPORTED_ENTRY(gd_backend_minimax_m3_index_topk)
-GD_UNSUPPORTED_ENTRY(gd_backend_minimax_m3_sparse_attention)
 GD_UNSUPPORTED_ENTRY(gd_backend_minimax_m3_sparse_attention_backward)
 GD_UNSUPPORTED_ENTRY(gd_backend_mse_backward)
 GD_UNSUPPORTED_ENTRY(gd_backend_mse_forward)

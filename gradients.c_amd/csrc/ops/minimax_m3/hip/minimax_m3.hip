@@ -1,0 +1,216 @@
+/*
+ * MiniMax-M3 block-sparse attention over packed sequences for gfx950, forward only: the block picker
+ * ("lightning indexer") and the attention over the picked blocks.  Semantics restate the reference's
+ * Metal kernels src/ops/minimax_m3_index_topk/metal_minimax_m3_index_topk.metal:20-137 and
+ * src/ops/minimax_m3_sparse_attention/metal_minimax_m3_sparse_attention.metal:36-113.
+ *
+ * Both kernels give every query row its own thread, as every row has its own list of blocks: q lives in
+ * registers as F16 pairs (products of two halfs are exact in F32, so v_dot2_f32_f16 loses nothing), scores and
+ * the softmax state are F32.
+ *   picker     one workgroup = 128 consecutive rows of one (sequence, kv head); the keys of the blocks these
+ *              rows can see pass through LDS in tiles of 64 (every thread reads the same key: broadcast reads);
+ *              the topk list is a register array kept sorted by a branch-free carry pass
+ *   attention  64 rows per workgroup; every row walks its blocks in list order with an online softmax and reads
+ *              its K / V rows straight from global memory (neighbouring rows mostly share their blocks, so the
+ *              lines come from L2)
+ * Bounds: picker = flops of a causal Q K^T (vector unit, not the matrix cores: a first version); attention =
+ * rows x topk x block keys.
+ */
+#include "../../_shared/hip_device.h"
+
+#define GD_M3_MAX_DH 64
+#define GD_M3_MAX_TOPK 16
+#define GD_M3_PICK_ROWS 128
+#define GD_M3_PICK_TILE 64
+#define GD_M3_ATTN_ROWS 64
+#define GD_NEG_INF (-__builtin_inff())
+
+struct gd_m3_params {
+    uint32_t total, batch, hq, hkv, dh;
+    uint32_t max_seqlen, block, topk, init_blocks, local_blocks;
+    float scale;
+};
+
+/* q . k over DH halfs, q as pairs in registers, k as 16-byte chunks */
+template <int DH>
+__device__ __forceinline__ float gd_m3_dot(const gd_half2 (&q)[DH / 2], const gd_half *k)
+{
+    float d = 0.f;
+    if (DH % 8 == 0) {
+#pragma unroll
+        for (int c = 0; c < DH / 8; ++c) {
+            const gd_half8 kv = *reinterpret_cast<const gd_half8 *>(k + 8 * c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                d = __builtin_amdgcn_fdot2(q[4 * c + e], (gd_half2){kv[2 * e], kv[2 * e + 1]}, d, false);
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < DH / 2; ++c) d = __builtin_amdgcn_fdot2(q[c], (gd_half2){k[2 * c], k[2 * c + 1]}, d, false);
+    }
+    return d;
+}
+
+template <int DH>
+__global__ void __launch_bounds__(GD_M3_PICK_ROWS)
+gd_m3_index_topk_kernel(const gd_half *__restrict__ q, const gd_half *__restrict__ k, const int32_t *__restrict__ cu,
+                        int32_t *__restrict__ topk, gd_m3_params p)
+{
+    __shared__ __attribute__((aligned(16))) gd_half ks[GD_M3_PICK_TILE * DH];
+    const int tid = threadIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int start = cu[b], T = cu[b + 1] - start;
+    const int q0 = blockIdx.x * GD_M3_PICK_ROWS;
+    if (q0 >= T) return;
+    const int i = q0 + tid;
+    const bool active = i < T;
+    const int block = (int)p.block;
+    const int valid = active ? (i + block) / block : 0;
+    const int last_row = min(q0 + GD_M3_PICK_ROWS - 1, T - 1);
+    const int max_valid = (last_row + block) / block;
+    const int local_start = max(0, valid - (int)p.local_blocks);
+
+    gd_half2 qh[DH / 2];
+    {
+        const gd_half *qr = q + ((size_t)(start + (active ? i : 0)) * p.hkv + h) * DH;
+#pragma unroll
+        for (int c = 0; c < DH / 2; ++c) qh[c] = active ? (gd_half2){qr[2 * c], qr[2 * c + 1]} : (gd_half2){(gd_half)0.f, (gd_half)0.f};
+    }
+    float score[GD_M3_MAX_TOPK];
+    int32_t index[GD_M3_MAX_TOPK];
+#pragma unroll
+    for (int t = 0; t < GD_M3_MAX_TOPK; ++t) {
+        score[t] = GD_NEG_INF;
+        index[t] = -1;
+    }
+    for (int blk = 0; blk < max_valid; ++blk) {
+        const int k_begin = blk * block, k_end = min(k_begin + block, T);
+        float best = GD_NEG_INF;
+        for (int kb = k_begin; kb < k_end; kb += GD_M3_PICK_TILE) {
+            const int tile = min(GD_M3_PICK_TILE, k_end - kb);
+            __syncthreads(); /* the previous tile has been read */
+            for (int idx = tid; idx < tile * DH / 2; idx += GD_M3_PICK_ROWS) {
+                const int jj = idx / (DH / 2), c = idx % (DH / 2);
+                reinterpret_cast<gd_half2 *>(ks)[idx] =
+                    reinterpret_cast<const gd_half2 *>(k + ((size_t)(start + kb + jj) * p.hkv + h) * DH)[c];
+            }
+            __syncthreads();
+            if (blk < valid) {
+                const int visible = min(tile, i - kb + 1); /* keys j <= i */
+                for (int jj = 0; jj < visible; ++jj) best = fmaxf(best, gd_m3_dot<DH>(qh, ks + jj * DH));
+            }
+        }
+        if (blk < valid) {
+            /* fmaxf drops a NaN operand: a block whose every score is NaN stays at -inf, as in the reference.
+             * First blocks rank highest, the last visible ones next (also when they are first blocks). */
+            if (blk < (int)p.init_blocks) best = 1.0e30f;
+            if (p.local_blocks > 0u && blk >= local_start) best = 1.0e29f;
+            /* sorted insertion without branches: the candidate takes the first slot it beats; what it pushes
+             * out is carried down and takes every following slot (it came from further up, so it wins ties) */
+            float cs = best;
+            int32_t ci = blk;
+            bool carrying = false;
+#pragma unroll
+            for (int t = 0; t < GD_M3_MAX_TOPK; ++t) {
+                if (t < (int)p.topk) {
+                    const bool take = carrying || cs > score[t];
+                    const float os = score[t];
+                    const int32_t oi = index[t];
+                    score[t] = take ? cs : os;
+                    index[t] = take ? ci : oi;
+                    cs = take ? os : cs;
+                    ci = take ? oi : ci;
+                    carrying = carrying || take;
+                }
+            }
+        }
+    }
+    if (active) {
+        int32_t *out = topk + ((size_t)h * p.total + (size_t)(start + i)) * p.topk;
+#pragma unroll
+        for (int t = 0; t < GD_M3_MAX_TOPK; ++t) {
+            if (t < (int)p.topk) out[t] = t < valid ? index[t] : -1;
+        }
+    }
+}
+
+template <int DH>
+__global__ void __launch_bounds__(GD_M3_ATTN_ROWS)
+gd_m3_sparse_attention_kernel(const gd_half *__restrict__ q, const gd_half *__restrict__ k,
+                              const gd_half *__restrict__ v, const int32_t *__restrict__ cu,
+                              const int32_t *__restrict__ topk, gd_half *__restrict__ out, gd_m3_params p)
+{
+    const int hq = blockIdx.y, b = blockIdx.z;
+    const int start = cu[b], T = cu[b + 1] - start;
+    const int i = blockIdx.x * GD_M3_ATTN_ROWS + threadIdx.x;
+    if (i >= T) return;
+    const int hkv = hq / (int)(p.hq / p.hkv);
+    const size_t qg = (size_t)(start + i);
+    const gd_half *qr = q + (qg * p.hq + hq) * DH;
+    gd_half2 qh[DH / 2];
+#pragma unroll
+    for (int c = 0; c < DH / 2; ++c) qh[c] = (gd_half2){qr[2 * c], qr[2 * c + 1]};
+    float acc[DH];
+#pragma unroll
+    for (int c = 0; c < DH; ++c) acc[c] = 0.f;
+    float m = GD_NEG_INF, l = 0.f;
+    const float scale2 = p.scale * 1.4426950408889634f; /* softmax in the exp2 domain */
+    const int32_t *list = topk + ((size_t)hkv * p.total + qg) * p.topk;
+    for (uint32_t t = 0; t < p.topk; ++t) {
+        const int blk = list[t];
+        if (blk < 0) continue;
+        const int k_begin = blk * (int)p.block;
+        const int k_end = min(min(k_begin + (int)p.block, T), i + 1);
+        for (int j = k_begin; j < k_end; ++j) {
+            const size_t row = ((size_t)(start + j) * p.hkv + hkv) * DH;
+            const float s = gd_m3_dot<DH>(qh, k + row) * scale2;
+            const float mn = fmaxf(m, s);
+            const float corr = exp2f(m - mn), e = exp2f(s - mn); /* exp2(-inf) = 0 on the first key */
+            l = l * corr + e;
+            if (DH % 8 == 0) {
+#pragma unroll
+                for (int c = 0; c < DH / 8; ++c) {
+                    const gd_half8 vv = *reinterpret_cast<const gd_half8 *>(v + row + 8 * c);
+#pragma unroll
+                    for (int x = 0; x < 8; ++x) acc[8 * c + x] = fmaf(e, (float)vv[x], acc[8 * c + x] * corr);
+                }
+            } else {
+#pragma unroll
+                for (int c = 0; c < DH; ++c) acc[c] = fmaf(e, (float)v[row + c], acc[c] * corr);
+            }
+            m = mn;
+        }
+    }
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    gd_half *o = out + (qg * p.hq + hq) * DH;
+#pragma unroll
+    for (int c = 0; c < DH; ++c) o[c] = (gd_half)(acc[c] * inv);
+}
+
+#define GD_M3_DISPATCH(DH_VALUE, STATEMENT)     \
+    switch (DH_VALUE) {                         \
+    case 4: { constexpr int DH = 4; STATEMENT; break; }   \
+    case 8: { constexpr int DH = 8; STATEMENT; break; }   \
+    case 16: { constexpr int DH = 16; STATEMENT; break; } \
+    case 32: { constexpr int DH = 32; STATEMENT; break; } \
+    case 64: { constexpr int DH = 64; STATEMENT; break; } \
+    default: return (int)hipErrorInvalidValue;  \
+    }
+
+extern "C" int gd_hip_launch_m3_index_topk(hipStream_t stream, const void *q, const void *k, const int32_t *cu,
+                                           int32_t *topk, const gd_m3_params *p)
+{
+    const dim3 grid((p->max_seqlen + GD_M3_PICK_ROWS - 1u) / GD_M3_PICK_ROWS, p->hkv, p->batch);
+    GD_M3_DISPATCH(p->dh, (gd_m3_index_topk_kernel<DH><<<grid, GD_M3_PICK_ROWS, 0, stream>>>(
+                              (const gd_half *)q, (const gd_half *)k, cu, topk, *p)));
+    return (int)hipGetLastError();
+}
+
+extern "C" int gd_hip_launch_m3_sparse_attention(hipStream_t stream, const void *q, const void *k, const void *v,
+                                                 const int32_t *cu, const int32_t *topk, void *out,
+                                                 const gd_m3_params *p)
+{
+    const dim3 grid((p->max_seqlen + GD_M3_ATTN_ROWS - 1u) / GD_M3_ATTN_ROWS, p->hq, p->batch);
+    GD_M3_DISPATCH(p->dh, (gd_m3_sparse_attention_kernel<DH><<<grid, GD_M3_ATTN_ROWS, 0, stream>>>(
+                              (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, cu, topk, (gd_half *)out, *p)));
+    return (int)hipGetLastError();
+}

@@ -640,6 +640,118 @@ GDO_API void gdo_argmax_rows_f16(const uint16_t *logits, int64_t rows, int64_t c
     }
 }
 
+/* ---- MiniMax-M3 block-sparse attention over packed sequences --------------- */
+
+/* Block picker.  reference src/ops/minimax_m3_index_topk/metal_minimax_m3_index_topk.metal:20-137
+ * (the in-test model tests/test_minimax_m3_sparse_attention.c:145-213 states the same): row i of a
+ * sequence sees the blocks 0 .. i / block; a block's score is the largest q_i . k_j over its keys
+ * j <= i (NaN counts as -inf); the first init_blocks blocks score 1e30, the last local_blocks
+ * visible ones 1e29 (which also overrides 1e30); the topk best are kept in descending order, an equal
+ * score never displaces an earlier block; slots beyond the number of visible blocks, and slots no
+ * block with a score above -inf reached, hold -1.  q, k [N,H,Dh]; out [H,N,topk]. */
+GDO_API void gdo_minimax_m3_index_topk_f16(const uint16_t *q, const uint16_t *k, const int32_t *cu, int64_t B,
+                                           int64_t H, int64_t Dh, int64_t block, int64_t topk,
+                                           int64_t init_blocks, int64_t local_blocks, int32_t *out)
+{
+    const int64_t N = cu[B];
+    for (int64_t i = 0; i < H * N * topk; ++i) out[i] = -1;
+#pragma omp parallel for collapse(2) schedule(dynamic)
+    for (int64_t b = 0; b < B; ++b) {
+        for (int64_t h = 0; h < H; ++h) {
+            const int64_t start = cu[b], T = cu[b + 1] - cu[b];
+            double *score = (double *)malloc((size_t)topk * sizeof(double));
+            int32_t *idx = (int32_t *)malloc((size_t)topk * sizeof(int32_t));
+            for (int64_t i = 0; i < T; ++i) {
+                const int64_t valid = (i + block) / block;
+                const int64_t local_start = valid > local_blocks ? valid - local_blocks : 0;
+                for (int64_t t = 0; t < topk; ++t) {
+                    score[t] = -HUGE_VAL;
+                    idx[t] = -1;
+                }
+                for (int64_t blk = 0; blk < valid; ++blk) {
+                    const int64_t k0 = blk * block, k1 = k0 + block < T ? k0 + block : T;
+                    double best = -HUGE_VAL;
+                    for (int64_t j = k0; j < k1 && j <= i; ++j) {
+                        double dot = 0.0;
+                        for (int64_t c = 0; c < Dh; ++c)
+                            dot += h2d(q[((start + i) * H + h) * Dh + c]) * h2d(k[((start + j) * H + h) * Dh + c]);
+                        if (dot > best) best = dot;
+                    }
+                    if (blk < init_blocks) best = 1.0e30;
+                    if (local_blocks > 0 && blk >= local_start) best = 1.0e29;
+                    for (int64_t slot = 0; slot < topk; ++slot) {
+                        if (best > score[slot]) {
+                            for (int64_t move = topk - 1; move > slot; --move) {
+                                score[move] = score[move - 1];
+                                idx[move] = idx[move - 1];
+                            }
+                            score[slot] = best;
+                            idx[slot] = (int32_t)blk;
+                            break;
+                        }
+                    }
+                }
+                for (int64_t t = 0; t < topk; ++t) out[(h * N + start + i) * topk + t] = t < valid ? idx[t] : -1;
+            }
+            free(score);
+            free(idx);
+        }
+    }
+}
+
+/* Attention of every row over the keys j <= i of its listed blocks.  reference
+ * src/ops/minimax_m3_sparse_attention/metal_minimax_m3_sparse_attention.metal:36-113 (in-test models
+ * tests/test_minimax_m3_sparse_attention.c:231-288, 423-483): blocks are visited in list order, -1
+ * entries skipped, a block listed twice counts twice; q [N,Hq,Dh], k / v [N,Hkv,Dh], topk
+ * [Hkv,N,topk]; a row without visible keys gives zeros.  F64 softmax, one F16 rounding. */
+GDO_API void gdo_minimax_m3_sparse_attention_f16(const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                                                 const int32_t *cu, const int32_t *topk, int64_t B, int64_t Hq,
+                                                 int64_t Hkv, int64_t Dh, int64_t block, int64_t tk, float scale,
+                                                 uint16_t *out)
+{
+    const int64_t N = cu[B], group = Hq / Hkv;
+#pragma omp parallel for collapse(2) schedule(dynamic)
+    for (int64_t b = 0; b < B; ++b) {
+        for (int64_t hq = 0; hq < Hq; ++hq) {
+            const int64_t start = cu[b], T = cu[b + 1] - cu[b], hkv = hq / group;
+            double *acc = (double *)malloc((size_t)Dh * sizeof(double));
+            double *sc = (double *)malloc((size_t)(tk * block) * sizeof(double));
+            for (int64_t i = 0; i < T; ++i) {
+                const int32_t *list = topk + (hkv * N + start + i) * tk;
+                const uint16_t *qr = q + ((start + i) * Hq + hq) * Dh;
+                double m = -HUGE_VAL, l = 0.0;
+                int64_t n = 0;
+                for (int64_t t = 0; t < tk; ++t) {
+                    if (list[t] < 0) continue;
+                    const int64_t k0 = (int64_t)list[t] * block, k1 = k0 + block < T ? k0 + block : T;
+                    for (int64_t j = k0; j < k1 && j <= i; ++j) {
+                        double dot = 0.0;
+                        for (int64_t c = 0; c < Dh; ++c) dot += h2d(qr[c]) * h2d(k[((start + j) * Hkv + hkv) * Dh + c]);
+                        sc[n] = (double)scale * dot;
+                        if (sc[n] > m) m = sc[n];
+                        ++n;
+                    }
+                }
+                for (int64_t c = 0; c < Dh; ++c) acc[c] = 0.0;
+                n = 0;
+                for (int64_t t = 0; t < tk; ++t) {
+                    if (list[t] < 0) continue;
+                    const int64_t k0 = (int64_t)list[t] * block, k1 = k0 + block < T ? k0 + block : T;
+                    for (int64_t j = k0; j < k1 && j <= i; ++j) {
+                        const double e = exp(sc[n++] - m);
+                        l += e;
+                        for (int64_t c = 0; c < Dh; ++c) acc[c] += e * h2d(v[((start + j) * Hkv + hkv) * Dh + c]);
+                    }
+                }
+                for (int64_t c = 0; c < Dh; ++c)
+                    out[((start + i) * Hq + hq) * Dh + c] = gdo_f32_to_f16((float)(l > 0.0 ? acc[c] / l : 0.0));
+            }
+            free(acc);
+            free(sc);
+        }
+    }
+}
+
 /* ---- sampling front end (the step after the logits) ------------------------ */
 
 /* reference examples/gpt_lm/gpt_lm_shared.c:1322-1331 */

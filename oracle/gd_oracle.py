@@ -75,6 +75,8 @@ def _declare(l):
         "gdo_embedding_f16": [_vp, _vp, _i64, _i64, _i64, _vp],
         "gdo_argmax_rows_f16": [_vp, _i64, _i64, _vp, _vp],
         "gdo_logits_softcap": [_vp, _i64, _f32],
+        "gdo_minimax_m3_index_topk_f16": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
+        "gdo_minimax_m3_sparse_attention_f16": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _vp],
         "gdo_repetition_penalty": [_vp, _i64, _vp, _i64, _f32],
         "gdo_decoder_destroy": [_vp],
         "gdo_decoder_untie_lm_head": [_vp, _u64],
@@ -297,6 +299,27 @@ def argmax_rows(logits):
     gap = np.empty(rows, np.float32)
     lib().gdo_argmax_rows_f16(_p(logits), rows, cols, _p(ids), _p(gap))
     return ids, gap
+
+
+def minimax_m3_index_topk(q, k, cu, block, topk, init_blocks=1, local_blocks=1):
+    """q, k [N,H,Dh] F16, cu [B+1] -> block ids [H,N,topk]."""
+    q, k, cu = _c(q, np.float16), _c(k, np.float16), _c(cu, np.int32)
+    N, H, Dh = q.shape
+    out = np.empty((H, N, topk), np.int32)
+    lib().gdo_minimax_m3_index_topk_f16(_p(q), _p(k), _p(cu), cu.size - 1, H, Dh, block, topk, init_blocks,
+                                        local_blocks, _p(out))
+    return out
+
+
+def minimax_m3_sparse_attention(q, k, v, cu, topk_idx, block, scale):
+    """q [N,Hq,Dh], k / v [N,Hkv,Dh], topk_idx [Hkv,N,topk] -> out [N,Hq,Dh] F16."""
+    q, k, v = _c(q, np.float16), _c(k, np.float16), _c(v, np.float16)
+    cu, topk_idx = _c(cu, np.int32), _c(topk_idx, np.int32)
+    N, Hq, Dh = q.shape
+    out = np.empty((N, Hq, Dh), np.float16)
+    lib().gdo_minimax_m3_sparse_attention_f16(_p(q), _p(k), _p(v), _p(cu), _p(topk_idx), cu.size - 1, Hq, k.shape[1],
+                                              Dh, block, topk_idx.shape[2], scale, _p(out))
+    return out
 
 
 def logits_softcap(logits, cap):

@@ -27,6 +27,8 @@ GD_NULL_OP(gd_backend_linear)
 GD_NULL_OP(gd_backend_linear_nt)
 GD_NULL_OP(gd_backend_matmul)
 GD_NULL_OP(gd_backend_matmul_nt)
+GD_NULL_OP(gd_backend_minimax_m3_index_topk)
+GD_NULL_OP(gd_backend_minimax_m3_sparse_attention)
 GD_NULL_OP(gd_backend_qkv_rope_append)
 GD_NULL_OP(gd_backend_qkv_split_rope_forward)
 GD_NULL_OP(gd_backend_rand_uniform)

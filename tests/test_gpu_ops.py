@@ -1145,3 +1145,113 @@ def test_sample_advance_on_the_reference_samplers_golden_cases(backend, arena, o
         same = (work == want) | (np.isnan(work) & np.isnan(want))
         assert np.all(same | (np.abs(work - want) <= 2e-6 * np.abs(want))), c
         assert np.array_equal(t["hist_len"].read(), hist_len + 1)
+
+
+# ---- MiniMax-M3 block-sparse attention --------------------------------------------------------------------------
+
+def _minimax_golden():
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "minimax_cases.npz"))
+    for c in sorted({k.split("_")[0] for k in z.files}, key=lambda s: int(s[1:])):
+        B, Hq, Hkv, Dh, block, topk, init, local, given = (int(x) for x in z[f"{c}_head"])
+        N = int(z[f"{c}_cu"][-1])
+        yield dict(name=c, Hq=Hq, Hkv=Hkv, Dh=Dh, block=block, topk=topk, init=init, local=local, given=bool(given),
+                   scale=float(z[f"{c}_scale"][0]), cu=z[f"{c}_cu"], q=z[f"{c}_q"].view(np.float16).reshape(N, Hq, Dh),
+                   k=z[f"{c}_k"].view(np.float16).reshape(N, Hkv, Dh), v=z[f"{c}_v"].view(np.float16).reshape(N, Hkv, Dh),
+                   topk_ref=z[f"{c}_topk"], out_ref=z[f"{c}_out"])
+
+
+def _assert_same_blocks(oracle, got, want, q, k, cu, block, init, local, where):
+    """Identical lists, or the rows that differ hold blocks whose scores tie within 1e-3 (the device sums the
+    products in F32, the models in F64)."""
+    bad = np.argwhere((got != want).any(axis=2))
+    for h, n in bad:
+        b = int(np.searchsorted(cu, n, side="right") - 1)
+        i = int(n - cu[b])
+        qs = q[n, h].astype(np.float64)
+
+        def score(blk):
+            j0, j1 = cu[b] + blk * block, cu[b] + min(min((blk + 1) * block, cu[b + 1] - cu[b]), i + 1)
+            return float((k[j0:j1, h].astype(np.float64) @ qs).max())
+        diff = [(int(x), int(y)) for x, y in zip(got[h, n], want[h, n]) if x != y]
+        for x, y in diff:
+            assert x >= 0 and y >= 0 and abs(score(x) - score(y)) < 1e-3, f"{where}: head {h} row {n}: {got[h, n]} vs {want[h, n]}"
+
+
+def test_minimax_m3_reference_models_golden_cases(backend, arena, oracle, gda):
+    """The reference's in-test models (tests/golden/minimax_cases.npz; its own two forward cases and six seeded
+    shapes): block ids identical, attention within the reference test's 2.5e-3."""
+    for c in _minimax_golden():
+        N = c["q"].shape[0]
+        tq, tk, tv, tcu = (arena.from_numpy(c[n]) for n in ("q", "k", "v", "cu"))
+        idx = arena.from_numpy(np.full((c["Hkv"], N, c["topk"]), -9, np.int32))
+        if not c["given"]:
+            backend.minimax_m3_index_topk(tq, tk, tcu, idx, c["block"], c["init"], c["local"])
+            _assert_same_blocks(oracle, idx.read(), c["topk_ref"], c["q"], c["k"], c["cu"], c["block"], c["init"], c["local"],
+                                c["name"])
+        idx.write(c["topk_ref"])
+        out = arena.from_numpy(np.full((N, c["Hq"], c["Dh"]), 7.0, np.float16))
+        backend.minimax_m3_sparse_attention(tq, tk, tv, tcu, idx, out, c["block"], c["scale"])
+        assert np.abs(out.read().astype(np.float32) - c["out_ref"]).max() < 2.5e-3, c["name"]
+
+
+@pytest.mark.parametrize("lens,H,Hkv,Dh,block,topk,init,local", [
+    ([300, 17, 129, 1], 4, 4, 64, 128, 4, 1, 1),
+    ([700], 8, 2, 64, 64, 16, 1, 2),
+    ([257, 256, 255], 2, 2, 32, 32, 5, 0, 0),
+    ([1000, 40], 2, 1, 16, 8, 8, 3, 1),
+])
+def test_minimax_m3_matches_oracle(backend, arena, oracle, gda, lens, H, Hkv, Dh, block, topk, init, local):
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    N = int(cu[-1])
+    q = oracle.normal_f16((N, H, Dh), 7100 + Dh)
+    kq = oracle.normal_f16((N, Hkv, Dh), 7101)            # index q has the kv heads' count
+    k = oracle.normal_f16((N, Hkv, Dh), 7102)
+    v = oracle.normal_f16((N, Hkv, Dh), 7103)
+    tcu, tk = arena.from_numpy(cu), arena.from_numpy(k)
+    idx = arena.alloc((Hkv, N, topk), gda.I32)
+    backend.minimax_m3_index_topk(arena.from_numpy(kq), tk, tcu, idx, block, init, local, max_seqlen=max(lens))
+    want_idx = oracle.minimax_m3_index_topk(kq, k, cu, block, topk, init, local)
+    _assert_same_blocks(oracle, idx.read(), want_idx, kq, k, cu, block, init, local, "picker")
+    idx.write(want_idx)
+    out = arena.from_numpy(np.full((N, H, Dh), 7.0, np.float16))
+    scale = float(1.0 / np.sqrt(Dh))
+    backend.minimax_m3_sparse_attention(arena.from_numpy(q), tk, arena.from_numpy(v), tcu, idx, out, block, scale,
+                                        max_seqlen=max(lens))
+    _close(out.read(), oracle.minimax_m3_sparse_attention(q, k, v, cu, want_idx, block, scale))
+
+
+def test_minimax_m3_all_blocks_is_dense_causal_attention(backend, arena, oracle, gda):
+    lens = [100, 33]
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    N, H, Dh, block = int(cu[-1]), 4, 64, 8
+    q, k, v = (oracle.normal_f16((N, H, Dh), s) for s in (7200, 7201, 7202))
+    tq, tk, tv, tcu = (arena.from_numpy(a) for a in (q, k, v, cu))
+    idx = arena.alloc((H, N, 13), gda.I32)                 # 13 slots >= 13 blocks of the longest sequence
+    backend.minimax_m3_index_topk(tq, tk, tcu, idx, block, 0, 0)
+    out = arena.alloc((N, H, Dh), gda.F16)
+    backend.minimax_m3_sparse_attention(tq, tk, tv, tcu, idx, out, block, 0.125)
+    _close(out.read(), oracle.sdpa_varlen(q, k, v, cu, 0.125))
+
+
+def test_minimax_m3_rejects_bad_arguments(backend, arena, gda):
+    N, H, Dh = 16, 2, 16
+    q, k = arena.alloc((N, H, Dh), gda.F16), arena.alloc((N, H, Dh), gda.F16)
+    cu, idx = arena.from_numpy(np.array([0, N], np.int32)), arena.alloc((H, N, 4), gda.I32)
+    for bad in (dict(k=arena.alloc((N, 1, Dh), gda.F16)), dict(idx=arena.alloc((H, N + 1, 4), gda.I32)),
+                dict(idx=arena.alloc((H, N, 17), gda.I32)), dict(block=129), dict(block=0),
+                dict(q=arena.alloc((N, H, Dh), gda.F32))):
+        a = dict(q=q, k=k, cu=cu, idx=idx, block=8)
+        a.update(bad)
+        with pytest.raises(gda.GdError) as err:
+            backend.minimax_m3_index_topk(a["q"], a["k"], a["cu"], a["idx"], a["block"])
+        assert err.value.status == gda.INVALID_ARGUMENT, bad
+    with pytest.raises(gda.GdError) as err:
+        backend.minimax_m3_index_topk(arena.alloc((N, H, 24), gda.F16), arena.alloc((N, H, 24), gda.F16), cu, idx, 8)
+    assert err.value.status == gda.UNSUPPORTED
+    out = arena.alloc((N, H, Dh), gda.F16)
+    with pytest.raises(gda.GdError) as err:
+        backend.minimax_m3_sparse_attention(q, k, arena.alloc((N, H, 8), gda.F16), cu, idx, out, 8, 0.25)
+    assert err.value.status == gda.INVALID_ARGUMENT
+    with pytest.raises(gda.GdError) as err:
+        backend.minimax_m3_sparse_attention(q, k, k, cu, idx, out, 8, 0.0)
+    assert err.value.status == gda.INVALID_ARGUMENT

@@ -688,3 +688,77 @@ def test_sampler_equals_the_reference_sampler_on_golden_cases(oracle):
             drew += new_state != state
             state = new_state
         assert (drew > 0) == (np.isfinite(temperature) and temperature > 0), c
+
+
+# ---- MiniMax-M3 block-sparse attention (reference tests/test_minimax_m3_sparse_attention.c) -------------------
+
+def _minimax_cases():
+    import os
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "minimax_cases.npz"))
+    for c in sorted({k.split("_")[0] for k in z.files}, key=lambda s: int(s[1:])):
+        B, Hq, Hkv, Dh, block, topk, init, local, given = (int(x) for x in z[f"{c}_head"])
+        N = int(z[f"{c}_cu"][-1])
+        yield dict(name=c, B=B, Hq=Hq, Hkv=Hkv, Dh=Dh, block=block, topk=topk, init=init, local=local, given=bool(given),
+                   scale=float(z[f"{c}_scale"][0]), cu=z[f"{c}_cu"], q=z[f"{c}_q"].view(np.float16).reshape(N, Hq, Dh),
+                   k=z[f"{c}_k"].view(np.float16).reshape(N, Hkv, Dh), v=z[f"{c}_v"].view(np.float16).reshape(N, Hkv, Dh),
+                   topk_ref=z[f"{c}_topk"], out_ref=z[f"{c}_out"])
+
+
+def test_minimax_block_picker_and_attention_equal_the_reference_models(oracle):
+    """tests/golden/minimax_cases.npz: the reference's own ref_topk / ref_sparse_fwd / ref_sparse_fwd_gqa (its test
+    program's functions, run by oracle/_ref/ref_minimax) on its two forward test cases and six seeded shapes.  Block
+    ids must be identical; outputs within the reference test's own bound (2.5e-3 absolute, :677, 762)."""
+    n = 0
+    for c in _minimax_cases():
+        if not c["given"]:
+            got = oracle.minimax_m3_index_topk(c["q"], c["k"], c["cu"], c["block"], c["topk"], c["init"], c["local"])
+            assert np.array_equal(got, c["topk_ref"]), c["name"]
+        out = oracle.minimax_m3_sparse_attention(c["q"], c["k"], c["v"], c["cu"], c["topk_ref"], c["block"], c["scale"])
+        assert np.abs(out.astype(np.float32) - c["out_ref"]).max() < 2.5e-3, c["name"]
+        assert np.abs(out.astype(np.float32) - c["out_ref"]).max() < 1e-3 * max(1.0, np.abs(c["out_ref"]).max())
+        n += 1
+    assert n == 8
+
+
+def test_minimax_all_blocks_selected_is_dense_causal_attention(oracle):
+    """With at least as many slots as blocks every visible block is listed: the operator pair must then equal plain
+    causal attention over the packed sequences (sdpa_varlen of this oracle, pinned elsewhere against numpy / torch)."""
+    rng = np.random.default_rng(5)
+    lens = [19, 1, 40]
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    N, Hq, Hkv, Dh, block = int(cu[-1]), 4, 2, 16, 8
+    q = rng.normal(0, 1, (N, Hq, Dh)).astype(np.float16)
+    k = rng.normal(0, 1, (N, Hkv, Dh)).astype(np.float16)
+    v = rng.normal(0, 1, (N, Hkv, Dh)).astype(np.float16)
+    idx = oracle.minimax_m3_index_topk(k, k, cu, block, 5, 0, 0)          # 5 slots, at most 5 blocks per row
+    for b in range(3):
+        for i in range(lens[b]):
+            row = idx[0, cu[b] + i]
+            assert sorted(x for x in row if x >= 0) == list(range(i // block + 1))
+    sparse = oracle.minimax_m3_sparse_attention(q, k, v, cu, idx, block, 0.25)
+    dense = oracle.sdpa_varlen(q, k, v, cu, 0.25)
+    assert np.abs(sparse.astype(np.float32) - dense.astype(np.float32)).max() < 2e-3
+
+
+def test_minimax_block_picker_priorities_and_ties(oracle):
+    # one sequence of 40 rows, block 4 -> 10 blocks; scores made explicit: q = e0, k_j = s_j * e0
+    block, T = 4, 40
+    scores = np.array([0.5, 3.0, 3.0, -1.0, 2.0, 9.0, 0.0, 1.0, 9.0, 4.0], np.float32)   # per block
+    q = np.zeros((T, 1, 4), np.float16)
+    q[:, 0, 0] = 1.0
+    k = np.zeros((T, 1, 4), np.float16)
+    k[:, 0, 0] = np.repeat(scores, block)
+    cu = [0, T]
+    last = oracle.minimax_m3_index_topk(q, k, cu, block, 4, 0, 0)[0, T - 1].tolist()
+    assert last == [5, 8, 9, 1]                       # 9.0 twice: the earlier block first; 3.0 twice: block 1 wins
+    assert oracle.minimax_m3_index_topk(q, k, cu, block, 4, 2, 0)[0, T - 1].tolist() == [0, 1, 5, 8]   # forced first blocks
+    assert oracle.minimax_m3_index_topk(q, k, cu, block, 4, 2, 1)[0, T - 1].tolist() == [0, 1, 9, 5]   # then the local one
+    assert oracle.minimax_m3_index_topk(q, k, cu, block, 4, 0, 2)[0, T - 1].tolist() == [8, 9, 5, 1]
+    row5 = oracle.minimax_m3_index_topk(q, k, cu, block, 4, 0, 0)[0, 5].tolist()
+    assert row5 == [1, 0, -1, -1]                     # row 5 sees blocks 0 and 1 only
+    # a block that is both first and local ranks as local (1e29 after 1e30): visible in the order of rows in block 0
+    assert oracle.minimax_m3_index_topk(q, k, cu, block, 2, 1, 1)[0, 2].tolist() == [0, -1]
+    assert oracle.minimax_m3_index_topk(q, k, cu, block, 2, 1, 1)[0, 9].tolist() == [0, 2]
+    k[:, 0, 0] = np.nan                               # NaN scores: nothing is picked unless forced
+    assert oracle.minimax_m3_index_topk(q, k, cu, block, 3, 0, 0)[0, T - 1].tolist() == [-1, -1, -1]
+    assert oracle.minimax_m3_index_topk(q, k, cu, block, 3, 1, 1)[0, T - 1].tolist() == [0, 9, -1]
