@@ -140,6 +140,11 @@ gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t 
         backend->sdpa_chunk = (int)value;
         return GD_OK;
     }
+    if (strcmp(name, "m3_simple") == 0) {
+        if (value != 0 && value != 1) return GD_ERR_INVALID_ARGUMENT;
+        backend->m3_simple = (int)value;
+        return GD_OK;
+    }
     if (strcmp(name, "sdpa_nontemporal") == 0) {
         if (value != 0 && value != 1) return GD_ERR_INVALID_ARGUMENT;
         backend->sdpa_nontemporal = (int)value;

@@ -35,6 +35,7 @@ struct gd_backend {
     int sdpa_waves;      /* 4 or 8 wavefronts per workgroup (0 = default 8) */
     int sdpa_unroll;     /* 4 or 8 key-row loads in flight per lane (0 = default 8) */
     int sdpa_nontemporal; /* 1: streaming hint on the K/V loads */
+    int m3_simple;        /* 1: MiniMax-M3 operators always take the per-row kernels (tests compare the two paths) */
     int linear_tiles;    /* few-row projections: 16-column tiles per workgroup, 1 / 2 / 4 (0 = automatic) */
     int linear_waves;    /* few-row projections: wavefronts per workgroup = K split, 4 / 8 (0 = automatic) */
 };

@@ -172,7 +172,8 @@ size_t gd_gpt_scratch_bytes(const gd_gpt_config *c, int32_t max_prefill_tokens)
      * 2 x hidden-wide F16 tensor per layer and row, each padded to 256 bytes; 10 % slack; one transient activation of
      * the many-row swiglu path; logits, picks and records; 64 MiB for everything small */
     const size_t rows = (size_t)(max_prefill_tokens > c->batch ? max_prefill_tokens : c->batch);
-    const size_t per_row = 2U * (13U * (size_t)c->d_model + 2U * (size_t)c->mlp_hidden) + 14U * 256U;
+    const size_t picked = c->m3_block_size > 0 ? (size_t)c->n_heads * 16U * 4U + 256U : 0U; /* block ids of a row */
+    const size_t per_row = 2U * (13U * (size_t)c->d_model + 2U * (size_t)c->mlp_hidden) + 14U * 256U + picked;
     const size_t layers = rows * per_row * (size_t)c->n_layers;
     return layers + layers / 10U + rows * ((size_t)c->d_model * 4U + (size_t)c->mlp_hidden * 2U) +
            (size_t)c->batch * (size_t)c->vocab * 4U + ((size_t)64 << 20);
@@ -189,7 +190,9 @@ gd_status gd_gpt_decoder_create(gd_context *ctx, const gd_gpt_config *cfg, gd_gp
     if (out != NULL) *out = NULL;
     if (ctx == NULL || cfg == NULL || out == NULL || cfg->vocab <= 0 || cfg->d_model <= 0 || cfg->n_layers <= 0 ||
         cfg->n_heads <= 0 || cfg->head_dim <= 0 || cfg->mlp_hidden <= 0 || cfg->max_seq <= 0 || cfg->batch <= 0 ||
-        cfg->n_heads * cfg->head_dim != cfg->d_model || cfg->sdpa_window < 0)
+        cfg->n_heads * cfg->head_dim != cfg->d_model || cfg->sdpa_window < 0 || cfg->m3_block_size < 0 ||
+        cfg->m3_block_size > 128 || cfg->m3_topk_blocks < 0 || cfg->m3_topk_blocks > 16 || cfg->m3_init_blocks < 0 ||
+        cfg->m3_local_blocks < 0 || (cfg->m3_block_size > 0 && cfg->head_dim > 64))
         return GD_ERR_INVALID_ARGUMENT;
     d = (gd_gpt_decoder *)calloc(1, sizeof(*d));
     if (d == NULL) return GD_ERR_OUT_OF_MEMORY;
@@ -601,7 +604,17 @@ static gd_status block_prefill(gd_gpt_decoder *d, int32_t l, const gd_tensor *x,
     TRY(linear_forward(ctx, &b->qkv_proj, &normed, &qkv));
     TRY(gd_qkv_split_rope(ctx, &qkv, positions, c->n_heads, c->head_dim, &rope, &q, &k, &v));
     TRY(gd_kv_cache_append_packed(ctx, &d->k_cache[l], &d->v_cache[l], cache_positions, cu, &k, &v));
-    TRY(gd_sdpa_varlen(ctx, &q, &k, &v, cu, &sdpa, &attn));
+    /* MiniMax-M3: picked blocks when the context is long enough for that to matter (reference :588-600, 918-933) */
+    if (c->m3_block_size > 0 && c->m3_topk_blocks > 0 && (int64_t)c->max_seq > (int64_t)c->m3_block_size * 8 &&
+        (int64_t)c->m3_block_size * c->m3_topk_blocks * 2 < (int64_t)c->max_seq) {
+        const gd_minimax_m3_sparse_config m3 = {0.0f, c->m3_block_size, c->m3_topk_blocks, c->m3_init_blocks,
+                                                c->m3_local_blocks, c->max_seq};
+        gd_tensor picked;
+        TRY(gd_minimax_m3_index_topk(ctx, &q, &k, cu, &m3, &picked));
+        TRY(gd_minimax_m3_sparse_attention(ctx, &q, &k, &v, cu, &picked, &m3, &attn));
+    } else {
+        TRY(gd_sdpa_varlen(ctx, &q, &k, &v, cu, &sdpa, &attn));
+    }
     TRY(gd_reshape(ctx, &attn, gd_shape_make(2U, flat_shape), &attn_flat));
     if (x->shape[0] >= 128) return block_tail_prefill(d, b, x, &attn_flat, out);
     return block_tail(d, b, x, &attn_flat, out);

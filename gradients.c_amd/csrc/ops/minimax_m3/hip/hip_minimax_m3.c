@@ -18,6 +18,37 @@ int gd_hip_launch_m3_index_topk(hipStream_t stream, const void *q, const void *k
 int gd_hip_launch_m3_sparse_attention(hipStream_t stream, const void *q, const void *k, const void *v,
                                       const int32_t *cu, const int32_t *topk, void *out, const gd_hip_m3_params *p);
 
+/* matrix-core kernels for head size 64 and block sizes that are multiples of 64 (minimax_m3_mfma.hip) */
+typedef struct gd_hip_m3f_params {
+    uint32_t n_rows, batch, hq, hkv;
+    uint32_t max_seqlen, block, topk, init_blocks, local_blocks;
+    float scale;
+} gd_hip_m3f_params;
+
+int gd_hip_launch_m3_mfma(hipStream_t stream, int picker, const void *q, const void *k, const void *v, const int32_t *cu,
+                          int32_t *topk, void *out, const gd_hip_m3f_params *p);
+
+static bool mfma_shape(const gd_backend *backend, const gd_hip_m3_params *p)
+{
+    const uint64_t rows = p->max_seqlen < p->total ? p->max_seqlen : p->total;
+    return backend->m3_simple == 0 && p->dh == 64u && (p->block % 64u) == 0u && (rows + p->block - 1u) / p->block <= 2048u &&
+           (uint64_t)p->total * p->hkv * 128u < 0xffffffffull && (uint64_t)p->total * p->hq * 128u < 0xffffffffull;
+}
+
+static void fast_params(const gd_hip_m3_params *p, gd_hip_m3f_params *f)
+{
+    f->n_rows = p->total;
+    f->batch = p->batch;
+    f->hq = p->hq;
+    f->hkv = p->hkv;
+    f->max_seqlen = p->max_seqlen;
+    f->block = p->block;
+    f->topk = p->topk;
+    f->init_blocks = p->init_blocks;
+    f->local_blocks = p->local_blocks;
+    f->scale = p->scale;
+}
+
 #define M3_MAX_DH 64
 #define M3_MAX_TOPK 16u
 #define M3_MAX_BLOCK 128u
@@ -74,6 +105,13 @@ gd_status gd_backend_minimax_m3_index_topk(gd_backend *backend, const gd_backend
         return GD_ERR_INVALID_ARGUMENT;
     if (!head_size_built(q->shape[2]) || ((q->offset | k->offset) & 15u) != 0u) return GD_ERR_UNSUPPORTED;
     fill(&p, q, k, cu, args);
+    if (mfma_shape(backend, &p)) {
+        gd_hip_m3f_params f;
+        fast_params(&p, &f);
+        return gd_hip_finish_op(backend, gd_hip_launch_m3_mfma(backend->stream, 1, gd_hip_view_ptr(q), gd_hip_view_ptr(k), NULL,
+                                                               (const int32_t *)gd_hip_view_ptr(cu),
+                                                               (int32_t *)gd_hip_view_ptr(topk), NULL, &f));
+    }
     return gd_hip_finish_op(backend, gd_hip_launch_m3_index_topk(backend->stream, gd_hip_view_ptr(q), gd_hip_view_ptr(k),
                                                                  (const int32_t *)gd_hip_view_ptr(cu),
                                                                  (int32_t *)gd_hip_view_ptr(topk), &p));
@@ -101,6 +139,13 @@ gd_status gd_backend_minimax_m3_sparse_attention(gd_backend *backend, const gd_b
     if (!head_size_built(q->shape[2]) || ((q->offset | k->offset | v->offset | out->offset) & 15u) != 0u)
         return GD_ERR_UNSUPPORTED;
     fill(&p, q, k, cu, args);
+    if (mfma_shape(backend, &p)) {
+        gd_hip_m3f_params f;
+        fast_params(&p, &f);
+        return gd_hip_finish_op(backend, gd_hip_launch_m3_mfma(backend->stream, 0, gd_hip_view_ptr(q), gd_hip_view_ptr(k),
+                                                               gd_hip_view_ptr(v), (const int32_t *)gd_hip_view_ptr(cu),
+                                                               (int32_t *)gd_hip_view_ptr(topk), gd_hip_view_ptr(out), &f));
+    }
     return gd_hip_finish_op(backend, gd_hip_launch_m3_sparse_attention(
         backend->stream, gd_hip_view_ptr(q), gd_hip_view_ptr(k), gd_hip_view_ptr(v), (const int32_t *)gd_hip_view_ptr(cu),
         (const int32_t *)gd_hip_view_ptr(topk), gd_hip_view_ptr(out), &p));

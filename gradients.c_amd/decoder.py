@@ -19,7 +19,8 @@ class GptConfig(C.Structure):  # gd_gpt_config
     _fields_ = [("vocab", C.c_int32), ("d_model", C.c_int32), ("n_layers", C.c_int32), ("n_heads", C.c_int32),
                 ("head_dim", C.c_int32), ("mlp_hidden", C.c_int32), ("max_seq", C.c_int32), ("batch", C.c_int32),
                 ("sdpa_window", C.c_int32), ("tie_lm_head", C.c_int32), ("rms_eps", C.c_float),
-                ("rope_theta", C.c_float), ("seed", C.c_uint64)]
+                ("rope_theta", C.c_float), ("seed", C.c_uint64), ("m3_block_size", C.c_int32),
+                ("m3_topk_blocks", C.c_int32), ("m3_init_blocks", C.c_int32), ("m3_local_blocks", C.c_int32)]
 
 
 class Span(C.Structure):  # gd_span
@@ -214,9 +215,11 @@ class Context:
 
 
 def gpt_config(vocab, d_model, n_layers, n_heads, head_dim, mlp_hidden, max_seq, batch, window=0, tie_lm_head=True,
-               seed=1000):
+               seed=1000, minimax_m3=None):
+    """minimax_m3: (block_size, topk_blocks, init_blocks, local_blocks) for the MiniMax-M3 architecture."""
+    m3 = tuple(minimax_m3) if minimax_m3 else (0, 0, 0, 0)
     return GptConfig(vocab, d_model, n_layers, n_heads, head_dim, mlp_hidden, max_seq, batch, window,
-                     int(tie_lm_head), 1e-5, 10000.0, seed)
+                     int(tie_lm_head), 1e-5, 10000.0, seed, *m3)
 
 
 def config_from_checkpoint(path, batch, max_seq=0, n_heads=0, head_dim=0, window=0, seed=1000):

@@ -422,7 +422,7 @@ gd_status gd_backend_argmax_advance(gd_backend *backend, const gd_backend_tensor
 /* MiniMax-M3 block-sparse attention over packed sequences, forward (reference src/core/backend.h:632-655; Metal
  * kernels metal_minimax_m3_index_topk.metal, metal_minimax_m3_sparse_attention.metal under src/ops).  All tensors
  * contiguous; q / k / v / out F16 [N, H, Dh] (Dh in {4, 8, 16, 32, 64}; other sizes up to 64, which the reference
- * accepts, are GD_ERR_UNSUPPORTED), cu_seqlens I32 [B+1], topk_idx I32 [Hkv, N, topk]; block_size <= 128,
+ * accepts, are GD_ERR_UNSUPPORTED; Dh = 64 with a block size of 64 or 128 runs on the matrix cores), cu_seqlens I32 [B+1], topk_idx I32 [Hkv, N, topk]; block_size <= 128,
  * topk <= 16; rows at or beyond max_seqlen inside their sequence are not processed.
  *   index_topk        index_q and index_k have the same number of heads.  Row i of a sequence sees blocks
  *                     0 .. i / block_size; a block's score is the largest q_i . k_j over its keys j <= i (NaN
@@ -530,7 +530,9 @@ gd_status gd_backend_device_info(const gd_backend *backend, char *name, size_t n
  * GD_HIP_SDPA_CHUNK); "sdpa_waves" (4 or 8 wavefronts per workgroup) and "sdpa_unroll" (2, 4 or 8
  * key-row loads per lane and trip) of the same kernel.  "linear_tiles" (1, 2 or 4 column tiles of 16
  * per workgroup) and "linear_waves" (4 or 8 wavefronts sharing the K range) of the few-row projection
- * kernel (environment: GD_HIP_LINEAR_TILES, GD_HIP_LINEAR_WAVES).  Unknown name -> GD_ERR_INVALID_ARGUMENT. */
+ * kernel (environment: GD_HIP_LINEAR_TILES, GD_HIP_LINEAR_WAVES).  "m3_simple" = 1: the MiniMax-M3 operators
+ * take their per-row kernels also where the matrix-core kernels apply (head size 64, block size a multiple of 64).
+ * Unknown name -> GD_ERR_INVALID_ARGUMENT. */
 gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t value);
 
 /* Raw device address of a buffer (base of the allocation). */

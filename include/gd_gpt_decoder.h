@@ -34,6 +34,12 @@ typedef struct gd_gpt_config {
     float rms_eps;       /* reference 1e-5 (gpt_lm_shared.h:58) */
     float rope_theta;    /* reference 10000 */
     uint64_t seed;
+    /* MiniMax-M3 architecture of the reference's example (gpt_lm_shared.h:29-40, 83; gpt_lm_shared.c:588-600,
+     * 918-933): with m3_block_size > 0 the packed prefill picks m3_topk_blocks key blocks per row (the first
+     * m3_init_blocks and the last m3_local_blocks forced) and attends over those, provided the context is long
+     * enough for that to matter (max_seq > 8 blocks and 2 x topk blocks < max_seq); the decode step is the dense
+     * one either way.  All zero: the plain architecture.  The reference's values: 128, 3, 1, 1. */
+    int32_t m3_block_size, m3_topk_blocks, m3_init_blocks, m3_local_blocks;
 } gd_gpt_config;
 
 typedef struct gd_gpt_decoder gd_gpt_decoder;

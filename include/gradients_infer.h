@@ -241,6 +241,25 @@ typedef struct gd_sdpa_varlen_config { /* ops.h:431-437 */
 gd_status gd_sdpa_varlen(gd_context *ctx, const gd_tensor *q, const gd_tensor *k, const gd_tensor *v,
                          const gd_tensor *cu_seqlens, const gd_sdpa_varlen_config *config, gd_tensor *out);
 
+/* MiniMax-M3 block picker + block-sparse attention over packed sequences (ops.h:383-413): index_q / index_k
+ * [N,H,Dh] give topk_idx I32 [H,N,topk] (scratch); sparse_attention attends over the keys j <= i of the listed
+ * blocks.  F16, Dh <= 64, block_size <= 128 (<= 0: 128), topk <= 16 (<= 0: 4), max_seqlen <= 0: N; a NULL
+ * configuration means one forced first and one forced last block. */
+typedef struct gd_minimax_m3_sparse_config { /* ops.h:390-397 */
+    float scale;
+    int32_t block_size;
+    int32_t topk;
+    int32_t init_blocks;
+    int32_t local_blocks;
+    int32_t max_seqlen;
+} gd_minimax_m3_sparse_config;
+gd_status gd_minimax_m3_index_topk(gd_context *ctx, const gd_tensor *index_q, const gd_tensor *index_k,
+                                   const gd_tensor *cu_seqlens, const gd_minimax_m3_sparse_config *config,
+                                   gd_tensor *topk_idx);
+gd_status gd_minimax_m3_sparse_attention(gd_context *ctx, const gd_tensor *q, const gd_tensor *k, const gd_tensor *v,
+                                         const gd_tensor *cu_seqlens, const gd_tensor *topk_idx,
+                                         const gd_minimax_m3_sparse_config *config, gd_tensor *out);
+
 typedef struct gd_sdpa_decode_config { /* ops.h:461-465 */
     float scale;
     int32_t sliding_window;

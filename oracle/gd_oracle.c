@@ -844,6 +844,9 @@ typedef struct gdo_decoder {
     uint16_t **w_down, **b_down;         /* [Hm,Dm], [Dm] */
     uint16_t **k_cache, **v_cache;       /* [B,Tmax,H,D] per layer */
     int32_t *pos;                        /* [B] live length of each sequence */
+    /* MiniMax-M3 architecture (reference gpt_lm_shared.c:588-600, 918-933): block_size > 0 switches the packed
+     * prefill to picked blocks when the context is long enough; the decode step stays dense */
+    int64_t m3_block, m3_topk, m3_init, m3_local;
 } gdo_decoder;
 
 static uint16_t *alloc_h(size_t n) { return (uint16_t *)calloc(n ? n : 1, sizeof(uint16_t)); }
@@ -995,10 +998,28 @@ static void attend_prefill(gdo_decoder *d, int64_t l, int64_t rows, const uint16
     gdo_kv_cache_append_packed((uint8_t *)d->k_cache[l], (uint8_t *)d->v_cache[l],
                                (const uint8_t *)k, (const uint8_t *)v, p->cache_pos, p->cu,
                                p->n_seq, rows, d->max_seq, H * D * 2);
+    if (d->m3_block > 0 && d->m3_topk > 0 && d->max_seq > d->m3_block * 8 && d->m3_block * d->m3_topk * 2 < d->max_seq) {
+        int32_t *idx = (int32_t *)malloc((size_t)(H * rows * d->m3_topk) * sizeof(int32_t));
+        gdo_minimax_m3_index_topk_f16(q, k, p->cu, p->n_seq, H, D, d->m3_block, d->m3_topk, d->m3_init, d->m3_local, idx);
+        gdo_minimax_m3_sparse_attention_f16(q, k, v, p->cu, idx, p->n_seq, H, H, D, d->m3_block, d->m3_topk,
+                                            (float)(1.0 / sqrt((double)D)), attn);
+        free(idx);
+        free(o);
+        return;
+    }
     gdo_sdpa_varlen_f16(q, k, v, p->cu, p->n_seq, H, H, D, (float)(1.0 / sqrt((double)D)), 1,
                         d->window, 0, d->max_seq, o);
     gdo_f32_to_f16_array(o, attn, (size_t)(rows * H * D));
     free(o);
+}
+
+GDO_API void gdo_decoder_set_minimax_m3(gdo_decoder *d, int64_t block, int64_t topk, int64_t init_blocks,
+                                        int64_t local_blocks)
+{
+    d->m3_block = block;
+    d->m3_topk = topk;
+    d->m3_init = init_blocks;
+    d->m3_local = local_blocks;
 }
 
 static void head_forward(gdo_decoder *d, int64_t rows, const uint16_t *x, uint16_t *logits)

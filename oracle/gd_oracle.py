@@ -80,6 +80,7 @@ def _declare(l):
         "gdo_repetition_penalty": [_vp, _i64, _vp, _i64, _f32],
         "gdo_decoder_destroy": [_vp],
         "gdo_decoder_untie_lm_head": [_vp, _u64],
+        "gdo_decoder_set_minimax_m3": [_vp, _i64, _i64, _i64, _i64],
         "gdo_decoder_step": [_vp, _vp, _vp, _vp, _vp],
         "gdo_decoder_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _vp],
     }
@@ -371,6 +372,10 @@ class Decoder:
                                            max_seq, batch, window, seed)
         if not tie_lm_head:
             lib().gdo_decoder_untie_lm_head(self._h, seed)
+
+    def set_minimax_m3(self, block, topk, init_blocks=1, local_blocks=1):
+        """MiniMax-M3 architecture: the packed prefill attends over picked blocks when the context is long enough."""
+        lib().gdo_decoder_set_minimax_m3(self._h, block, topk, init_blocks, local_blocks)
 
     def close(self):
         if self._h:

@@ -388,3 +388,47 @@ def test_generate_with_the_sampling_front_end(gda, oracle, params, stop, max_new
     finally:
         dev.close()
         ref.close()
+
+
+def test_minimax_m3_architecture_prefill_and_steps(gda, oracle):
+    """The reference's MiniMax-M3 architecture (gpt_lm_shared.c:588-600, 918-933): the packed prefill picks blocks and
+    attends over them, the decode step is the dense one.  Block size 8, 3 blocks per row (first and last forced),
+    context 128, so that the rule "context > 8 blocks and 2 x picked keys < context" holds; ragged prompts with a
+    sequence of one token, one inside the first block and two long ones."""
+    from gradients_c_amd import decoder as D
+    V, Dm, L, H, Dh, Hm, T, B = 256, 128, 2, 4, 32, 256, 128, 4
+    m3 = (8, 3, 1, 1)
+    dev = D.GptDecoder(D.gpt_config(V, Dm, L, H, Dh, Hm, T, B, 0, True, 77, minimax_m3=m3), max_prefill_tokens=B * T)
+    ref = oracle.Decoder(V, Dm, L, H, Dh, Hm, T, B, 0, 77, True)
+    ref.set_minimax_m3(*m3)
+    dense = oracle.Decoder(V, Dm, L, H, Dh, Hm, T, B, 0, 77, True)
+    try:
+        lens = [100, 1, 5, 90]
+        cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        prompt = oracle.uniform_i32(int(cu[-1]), 8, 0, V - 1)
+        lg_d, nx_d, gp_d = dev.prefill(prompt, cu)
+        lg_r, nx_r, gp_r = ref.prefill(prompt, cu)
+        lg_x, _, _ = dense.prefill(prompt, cu)
+        err = np.abs(lg_d.astype(np.float32) - lg_r.astype(np.float32)).max()
+        apart = np.abs(lg_x.astype(np.float32) - lg_r.astype(np.float32))
+        print("minimax prefill: worst difference", err, "dense vs picked blocks", apart.max(axis=1))
+        assert err < 4e-3
+        assert apart[0].max() > 0.02 and apart[3].max() > 0.02      # long rows: picked blocks are not the dense result
+        assert apart[1].max() < 1e-3 and apart[2].max() < 1e-3      # rows inside the first block: identical
+        for l in range(L):
+            got = dev.read_tensor("k_cache", l).reshape(B, T, H, Dh)[0, :100].astype(np.float32)
+            want = ref.tensor("k_cache", l).reshape(B, T, H, Dh)[0, :100].astype(np.float32)
+            assert np.abs(got - want).max() < 4e-3, l
+        near = _assert_ids(nx_d, nx_r, gp_d, gp_r, "minimax prefill")
+        tok = nx_r.copy()
+        for s in range(6):
+            lg_d, nx_d, gp_d = dev.step(tok)
+            lg_r, nx_r, gp_r = ref.step(tok)
+            assert np.abs(lg_d.astype(np.float32) - lg_r.astype(np.float32)).max() < 4e-3, s
+            near += _assert_ids(nx_d, nx_r, gp_d, gp_r, f"minimax step {s}")
+            tok = nx_r.copy()
+        print("near-ties:", near)
+    finally:
+        dev.close()
+        ref.close()
+        dense.close()

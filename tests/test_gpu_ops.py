@@ -1220,6 +1220,54 @@ def test_minimax_m3_matches_oracle(backend, arena, oracle, gda, lens, H, Hkv, Dh
     _close(out.read(), oracle.minimax_m3_sparse_attention(q, k, v, cu, want_idx, block, scale))
 
 
+@pytest.mark.parametrize("lens,H,Hkv,block,topk,init,local", [
+    ([300, 17, 129, 1, 640], 4, 4, 128, 4, 1, 1),
+    ([1500], 4, 2, 64, 16, 1, 2),
+    ([257, 256, 255, 64, 65], 2, 2, 64, 5, 0, 0),
+    ([2100, 40], 2, 1, 128, 3, 2, 0),
+])
+def test_minimax_m3_matrix_core_kernels(backend, arena, oracle, gda, lens, H, Hkv, block, topk, init, local):
+    """Head size 64 with block sizes 64 / 128 (the reference's M3 configuration) takes the matrix-core kernels: both
+    against the oracle, and the attention also against the per-row kernel on lists that repeat a block, name blocks
+    out of range or past the row, and leave slots empty (lists the picker never produces, the operator must take)."""
+    Dh = 64
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    N = int(cu[-1])
+    q = oracle.normal_f16((N, H, Dh), 7300 + block)
+    kq = oracle.normal_f16((N, Hkv, Dh), 7301)
+    k = oracle.normal_f16((N, Hkv, Dh), 7302)
+    v = oracle.normal_f16((N, Hkv, Dh), 7303)
+    tcu, tk, tq, tv = arena.from_numpy(cu), arena.from_numpy(k), arena.from_numpy(q), arena.from_numpy(v)
+    idx = arena.from_numpy(np.full((Hkv, N, topk), -9, np.int32))
+    backend.minimax_m3_index_topk(arena.from_numpy(kq), tk, tcu, idx, block, init, local, max_seqlen=max(lens))
+    want_idx = oracle.minimax_m3_index_topk(kq, k, cu, block, topk, init, local)
+    _assert_same_blocks(oracle, idx.read(), want_idx, kq, k, cu, block, init, local, "matrix-core picker")
+    scale = 0.125
+    idx.write(want_idx)
+    out = arena.from_numpy(np.full((N, H, Dh), 7.0, np.float16))
+    backend.minimax_m3_sparse_attention(tq, tk, tv, tcu, idx, out, block, scale, max_seqlen=max(lens))
+    _close(out.read(), oracle.minimax_m3_sparse_attention(q, k, v, cu, want_idx, block, scale))
+    # hand-made lists
+    rng = np.random.default_rng(block + topk)
+    odd = rng.integers(-1, max(lens) // block + 3, (Hkv, N, topk)).astype(np.int32)
+    odd[:, ::7, 0] = odd[:, ::7, topk - 1]                 # repeated blocks
+    idx.write(odd)
+    out2 = arena.from_numpy(np.full((N, H, Dh), 7.0, np.float16))
+    backend.minimax_m3_sparse_attention(tq, tk, tv, tcu, idx, out2, block, scale, max_seqlen=max(lens))
+    want = oracle.minimax_m3_sparse_attention(q, k, v, cu, odd, block, scale)
+    _close(out2.read(), want)
+    backend.set_tunable("m3_simple", 1)
+    try:
+        out3 = arena.from_numpy(np.full((N, H, Dh), 7.0, np.float16))
+        backend.minimax_m3_sparse_attention(tq, tk, tv, tcu, idx, out3, block, scale, max_seqlen=max(lens))
+        idx2 = arena.from_numpy(np.full((Hkv, N, topk), -9, np.int32))
+        backend.minimax_m3_index_topk(arena.from_numpy(kq), tk, tcu, idx2, block, init, local, max_seqlen=max(lens))
+    finally:
+        backend.set_tunable("m3_simple", 0)
+    _close(out3.read(), want)
+    _assert_same_blocks(oracle, idx2.read(), want_idx, kq, k, cu, block, init, local, "per-row picker")
+
+
 def test_minimax_m3_all_blocks_is_dense_causal_attention(backend, arena, oracle, gda):
     lens = [100, 33]
     cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
