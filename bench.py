@@ -216,6 +216,62 @@ def long_context_workload(a, pkg, oracle, D, which):
     print(json.dumps(line))
 
 
+def minimax_kernels(pkg, reps=10):
+    """gd_backend_minimax_m3_index_topk and gd_backend_minimax_m3_sparse_attention at the reference's M3 settings
+    (block 128, head size 64, first and last block forced) on packed sequences of uniform random values: the lists
+    the picker makes from such data differ from row to row (the worst case for the attention, which walks the union
+    of the lists of 128 rows), so the attention is also timed on lists that neighbouring rows share (first block, own
+    block and the blocks before it).  Dense causal attention over the same tensors for comparison.  Times per launch
+    from stream events around graph replays."""
+    be = pkg.Backend()
+    arena = be.buffer(1 << 30)
+    be.scope_begin()
+    tm = pkg.Timer(be)
+    results = []
+    for (B, T, H, topk) in ((8, 4096, 8, 4), (2, 16384, 8, 4)):
+        Dh, block = 64, 128
+        arena._top = 0
+        N = B * T
+        cu = arena.from_numpy((np.arange(B + 1) * T).astype(np.int32))
+        q, k, v, out = (arena.alloc((N, H, Dh), pkg.F16) for _ in range(4))
+        for n, t in enumerate((q, k, v)):
+            be.rand_uniform(t, 10 + n, -1.0, 1.0)
+        idx = arena.alloc((H, N, topk), pkg.I32)
+
+        def timed(fn):
+            fn()
+            be.graph_begin_capture()
+            for _ in range(reps):
+                fn()
+            graph = be.graph_end_capture()
+            ms = 0.0
+            for _ in range(2):
+                tm.start()
+                be.graph_launch(graph)
+                tm.stop()
+                ms = tm.elapsed_ms()
+            return ms * 1e3 / reps
+
+        pick = timed(lambda: be.minimax_m3_index_topk(q, k, cu, idx, block, 1, 1, max_seqlen=T))
+        attn = timed(lambda: be.minimax_m3_sparse_attention(q, k, v, cu, idx, out, block, 0.125, max_seqlen=T))
+        own = np.arange(T) // block
+        shared = np.stack([np.zeros(T, np.int64), own, own - 1, own - 2], 1)[:, :topk]
+        shared[:, 1:][shared[:, 1:] <= 0] = -1          # block 0 is listed once; nothing in front of the sequence
+        idx.write(np.tile(shared[None, None], (H, B, 1, 1)).reshape(H, N, topk).astype(np.int32))
+        attn_shared = timed(lambda: be.minimax_m3_sparse_attention(q, k, v, cu, idx, out, block, 0.125, max_seqlen=T))
+        dense = timed(lambda: be.sdpa_varlen(q, k, v, cu, out, 0.125, True, 0, 0, T))
+        pairs = B * H * (T * (T + 1) // 2)
+        results.append({"sequences": B, "tokens_each": T, "heads": H, "head_dim": Dh, "block": block, "topk": topk,
+                        "picker_us": round(pick, 1), "picker_tflops": round(2 * Dh * pairs / pick / 1e6, 1),
+                        "sparse_attention_random_lists_us": round(attn, 1),
+                        "sparse_attention_shared_lists_us": round(attn_shared, 1),
+                        "dense_causal_attention_us": round(dense, 1),
+                        "dense_tflops": round(4 * Dh * pairs / dense / 1e6, 1)})
+    be.close()
+    print(json.dumps({"metric": "MiniMax-M3 prefill attention kernels, time per launch", "unit": "us", "dtype": "f16",
+                      "data": "synthetic", "peak_tflops_f16_mfma": 2500.0, "results": results}))
+
+
 def sampled_workload(a, oracle, D):
     """The headline step (B=64, 511 cached tokens, positions held) with gd_backend_sample_advance after the LM head.
     Cache rows are allocated for 1024 tokens so that the rows' histories (prompt + sampled tokens, which the
@@ -268,6 +324,9 @@ def main():
                     help="the headline step with the sampling front end (soft cap 20, repetition penalty 1.3, "
                          "temperature 0.8, min-p 0.05) in place of the greedy pick; reported without roofline / "
                          "cpu_baseline objects")
+    ap.add_argument("--minimax-kernels", action="store_true",
+                    help="time the MiniMax-M3 block picker and block-sparse attention next to dense causal attention on "
+                         "packed sequences (auxiliary: prints its own JSON line, not the headline metric)")
     ap.add_argument("--kernel-only", action="store_true",
                     help="only launch sdpa_decode at the benchmark shape plus calibration copies (for --pmc runs)")
     a = ap.parse_args()
@@ -279,6 +338,9 @@ def main():
     pkg.lib()
     if a.kernel_only:
         kernel_only(pkg)
+        return
+    if a.minimax_kernels:
+        minimax_kernels(pkg)
         return
     from gradients_c_amd import decoder as D
     if a.workload != 2:
