@@ -300,6 +300,36 @@ gd_status gd_backend_kv_cache_append_packed(gd_backend *backend,
                                             const gd_backend_tensor_view *v_new,
                                             const gd_backend_kv_cache_append_args *args);
 
+/* MiniMax-M3 block-sparse attention over packed sequences, forward (reference src/core/backend.h:632-655; Metal
+ * kernels metal_minimax_m3_index_topk.metal, metal_minimax_m3_sparse_attention.metal under src/ops).  All tensors
+ * contiguous; q / k / v / out F16 [N, H, Dh] (Dh in {4, 8, 16, 32, 64}; other sizes up to 64, which the reference
+ * accepts, are GD_ERR_UNSUPPORTED; Dh = 64 with a block size of 64 or 128 runs on the matrix cores), cu_seqlens
+ * I32 [B+1], topk_idx I32 [Hkv, N, topk]; block_size <= 128,
+ * topk <= 16; rows at or beyond max_seqlen inside their sequence are not processed.
+ *   index_topk        index_q and index_k have the same number of heads.  Row i of a sequence sees blocks
+ *                     0 .. i / block_size; a block's score is the largest q_i . k_j over its keys j <= i (NaN
+ *                     counts as -inf); the first init_blocks blocks rank highest, the last local_blocks visible
+ *                     ones next; the topk best are stored in descending order, an equal score never displaces
+ *                     an earlier block; unused slots hold -1
+ *   sparse_attention  softmax(scale q_i . k_j) v_j over the keys j <= i of the row's listed blocks, query head
+ *                     hq using the list and the K / V of kv head hq / (Hq / Hkv); zeros when nothing is visible */
+typedef struct gd_backend_minimax_m3_sparse_args {
+    float scale;
+    uint32_t block_size, topk, init_blocks, local_blocks, max_seqlen;
+} gd_backend_minimax_m3_sparse_args;
+
+gd_status gd_backend_minimax_m3_index_topk(gd_backend *backend, const gd_backend_tensor_view *index_q,
+                                           const gd_backend_tensor_view *index_k,
+                                           const gd_backend_tensor_view *cu_seqlens,
+                                           const gd_backend_tensor_view *topk_idx,
+                                           const gd_backend_minimax_m3_sparse_args *args);
+gd_status gd_backend_minimax_m3_sparse_attention(gd_backend *backend, const gd_backend_tensor_view *q,
+                                                 const gd_backend_tensor_view *k, const gd_backend_tensor_view *v,
+                                                 const gd_backend_tensor_view *cu_seqlens,
+                                                 const gd_backend_tensor_view *topk_idx,
+                                                 const gd_backend_tensor_view *out,
+                                                 const gd_backend_minimax_m3_sparse_args *args);
+
 /* ---- part 4: entry points without a counterpart in the reference --------- */
 
 /* Greedy next token on the device.  The reference downloads the logits and
@@ -418,35 +448,6 @@ gd_status gd_backend_argmax_advance(gd_backend *backend, const gd_backend_tensor
                                     const gd_backend_tensor_view *out_ids, const gd_backend_tensor_view *out_gaps,
                                     int32_t pos_delta, const gd_backend_tensor_view *table,
                                     const gd_backend_tensor_view *next_x);
-
-/* MiniMax-M3 block-sparse attention over packed sequences, forward (reference src/core/backend.h:632-655; Metal
- * kernels metal_minimax_m3_index_topk.metal, metal_minimax_m3_sparse_attention.metal under src/ops).  All tensors
- * contiguous; q / k / v / out F16 [N, H, Dh] (Dh in {4, 8, 16, 32, 64}; other sizes up to 64, which the reference
- * accepts, are GD_ERR_UNSUPPORTED; Dh = 64 with a block size of 64 or 128 runs on the matrix cores), cu_seqlens I32 [B+1], topk_idx I32 [Hkv, N, topk]; block_size <= 128,
- * topk <= 16; rows at or beyond max_seqlen inside their sequence are not processed.
- *   index_topk        index_q and index_k have the same number of heads.  Row i of a sequence sees blocks
- *                     0 .. i / block_size; a block's score is the largest q_i . k_j over its keys j <= i (NaN
- *                     counts as -inf); the first init_blocks blocks rank highest, the last local_blocks visible
- *                     ones next; the topk best are stored in descending order, an equal score never displaces
- *                     an earlier block; unused slots hold -1
- *   sparse_attention  softmax(scale q_i . k_j) v_j over the keys j <= i of the row's listed blocks, query head
- *                     hq using the list and the K / V of kv head hq / (Hq / Hkv); zeros when nothing is visible */
-typedef struct gd_backend_minimax_m3_sparse_args {
-    float scale;
-    uint32_t block_size, topk, init_blocks, local_blocks, max_seqlen;
-} gd_backend_minimax_m3_sparse_args;
-
-gd_status gd_backend_minimax_m3_index_topk(gd_backend *backend, const gd_backend_tensor_view *index_q,
-                                           const gd_backend_tensor_view *index_k,
-                                           const gd_backend_tensor_view *cu_seqlens,
-                                           const gd_backend_tensor_view *topk_idx,
-                                           const gd_backend_minimax_m3_sparse_args *args);
-gd_status gd_backend_minimax_m3_sparse_attention(gd_backend *backend, const gd_backend_tensor_view *q,
-                                                 const gd_backend_tensor_view *k, const gd_backend_tensor_view *v,
-                                                 const gd_backend_tensor_view *cu_seqlens,
-                                                 const gd_backend_tensor_view *topk_idx,
-                                                 const gd_backend_tensor_view *out,
-                                                 const gd_backend_minimax_m3_sparse_args *args);
 
 /* Next-token sampling and the bookkeeping of a generation loop on the device, two launches.  What the
  * reference's example does on the host with the downloaded logits (examples/gpt_lm/gpt_lm_shared.c):
