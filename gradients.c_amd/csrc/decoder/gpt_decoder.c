@@ -508,6 +508,25 @@ gd_status gd_gpt_config_from_checkpoint(const char *path, gd_gpt_config *cfg)
     if (metadata_i32(blob, blob_len, "head_dim", &v)) cfg->head_dim = v;
     if (metadata_i32(blob, blob_len, "sdpa_window", &v)) cfg->sdpa_window = v;
     if (cfg->max_seq <= 0 && metadata_i32(blob, blob_len, "context_length", &v)) cfg->max_seq = v;
+    /* "architecture=minimax_m3" switches the packed prefill to picked blocks (the reference's inference programs
+     * read the same keys, infer.c:407-421); the other lines give the block size and counts */
+    {
+        static const char key[] = "architecture=minimax_m3";
+        size_t at = 0U;
+        bool m3 = false;
+        while (at < blob_len && !m3) {
+            size_t end = at;
+            while (end < blob_len && blob[end] != '\n') ++end;
+            m3 = end - at == sizeof(key) - 1U && strncmp(blob + at, key, sizeof(key) - 1U) == 0;
+            at = end < blob_len ? end + 1U : end;
+        }
+        if (m3) {
+            cfg->m3_block_size = metadata_i32(blob, blob_len, "minimax_m3_block_size", &v) && v > 0 ? v : 128;
+            cfg->m3_topk_blocks = metadata_i32(blob, blob_len, "minimax_m3_topk_blocks", &v) && v > 0 ? v : 3;
+            cfg->m3_init_blocks = metadata_i32(blob, blob_len, "minimax_m3_init_blocks", &v) ? v : 1;
+            cfg->m3_local_blocks = metadata_i32(blob, blob_len, "minimax_m3_local_blocks", &v) ? v : 1;
+        }
+    }
     free(blob);
     if (cfg->n_heads > 0 && cfg->head_dim <= 0 && cfg->d_model % cfg->n_heads == 0) cfg->head_dim = cfg->d_model / cfg->n_heads;
     if (cfg->head_dim > 0 && cfg->n_heads <= 0 && cfg->d_model % cfg->head_dim == 0) cfg->n_heads = cfg->d_model / cfg->head_dim;

@@ -81,7 +81,8 @@ gd_status gd_gpt_decoder_load_checkpoint(gd_gpt_decoder *dec, const char *path, 
  * programs size the model before loading (examples/gpt_lm/infer.c:344-432, 464-478): vocab, d_model, mlp_hidden
  * and n_layers from the directory (shapes of "gpt_lm.token_embedding" and "gpt_lm.blocks.0.down_proj.weight",
  * highest block index); n_heads, head_dim, sdpa_window and (only if cfg->max_seq <= 0) max_seq = context_length
- * from the "key=value" lines the reference's trainer stores as metadata (examples/gpt_lm/main.c:1836-1864).
+ * from the "key=value" lines the reference's trainer stores as metadata (examples/gpt_lm/main.c:1836-1864); a line
+ * "architecture=minimax_m3" also sets m3_* from the minimax_m3_* lines (defaults 128, 3, 1, 1).
  * Fields the file does not tell keep the caller's values (n_heads / head_dim given by the caller complete each
  * other through d_model); tie_lm_head is set (the reference ties).  GD_ERR_BAD_STATE if the expected tensors are
  * absent, if metadata and directory contradict each other, or if n_heads x head_dim != d_model at the end. */

@@ -371,6 +371,17 @@ def test_config_from_checkpoint(host, raw, tmp_path):
         dev.load_checkpoint(str(p))
     finally:
         dev.close()
+    # the second architecture of the reference's example
+    q = tmp_path / "m3.gdckpt"
+    q.write_bytes(with_metadata(raw, TRAINER_METADATA.replace(b"architecture=gpt\n", b"architecture=minimax_m3\n"
+                                b"minimax_m3_block_size=64\nminimax_m3_topk_blocks=4\nminimax_m3_init_blocks=2\n"
+                                b"minimax_m3_local_blocks=0\n")))
+    m3 = D.config_from_checkpoint(str(q), batch=1)
+    assert (m3.m3_block_size, m3.m3_topk_blocks, m3.m3_init_blocks, m3.m3_local_blocks) == (64, 4, 2, 0)
+    q.write_bytes(with_metadata(raw, TRAINER_METADATA.replace(b"architecture=gpt\n", b"architecture=minimax_m3\n")))
+    m3 = D.config_from_checkpoint(str(q), batch=1)
+    assert (m3.m3_block_size, m3.m3_topk_blocks, m3.m3_init_blocks, m3.m3_local_blocks) == (128, 3, 1, 1)
+    assert (cfg.m3_block_size, cfg.m3_topk_blocks) == (0, 0)
     # metadata that contradicts the directory
     for key, value in ((b"d_model=64", b"d_model=96"), (b"n_layers=2", b"n_layers=3"), (b"vocab_size=64", b"vocab_size=65"),
                        (b"mlp_hidden=128", b"mlp_hidden=64"), (b"n_heads=2", b"n_heads=3")):
