@@ -99,6 +99,16 @@ gd_status gd_checkpoint_read_metadata(const char *path, char **metadata_out, siz
         fclose(f);
         return GD_ERR_OUT_OF_MEMORY;
     }
+    {
+        /* a length that runs past the end of the file is the short read it would end in, found before the
+         * allocation: a damaged header cannot ask for more memory than the file holds */
+        off_t size;
+        if (fseeko(f, 0, SEEK_END) != 0 || (size = ftello(f)) < 0 || h.metadata_offset > (uint64_t)size ||
+            h.metadata_len > (uint64_t)size - h.metadata_offset) {
+            fclose(f);
+            return GD_ERR_IO;
+        }
+    }
     blob = (char *)malloc((size_t)h.metadata_len + 1U);
     if (blob == NULL) {
         fclose(f);
@@ -141,6 +151,8 @@ static gd_status read_directory(gd_checkpoint *c)
     if (h->tensor_count > (uint64_t)UINT32_MAX) return GD_ERR_INVALID_ARGUMENT;
     /* every entry takes at least its fixed part: a count the directory cannot hold is refused before allocating */
     if (h->tensor_count * (uint64_t)CKPT_ENTRY_FIXED_BYTES > h->dir_size) return GD_ERR_BAD_STATE;
+    /* a directory that runs past the end of the file is the short read it would end in, found before allocating */
+    if (h->dir_offset > c->file_size || h->dir_size > c->file_size - h->dir_offset) return GD_ERR_IO;
     c->count = (uint32_t)h->tensor_count;
     if (c->count == 0U) return h->dir_size == 0U ? GD_OK : GD_ERR_BAD_STATE;
     c->entries = (gd_checkpoint_entry *)calloc(c->count, sizeof(gd_checkpoint_entry));

@@ -487,11 +487,11 @@ gd_status gd_gpt_config_from_checkpoint(const char *path, gd_gpt_config *cfg)
         gd_checkpoint_close(ck);
         return GD_ERR_BAD_STATE;
     }
-    gd_checkpoint_close(ck);
     cfg->vocab = (int32_t)embed->shape[0];
     cfg->d_model = (int32_t)embed->shape[1];
     cfg->mlp_hidden = (int32_t)down->shape[0];
     cfg->n_layers = layers;
+    gd_checkpoint_close(ck); /* embed and down point into ck: nothing reads them past this line */
     cfg->tie_lm_head = 1;
     /* the metadata the reference's trainer writes (examples/gpt_lm/main.c:1836-1864) carries what shapes cannot
      * tell; where it repeats what the directory fixes, the two must agree */
@@ -671,6 +671,7 @@ gd_status gd_gpt_decoder_step(gd_gpt_decoder *d, const int32_t *ids, int32_t *ne
     gd_status st;
     int32_t l, b;
     if (d == NULL || ids == NULL) return GD_ERR_INVALID_ARGUMENT;
+    if (d->resident_open) return GD_ERR_BUSY;
     ctx = d->ctx;
     TRY(gd_begin_step(ctx, GD_SCOPE_INFER, gd_batch_empty()));
     st = data_i32(ctx, ids, d->cfg.batch, &t_ids);
@@ -700,6 +701,7 @@ gd_status gd_gpt_decoder_prefill(gd_gpt_decoder *d, const int32_t *ids, const in
     int32_t *positions, *zero, *last_rows;
     int32_t B, N, b, r, l;
     if (d == NULL || ids == NULL || cu == NULL) return GD_ERR_INVALID_ARGUMENT;
+    if (d->resident_open) return GD_ERR_BUSY;
     ctx = d->ctx;
     B = d->cfg.batch;
     N = cu[B];
@@ -1039,7 +1041,7 @@ static gd_status resident_begin_impl(gd_gpt_decoder *d, const int32_t *first_ids
     int64_t dims[1];
     int32_t b, zero = 0;
     if (d == NULL || (first_ids == NULL && sampling == NULL) || max_steps <= 0) return GD_ERR_INVALID_ARGUMENT;
-    if (d->resident_open) return GD_ERR_BAD_STATE;
+    if (d->resident_open) return GD_ERR_BUSY;
     ctx = d->ctx;
     be = gd_context_backend(ctx);
     for (b = 0; b < d->cfg.batch; ++b) {

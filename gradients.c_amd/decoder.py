@@ -330,20 +330,20 @@ class GptDecoder:
 
     def resident_begin(self, first_ids, max_steps, hold_positions=False, unfused=False):
         first = np.ascontiguousarray(first_ids, np.int32)
-        self._resident_max = max_steps
         flags = (1 if hold_positions else 0) | (2 if unfused else 0)
         self.ctx.check(lib().gd_gpt_decoder_resident_begin(self.handle, first.ctypes.data_as(_vp), max_steps, flags),
                        "gd_gpt_decoder_resident_begin")
+        self._resident_max = max_steps  # only a session that opened sizes what resident_end downloads
 
     def resident_begin_sampled(self, ids, cu, max_picks, temperature, min_p=0.0, repetition_penalty=1.0,
                                logits_softcap=0.0, stop_token=-1, rng_state=0, hold_positions=False, unfused=False):
         ids, cu = np.ascontiguousarray(ids, np.int32), np.ascontiguousarray(cu, np.int32)
-        self._resident_max = max_picks
         s = GptSampling(temperature, min_p, repetition_penalty, logits_softcap, stop_token, rng_state)
         flags = (1 if hold_positions else 0) | (2 if unfused else 0)
         self.ctx.check(lib().gd_gpt_decoder_resident_begin_sampled(self.handle, ids.ctypes.data_as(_vp),
                                                                    cu.ctypes.data_as(_vp), max_picks, flags, C.byref(s)),
                        "gd_gpt_decoder_resident_begin_sampled")
+        self._resident_max = max_picks
 
     def resident_run(self, n_steps):
         self.ctx.check(lib().gd_gpt_decoder_resident_run(self.handle, n_steps), "gd_gpt_decoder_resident_run")

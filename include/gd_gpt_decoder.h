@@ -107,7 +107,9 @@ gd_status gd_gpt_decoder_step(gd_gpt_decoder *dec, const int32_t *ids, int32_t *
  *   sync   waits for everything enqueued;
  *   end    closes the scope and downloads the tokens of all steps run so far: out_ids
  *          [steps, batch] and (may be NULL) out_gaps; steps_done (may be NULL) = rows written.
- * At most max_steps steps can run in a session.  flags:
+ * At most max_steps steps can run in a session (run beyond that: GD_ERR_INVALID_ARGUMENT); run, sync and end
+ * without an open session are GD_ERR_BAD_STATE.  While a session is open the decoder is busy: prefill, step,
+ * generate, load_checkpoint and another begin return GD_ERR_BUSY and change nothing.  flags:
  *   GD_GPT_RESIDENT_HOLD_POSITIONS  the cache positions do not advance: every step appends at the
  *                                   same row and attends over the same number of keys (used to time
  *                                   one fixed-shape step repeatedly);

@@ -186,8 +186,31 @@ gd_status gd_backend_timer_elapsed_ms(gd_backend_timer *t, float *ms)
     return GD_OK;
 }
 
-gd_status gd_backend_graph_begin_capture(gd_backend *b) { (void)b; return GD_ERR_UNSUPPORTED; }
-gd_status gd_backend_graph_end_capture(gd_backend *b, gd_backend_graph **out) { (void)b; (void)out; return GD_ERR_UNSUPPORTED; }
-gd_status gd_backend_graph_launch(gd_backend *b, gd_backend_graph *g) { (void)b; (void)g; return GD_ERR_UNSUPPORTED; }
-void gd_backend_graph_destroy(gd_backend_graph *g) { (void)g; }
+/* Graphs that record nothing: capture and replay succeed and are counted, so that the host logic of the resident
+ * sessions (step accounting, the order of calls, what a session refuses) runs without a device. */
+static int g_capturing;
+static uint64_t g_graph_launches;
+uint64_t gd_null_backend_graph_launches(void) { return g_graph_launches; }
+gd_status gd_backend_graph_begin_capture(gd_backend *b)
+{
+    if (b == NULL) return GD_ERR_INVALID_ARGUMENT;
+    if (g_capturing) return GD_ERR_BAD_STATE;
+    g_capturing = 1;
+    return GD_OK;
+}
+gd_status gd_backend_graph_end_capture(gd_backend *b, gd_backend_graph **out)
+{
+    if (b == NULL || out == NULL) return GD_ERR_INVALID_ARGUMENT;
+    if (!g_capturing) return GD_ERR_BAD_STATE;
+    g_capturing = 0;
+    *out = (gd_backend_graph *)calloc(1, sizeof(gd_backend_graph));
+    return *out != NULL ? GD_OK : GD_ERR_OUT_OF_MEMORY;
+}
+gd_status gd_backend_graph_launch(gd_backend *b, gd_backend_graph *g)
+{
+    if (b == NULL || g == NULL) return GD_ERR_INVALID_ARGUMENT;
+    ++g_graph_launches;
+    return GD_OK;
+}
+void gd_backend_graph_destroy(gd_backend_graph *g) { free(g); }
 #pragma GCC visibility pop

@@ -215,6 +215,7 @@ def test_reader_refuses_damaged_files(host, raw, tmp_path):
         ("data_past_end", put("<Q", e1["at"] + 80, size - 2), GD_ERR_BAD_STATE),
         ("path_repeated", rename_to_second, GD_ERR_BAD_STATE),
         ("nul_in_path", put("<B", e0["at"] + ENTRY_FIXED + 2, 0), GD_ERR_BAD_STATE),
+        ("dir_size_beyond_file", put("<Q", 32, 1 << 60), GD_ERR_IO),  # refused before anything is allocated for it
         ("cut_in_header", lambda d: d[:40], GD_ERR_IO),
         ("cut_in_magic", lambda d: d[:5], GD_ERR_IO),
         ("cut_in_directory", lambda d: d[:info["dir_off"] + 50], GD_ERR_IO),
@@ -245,7 +246,9 @@ def test_metadata_reader_checks_the_header_only(host, raw, tmp_path):
     assert C.string_at(blob, n.value + 1)[-1:] == b"\0"
     D._libc_free(blob)
     for name, edit, status in [("m_magic", put("<B", 0, 0x58), GD_ERR_BAD_STATE),
-                               ("m_cut", lambda d: d[:info["meta_off"] + 3], GD_ERR_IO)]:
+                               ("m_cut", lambda d: d[:info["meta_off"] + 3], GD_ERR_IO),
+                               ("m_len_beyond_file", put("<Q", 48, 1 << 60), GD_ERR_IO),
+                               ("m_offset_beyond_file", put("<Q", 40, 1 << 40), GD_ERR_BAD_STATE)]:
         p = damaged(tmp_path, raw, name, edit)
         assert D.lib().gd_checkpoint_read_metadata(p.encode(), C.byref(blob), C.byref(n)) == status, name
         assert not blob.value and n.value == 0

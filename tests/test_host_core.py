@@ -332,3 +332,56 @@ def test_decoder_weights_equal_the_oracle_without_a_gpu(host, oracle):
     finally:
         dev.close()
         ref.close()
+
+
+# ---- decoder: the accounting of a resident session, on the CPU ----------------------------------------------------
+
+def test_resident_sessions_count_steps_and_refuse_what_does_not_fit(host):
+    """The device-less backend records graphs that hold nothing and counts their replays, so the tokens mean
+    nothing here; what is held is the order of calls a session accepts, how many steps it lets run, and what the
+    decoder refuses while one is open."""
+    pkg, D = host
+    l = D.lib()
+    l.gd_null_backend_graph_launches.restype = C.c_uint64
+    cfg = D.gpt_config(96, 32, 2, 4, 8, 48, 32, 3, 0, True, 1000)
+    dev = D.GptDecoder(cfg, max_prefill_tokens=24)
+    ids, cu = np.arange(20, dtype=np.int32), np.array([0, 8, 9, 20], np.int32)
+    try:
+        with pytest.raises(pkg.GdError) as e:  # no session open
+            dev.resident_run(1)
+        assert e.value.status == BAD_STATE
+        dev.prefill(ids, cu)
+        before = l.gd_null_backend_graph_launches()
+        dev.resident_begin([1, 2, 3], 5)  # the first step runs inside begin
+        dev.resident_run(3)
+        assert l.gd_null_backend_graph_launches() == before + 3
+        with pytest.raises(pkg.GdError) as e:  # 1 + 3 + 2 > 5
+            dev.resident_run(2)
+        assert e.value.status == INVALID
+        for call in (lambda: dev.prefill(ids, cu), lambda: dev.step([1, 2, 3]), lambda: dev.generate(ids, cu, 4),
+                     lambda: dev.resident_begin([1, 2, 3], 2), lambda: dev.load_checkpoint("/nonexistent", True)):
+            with pytest.raises(pkg.GdError) as e:
+                call()
+            assert e.value.status == -4, "busy while a session is open"
+        dev.resident_run(1)
+        out, gaps = dev.resident_end()
+        assert out.shape == (5, 3)
+        assert list(dev.positions) == [8 + 5, 1 + 5, 11 + 5]
+        # a sampled session starts from the prefill's logits: its first pick costs no step
+        dev.prefill(ids, cu)
+        before = l.gd_null_backend_graph_launches()
+        dev.resident_begin_sampled(ids, cu, 6, 0.8, min_p=0.05, repetition_penalty=1.1, stop_token=5)
+        dev.resident_run(4)
+        assert l.gd_null_backend_graph_launches() == before + 4
+        with pytest.raises(pkg.GdError):
+            dev.resident_run(1)
+        out, _ = dev.resident_end()
+        assert out.shape == (6, 3)
+        # rows stop where the context ends: 32 - 11 = 21 tokens fit the longest row, whatever max_new asks
+        rows = dev.generate(ids, cu, 100, temperature=0.0)
+        assert [len(r) <= 32 - n for r, n in zip(rows, (8, 1, 11))] == [True] * 3
+        with pytest.raises(pkg.GdError) as e:  # empty prompt
+            dev.generate(ids, np.array([0, 0, 9, 20], np.int32), 4)
+        assert e.value.status == INVALID
+    finally:
+        dev.close()
