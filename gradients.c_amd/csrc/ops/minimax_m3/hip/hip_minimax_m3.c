@@ -2,8 +2,9 @@
  * Host dispatch of gd_backend_minimax_m3_index_topk and gd_backend_minimax_m3_sparse_attention.  Validation
  * restates the reference's src/ops/minimax_m3_index_topk/metal_minimax_m3_index_topk.m:74-104 and the matching
  * checks of metal_minimax_m3_sparse_attention.m: contiguous F16 [N,H,Dh] tensors, I32 cu [B+1] and topk
- * [Hkv,N,topk], head size <= 64, topk <= 16, block size <= 128.  Head sizes other than 4, 8, 16, 32, 64 are
- * GD_ERR_UNSUPPORTED here.
+ * [Hkv,N,topk], head size <= 64, topk <= 16, block size <= 128.  Head sizes 4, 8, 16, 32, 64 on 16-byte aligned
+ * operands take kernels of their own (size 64 with block sizes 64 / 128: the matrix cores); every other head size
+ * and alignment takes a half-by-half variant of the per-row kernels.
  */
 #include "../../../backends/hip/backend_hip_internal.h"
 
@@ -11,6 +12,7 @@ typedef struct gd_hip_m3_params {
     uint32_t total, batch, hq, hkv, dh;
     uint32_t max_seqlen, block, topk, init_blocks, local_blocks;
     float scale;
+    uint32_t unaligned; /* an operand starts off a 16-byte boundary */
 } gd_hip_m3_params;
 
 int gd_hip_launch_m3_index_topk(hipStream_t stream, const void *q, const void *k, const int32_t *cu, int32_t *topk,
@@ -31,7 +33,7 @@ int gd_hip_launch_m3_mfma(hipStream_t stream, int picker, const void *q, const v
 static bool mfma_shape(const gd_backend *backend, const gd_hip_m3_params *p)
 {
     const uint64_t rows = p->max_seqlen < p->total ? p->max_seqlen : p->total;
-    return backend->m3_simple == 0 && p->dh == 64u && (p->block % 64u) == 0u && (rows + p->block - 1u) / p->block <= 2048u &&
+    return backend->m3_simple == 0 && p->unaligned == 0u && p->dh == 64u && (p->block % 64u) == 0u && (rows + p->block - 1u) / p->block <= 2048u &&
            (uint64_t)p->total * p->hkv * 128u < 0xffffffffull && (uint64_t)p->total * p->hq * 128u < 0xffffffffull;
 }
 
@@ -65,8 +67,6 @@ static bool contiguous(const gd_backend_tensor_view *v)
     return true;
 }
 
-static bool head_size_built(int64_t dh) { return dh == 4 || dh == 8 || dh == 16 || dh == 32 || dh == 64; }
-
 static bool args_ok(const gd_backend_minimax_m3_sparse_args *a)
 {
     return a != NULL && a->topk > 0u && a->topk <= M3_MAX_TOPK && a->block_size > 0u && a->block_size <= M3_MAX_BLOCK &&
@@ -87,6 +87,7 @@ static void fill(gd_hip_m3_params *p, const gd_backend_tensor_view *q, const gd_
     p->init_blocks = a->init_blocks;
     p->local_blocks = a->local_blocks;
     p->scale = a->scale;
+    p->unaligned = 0u;
 }
 
 gd_status gd_backend_minimax_m3_index_topk(gd_backend *backend, const gd_backend_tensor_view *q,
@@ -103,8 +104,8 @@ gd_status gd_backend_minimax_m3_index_topk(gd_backend *backend, const gd_backend
         topk->shape[2] != (int64_t)args->topk || q->shape[0] > 0x7fffffff || q->shape[1] > 65535 ||
         cu->shape[0] - 1 > 65535)
         return GD_ERR_INVALID_ARGUMENT;
-    if (!head_size_built(q->shape[2]) || ((q->offset | k->offset) & 15u) != 0u) return GD_ERR_UNSUPPORTED;
     fill(&p, q, k, cu, args);
+    p.unaligned = ((q->offset | k->offset) & 15u) != 0u;
     if (mfma_shape(backend, &p)) {
         gd_hip_m3f_params f;
         fast_params(&p, &f);
@@ -136,9 +137,8 @@ gd_status gd_backend_minimax_m3_sparse_attention(gd_backend *backend, const gd_b
         topk->shape[2] != (int64_t)args->topk || q->shape[0] > 0x7fffffff || q->shape[1] > 65535 ||
         cu->shape[0] - 1 > 65535 || !(args->scale > 0.0f))
         return GD_ERR_INVALID_ARGUMENT;
-    if (!head_size_built(q->shape[2]) || ((q->offset | k->offset | v->offset | out->offset) & 15u) != 0u)
-        return GD_ERR_UNSUPPORTED;
     fill(&p, q, k, cu, args);
+    p.unaligned = ((q->offset | k->offset | v->offset | out->offset) & 15u) != 0u;
     if (mfma_shape(backend, &p)) {
         gd_hip_m3f_params f;
         fast_params(&p, &f);

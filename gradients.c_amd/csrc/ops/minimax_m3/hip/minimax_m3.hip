@@ -13,6 +13,10 @@
  *   attention  64 rows per workgroup; every row walks its blocks in list order with an online softmax and reads
  *              its K / V rows straight from global memory (neighbouring rows mostly share their blocks, so the
  *              lines come from L2)
+ * Head sizes 4, 8, 16, 32 and 64 have kernels of their own; any other size up to 64 (odd ones too), and any size
+ * whose operands do not start on 16-byte boundaries, runs the size-64 code with ANY set: q, the LDS key tiles and the accumulators are padded with zeros to 64, global rows
+ * keep their real stride and are read half by half.  The padding adds exact zeros, so results do not depend on
+ * which of the two paths a size takes.
  * Bounds: picker = flops of a causal Q K^T (vector unit, not the matrix cores: a first version); attention =
  * rows x topk x block keys.
  */
@@ -29,6 +33,7 @@ struct gd_m3_params {
     uint32_t total, batch, hq, hkv, dh;
     uint32_t max_seqlen, block, topk, init_blocks, local_blocks;
     float scale;
+    uint32_t unaligned; /* some operand does not start on a 16-byte boundary: take the half-by-half path */
 };
 
 /* q . k over DH halfs, q as pairs in registers, k as 16-byte chunks */
@@ -51,7 +56,20 @@ __device__ __forceinline__ float gd_m3_dot(const gd_half2 (&q)[DH / 2], const gd
     return d;
 }
 
+/* the same over a global row of dh <= DH halfs at any alignment; the missing tail counts as zeros */
 template <int DH>
+__device__ __forceinline__ float gd_m3_dot_any(const gd_half2 (&q)[DH / 2], const gd_half *k, int dh)
+{
+    float d = 0.f;
+#pragma unroll
+    for (int c = 0; c < DH / 2; ++c) {
+        const gd_half k0 = 2 * c < dh ? k[2 * c] : (gd_half)0.f, k1 = 2 * c + 1 < dh ? k[2 * c + 1] : (gd_half)0.f;
+        d = __builtin_amdgcn_fdot2(q[c], (gd_half2){k0, k1}, d, false);
+    }
+    return d;
+}
+
+template <int DH, bool ANY>
 __global__ void __launch_bounds__(GD_M3_PICK_ROWS)
 gd_m3_index_topk_kernel(const gd_half *__restrict__ q, const gd_half *__restrict__ k, const int32_t *__restrict__ cu,
                         int32_t *__restrict__ topk, gd_m3_params p)
@@ -69,11 +87,16 @@ gd_m3_index_topk_kernel(const gd_half *__restrict__ q, const gd_half *__restrict
     const int max_valid = (last_row + block) / block;
     const int local_start = max(0, valid - (int)p.local_blocks);
 
+    const int dh = ANY ? (int)p.dh : DH; /* halfs per row in global memory */
     gd_half2 qh[DH / 2];
     {
-        const gd_half *qr = q + ((size_t)(start + (active ? i : 0)) * p.hkv + h) * DH;
+        const gd_half *qr = q + ((size_t)(start + (active ? i : 0)) * p.hkv + h) * dh;
 #pragma unroll
-        for (int c = 0; c < DH / 2; ++c) qh[c] = active ? (gd_half2){qr[2 * c], qr[2 * c + 1]} : (gd_half2){(gd_half)0.f, (gd_half)0.f};
+        for (int c = 0; c < DH / 2; ++c) {
+            const gd_half q0v = active && 2 * c < dh ? qr[2 * c] : (gd_half)0.f;
+            const gd_half q1v = active && 2 * c + 1 < dh ? qr[2 * c + 1] : (gd_half)0.f;
+            qh[c] = (gd_half2){q0v, q1v};
+        }
     }
     float score[GD_M3_MAX_TOPK];
     int32_t index[GD_M3_MAX_TOPK];
@@ -88,10 +111,17 @@ gd_m3_index_topk_kernel(const gd_half *__restrict__ q, const gd_half *__restrict
         for (int kb = k_begin; kb < k_end; kb += GD_M3_PICK_TILE) {
             const int tile = min(GD_M3_PICK_TILE, k_end - kb);
             __syncthreads(); /* the previous tile has been read */
-            for (int idx = tid; idx < tile * DH / 2; idx += GD_M3_PICK_ROWS) {
-                const int jj = idx / (DH / 2), c = idx % (DH / 2);
-                reinterpret_cast<gd_half2 *>(ks)[idx] =
-                    reinterpret_cast<const gd_half2 *>(k + ((size_t)(start + kb + jj) * p.hkv + h) * DH)[c];
+            if (ANY) {
+                for (int idx = tid; idx < tile * DH; idx += GD_M3_PICK_ROWS) {
+                    const int jj = idx / DH, c = idx % DH;
+                    ks[idx] = c < dh ? k[((size_t)(start + kb + jj) * p.hkv + h) * dh + c] : (gd_half)0.f;
+                }
+            } else {
+                for (int idx = tid; idx < tile * DH / 2; idx += GD_M3_PICK_ROWS) {
+                    const int jj = idx / (DH / 2), c = idx % (DH / 2);
+                    reinterpret_cast<gd_half2 *>(ks)[idx] =
+                        reinterpret_cast<const gd_half2 *>(k + ((size_t)(start + kb + jj) * p.hkv + h) * DH)[c];
+                }
             }
             __syncthreads();
             if (blk < valid) {
@@ -133,7 +163,7 @@ gd_m3_index_topk_kernel(const gd_half *__restrict__ q, const gd_half *__restrict
     }
 }
 
-template <int DH>
+template <int DH, bool ANY>
 __global__ void __launch_bounds__(GD_M3_ATTN_ROWS)
 gd_m3_sparse_attention_kernel(const gd_half *__restrict__ q, const gd_half *__restrict__ k,
                               const gd_half *__restrict__ v, const int32_t *__restrict__ cu,
@@ -145,10 +175,12 @@ gd_m3_sparse_attention_kernel(const gd_half *__restrict__ q, const gd_half *__re
     if (i >= T) return;
     const int hkv = hq / (int)(p.hq / p.hkv);
     const size_t qg = (size_t)(start + i);
-    const gd_half *qr = q + (qg * p.hq + hq) * DH;
+    const int dh = ANY ? (int)p.dh : DH; /* halfs per row in global memory */
+    const gd_half *qr = q + (qg * p.hq + hq) * dh;
     gd_half2 qh[DH / 2];
 #pragma unroll
-    for (int c = 0; c < DH / 2; ++c) qh[c] = (gd_half2){qr[2 * c], qr[2 * c + 1]};
+    for (int c = 0; c < DH / 2; ++c)
+        qh[c] = (gd_half2){2 * c < dh ? qr[2 * c] : (gd_half)0.f, 2 * c + 1 < dh ? qr[2 * c + 1] : (gd_half)0.f};
     float acc[DH];
 #pragma unroll
     for (int c = 0; c < DH; ++c) acc[c] = 0.f;
@@ -161,12 +193,15 @@ gd_m3_sparse_attention_kernel(const gd_half *__restrict__ q, const gd_half *__re
         const int k_begin = blk * (int)p.block;
         const int k_end = min(min(k_begin + (int)p.block, T), i + 1);
         for (int j = k_begin; j < k_end; ++j) {
-            const size_t row = ((size_t)(start + j) * p.hkv + hkv) * DH;
-            const float s = gd_m3_dot<DH>(qh, k + row) * scale2;
+            const size_t row = ((size_t)(start + j) * p.hkv + hkv) * dh;
+            const float s = (ANY ? gd_m3_dot_any<DH>(qh, k + row, dh) : gd_m3_dot<DH>(qh, k + row)) * scale2;
             const float mn = fmaxf(m, s);
             const float corr = exp2f(m - mn), e = exp2f(s - mn); /* exp2(-inf) = 0 on the first key */
             l = l * corr + e;
-            if (DH % 8 == 0) {
+            if (ANY) {
+#pragma unroll
+                for (int c = 0; c < DH; ++c) acc[c] = fmaf(e, c < dh ? (float)v[row + c] : 0.f, acc[c] * corr);
+            } else if (DH % 8 == 0) {
 #pragma unroll
                 for (int c = 0; c < DH / 8; ++c) {
                     const gd_half8 vv = *reinterpret_cast<const gd_half8 *>(v + row + 8 * c);
@@ -181,26 +216,29 @@ gd_m3_sparse_attention_kernel(const gd_half *__restrict__ q, const gd_half *__re
         }
     }
     const float inv = l > 0.f ? 1.f / l : 0.f;
-    gd_half *o = out + (qg * p.hq + hq) * DH;
+    gd_half *o = out + (qg * p.hq + hq) * dh;
 #pragma unroll
-    for (int c = 0; c < DH; ++c) o[c] = (gd_half)(acc[c] * inv);
+    for (int c = 0; c < DH; ++c) {
+        if (c < dh) o[c] = (gd_half)(acc[c] * inv);
+    }
 }
 
-#define GD_M3_DISPATCH(DH_VALUE, STATEMENT)     \
-    switch (DH_VALUE) {                         \
-    case 4: { constexpr int DH = 4; STATEMENT; break; }   \
-    case 8: { constexpr int DH = 8; STATEMENT; break; }   \
-    case 16: { constexpr int DH = 16; STATEMENT; break; } \
-    case 32: { constexpr int DH = 32; STATEMENT; break; } \
-    case 64: { constexpr int DH = 64; STATEMENT; break; } \
-    default: return (int)hipErrorInvalidValue;  \
+#define GD_M3_DISPATCH(PARAMS, STATEMENT)                                      \
+    if ((PARAMS)->dh == 0u || (PARAMS)->dh > GD_M3_MAX_DH) return (int)hipErrorInvalidValue; \
+    switch ((PARAMS)->unaligned != 0u ? 0u : (PARAMS)->dh) {                                                      \
+    case 4: { constexpr int DH = 4; constexpr bool ANY = false; STATEMENT; break; }   \
+    case 8: { constexpr int DH = 8; constexpr bool ANY = false; STATEMENT; break; }   \
+    case 16: { constexpr int DH = 16; constexpr bool ANY = false; STATEMENT; break; } \
+    case 32: { constexpr int DH = 32; constexpr bool ANY = false; STATEMENT; break; } \
+    case 64: { constexpr int DH = 64; constexpr bool ANY = false; STATEMENT; break; } \
+    default: { constexpr int DH = GD_M3_MAX_DH; constexpr bool ANY = true; STATEMENT; break; } \
     }
 
 extern "C" int gd_hip_launch_m3_index_topk(hipStream_t stream, const void *q, const void *k, const int32_t *cu,
                                            int32_t *topk, const gd_m3_params *p)
 {
     const dim3 grid((p->max_seqlen + GD_M3_PICK_ROWS - 1u) / GD_M3_PICK_ROWS, p->hkv, p->batch);
-    GD_M3_DISPATCH(p->dh, (gd_m3_index_topk_kernel<DH><<<grid, GD_M3_PICK_ROWS, 0, stream>>>(
+    GD_M3_DISPATCH(p, (gd_m3_index_topk_kernel<DH, ANY><<<grid, GD_M3_PICK_ROWS, 0, stream>>>(
                               (const gd_half *)q, (const gd_half *)k, cu, topk, *p)));
     return (int)hipGetLastError();
 }
@@ -210,7 +248,7 @@ extern "C" int gd_hip_launch_m3_sparse_attention(hipStream_t stream, const void 
                                                  const gd_m3_params *p)
 {
     const dim3 grid((p->max_seqlen + GD_M3_ATTN_ROWS - 1u) / GD_M3_ATTN_ROWS, p->hq, p->batch);
-    GD_M3_DISPATCH(p->dh, (gd_m3_sparse_attention_kernel<DH><<<grid, GD_M3_ATTN_ROWS, 0, stream>>>(
+    GD_M3_DISPATCH(p, (gd_m3_sparse_attention_kernel<DH, ANY><<<grid, GD_M3_ATTN_ROWS, 0, stream>>>(
                               (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, cu, topk, (gd_half *)out, *p)));
     return (int)hipGetLastError();
 }

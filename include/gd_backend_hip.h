@@ -302,8 +302,9 @@ gd_status gd_backend_kv_cache_append_packed(gd_backend *backend,
 
 /* MiniMax-M3 block-sparse attention over packed sequences, forward (reference src/core/backend.h:632-655; Metal
  * kernels metal_minimax_m3_index_topk.metal, metal_minimax_m3_sparse_attention.metal under src/ops).  All tensors
- * contiguous; q / k / v / out F16 [N, H, Dh] (Dh in {4, 8, 16, 32, 64}; other sizes up to 64, which the reference
- * accepts, are GD_ERR_UNSUPPORTED; Dh = 64 with a block size of 64 or 128 runs on the matrix cores), cu_seqlens
+ * contiguous; q / k / v / out F16 [N, H, Dh] (Dh <= 64 as in the reference, odd sizes included; Dh = 64 with a block
+ * size of 64 or 128 on 16-byte aligned views runs on the matrix cores, Dh in {4, 8, 16, 32, 64} on aligned views
+ * with vector loads, everything else half by half), cu_seqlens
  * I32 [B+1], topk_idx I32 [Hkv, N, topk]; block_size <= 128,
  * topk <= 16; rows at or beyond max_seqlen inside their sequence are not processed.
  *   index_topk        index_q and index_k have the same number of heads.  Row i of a sequence sees blocks

@@ -1220,6 +1220,36 @@ def test_minimax_m3_matches_oracle(backend, arena, oracle, gda, lens, H, Hkv, Dh
     _close(out.read(), oracle.minimax_m3_sparse_attention(q, k, v, cu, want_idx, block, scale))
 
 
+@pytest.mark.parametrize("Dh,shift", [(24, 0), (7, 0), (1, 0), (63, 0), (48, 0), (16, 3), (64, 1)])
+def test_minimax_m3_any_head_size_and_alignment(backend, arena, oracle, gda, Dh, shift):
+    """Head sizes without a kernel of their own (the reference takes every size up to 64) and views that start off
+    a 16-byte boundary take the half-by-half path; the padding it adds is exact zeros, so the bar is the same."""
+    lens, H, Hkv, block, topk = [37, 70], 4, 2, 8, 3
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    N = int(cu[-1])
+    q, v = oracle.normal_f16((N, H, Dh), 7300 + Dh), oracle.normal_f16((N, Hkv, Dh), 7400 + Dh)
+    k, iq = oracle.normal_f16((N, Hkv, Dh), 7500 + Dh), oracle.normal_f16((N, Hkv, Dh), 7600 + Dh)
+
+    def put(a):  # the view starts `shift` halfs into its allocation
+        if shift == 0:
+            return arena.from_numpy(a)
+        whole = arena.alloc((a.size + shift,), gda.F16)
+        whole.write(np.concatenate([np.zeros(shift, np.float16), a.ravel()]))
+        return gda.Tensor(whole.buffer, whole.offset + 2 * shift, a.shape, gda.F16)
+
+    tq, tk, tv, tiq = put(q), put(k), put(v), put(iq)
+    tcu = arena.from_numpy(cu)
+    idx = arena.alloc((Hkv, N, topk), gda.I32)
+    backend.minimax_m3_index_topk(tiq, tk, tcu, idx, block, 1, 1)
+    want_idx = oracle.minimax_m3_index_topk(iq, k, cu, block, topk, 1, 1)
+    _assert_same_blocks(oracle, idx.read(), want_idx, iq, k, cu, block, 1, 1, "picker")
+    idx.write(want_idx)
+    out = put(np.full((N, H, Dh), 7.0, np.float16))
+    scale = float(1.0 / np.sqrt(Dh))
+    backend.minimax_m3_sparse_attention(tq, tk, tv, tcu, idx, out, block, scale)
+    _close(out.read(), oracle.minimax_m3_sparse_attention(q, k, v, cu, want_idx, block, scale))
+
+
 @pytest.mark.parametrize("lens,H,Hkv,block,topk,init,local", [
     ([300, 17, 129, 1, 640], 4, 4, 128, 4, 1, 1),
     ([1500], 4, 2, 64, 16, 1, 2),
@@ -1293,9 +1323,9 @@ def test_minimax_m3_rejects_bad_arguments(backend, arena, gda):
         with pytest.raises(gda.GdError) as err:
             backend.minimax_m3_index_topk(a["q"], a["k"], a["cu"], a["idx"], a["block"])
         assert err.value.status == gda.INVALID_ARGUMENT, bad
-    with pytest.raises(gda.GdError) as err:
-        backend.minimax_m3_index_topk(arena.alloc((N, H, 24), gda.F16), arena.alloc((N, H, 24), gda.F16), cu, idx, 8)
-    assert err.value.status == gda.UNSUPPORTED
+    with pytest.raises(gda.GdError) as err:  # the reference's limit on the head size
+        backend.minimax_m3_index_topk(arena.alloc((N, H, 65), gda.F16), arena.alloc((N, H, 65), gda.F16), cu, idx, 8)
+    assert err.value.status == gda.INVALID_ARGUMENT
     out = arena.alloc((N, H, Dh), gda.F16)
     with pytest.raises(gda.GdError) as err:
         backend.minimax_m3_sparse_attention(q, k, arena.alloc((N, H, 8), gda.F16), cu, idx, out, 8, 0.25)
