@@ -80,7 +80,7 @@ gd_m3_index_topk_kernel(const gd_half *__restrict__ q, const gd_half *__restrict
     const int q0 = blockIdx.x * GD_M3_PICK_ROWS;
     if (q0 >= T) return;
     const int i = q0 + tid;
-    const bool active = i < T;
+    const bool active = i < T && i < (int)p.max_seqlen; /* rows at or beyond max_seqlen are not processed */
     const int block = (int)p.block;
     const int valid = active ? (i + block) / block : 0;
     const int last_row = min(q0 + GD_M3_PICK_ROWS - 1, T - 1);
@@ -172,7 +172,7 @@ gd_m3_sparse_attention_kernel(const gd_half *__restrict__ q, const gd_half *__re
     const int hq = blockIdx.y, b = blockIdx.z;
     const int start = cu[b], T = cu[b + 1] - start;
     const int i = blockIdx.x * GD_M3_ATTN_ROWS + threadIdx.x;
-    if (i >= T) return;
+    if (i >= T || i >= (int)p.max_seqlen) return; /* rows at or beyond max_seqlen are not processed */
     const int hkv = hq / (int)(p.hq / p.hkv);
     const size_t qg = (size_t)(start + i);
     const int dh = ANY ? (int)p.dh : DH; /* halfs per row in global memory */

@@ -1298,6 +1298,31 @@ def test_minimax_m3_matrix_core_kernels(backend, arena, oracle, gda, lens, H, Hk
     _assert_same_blocks(oracle, idx2.read(), want_idx, kq, k, cu, block, init, local, "per-row picker")
 
 
+@pytest.mark.parametrize("Dh,block", [(64, 64), (32, 16)])
+def test_minimax_m3_max_seqlen_cuts_rows_exactly(backend, arena, oracle, gda, Dh, block):
+    """Rows at or beyond max_seqlen inside their sequence keep what the outputs held; the rows in front of it are
+    what they are without the limit (matrix-core and per-row kernels, a limit inside a row tile)."""
+    lens, H, Hkv, topk, limit = [300, 90, 200], 4, 2, 4, 150
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    N = int(cu[-1])
+    q, iq, k, v = (oracle.normal_f16((N, h, Dh), s) for h, s in ((H, 7700), (Hkv, 7701), (Hkv, 7702), (Hkv, 7703)))
+    tq, tiq, tk, tv, tcu = (arena.from_numpy(a) for a in (q, iq, k, v, cu))
+    inside = np.concatenate([np.arange(n) < limit for n in lens])
+    full_idx = arena.alloc((Hkv, N, topk), gda.I32)
+    backend.minimax_m3_index_topk(tiq, tk, tcu, full_idx, block, 1, 1)
+    idx = arena.from_numpy(np.full((Hkv, N, topk), -7, np.int32))
+    backend.minimax_m3_index_topk(tiq, tk, tcu, idx, block, 1, 1, max_seqlen=limit)
+    got, want = idx.read(), full_idx.read()
+    assert np.array_equal(got[:, inside], want[:, inside]) and (got[:, ~inside] == -7).all()
+    scale = float(1.0 / np.sqrt(Dh))
+    full_out = arena.alloc((N, H, Dh), gda.F16)
+    backend.minimax_m3_sparse_attention(tq, tk, tv, tcu, full_idx, full_out, block, scale)
+    out = arena.from_numpy(np.full((N, H, Dh), 7.0, np.float16))
+    backend.minimax_m3_sparse_attention(tq, tk, tv, tcu, full_idx, out, block, scale, max_seqlen=limit)
+    got, want = out.read(), full_out.read()
+    assert np.array_equal(got[inside], want[inside]) and (got[~inside] == 7.0).all()
+
+
 def test_minimax_m3_all_blocks_is_dense_causal_attention(backend, arena, oracle, gda):
     lens = [100, 33]
     cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
