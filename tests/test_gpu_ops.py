@@ -1298,6 +1298,29 @@ def test_minimax_m3_matrix_core_kernels(backend, arena, oracle, gda, lens, H, Hk
     _assert_same_blocks(oracle, idx2.read(), want_idx, kq, k, cu, block, init, local, "per-row picker")
 
 
+def test_minimax_m3_full_size_prefill(backend, arena, oracle, gda):
+    """The reference's M3 settings (head size 64, blocks of 128, 3 picked, first and last block always) at two full
+    4096-token sequences: every list and every output row against the oracle; and rows whose whole context fits
+    the picked blocks (the first 3 x 128) equal dense causal attention."""
+    lens, H, Hkv, Dh, block, topk = [4096, 4096], 4, 2, 64, 128, 3
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    N = int(cu[-1])
+    q, iq, k, v = (oracle.normal_f16((N, h, Dh), s) for h, s in ((H, 7800), (Hkv, 7801), (Hkv, 7802), (Hkv, 7803)))
+    tq, tiq, tk, tv, tcu = (arena.from_numpy(a) for a in (q, iq, k, v, cu))
+    idx = arena.alloc((Hkv, N, topk), gda.I32)
+    backend.minimax_m3_index_topk(tiq, tk, tcu, idx, block, 1, 1, max_seqlen=4096)
+    want_idx = oracle.minimax_m3_index_topk(iq, k, cu, block, topk, 1, 1)
+    _assert_same_blocks(oracle, idx.read(), want_idx, iq, k, cu, block, 1, 1, "full-size picker")
+    idx.write(want_idx)
+    out = arena.alloc((N, H, Dh), gda.F16)
+    backend.minimax_m3_sparse_attention(tq, tk, tv, tcu, idx, out, block, 0.125, max_seqlen=4096)
+    got = out.read()
+    _close(got, oracle.minimax_m3_sparse_attention(q, k, v, cu, want_idx, block, 0.125))
+    head = slice(4096, 4096 + topk * block)  # second sequence, rows that see at most 3 blocks
+    dense = oracle.sdpa_varlen(q[head], k[head], v[head], np.array([0, topk * block], np.int32), 0.125)
+    _close(got[head], dense)
+
+
 @pytest.mark.parametrize("Dh,block", [(64, 64), (32, 16)])
 def test_minimax_m3_max_seqlen_cuts_rows_exactly(backend, arena, oracle, gda, Dh, block):
     """Rows at or beyond max_seqlen inside their sequence keep what the outputs held; the rows in front of it are
