@@ -32,9 +32,10 @@ def test_f16_to_f32_all_bit_patterns(oracle):
 
 def test_f32_to_f16_matches_ieee_rne(oracle):
     rng = np.random.default_rng(7)
+    exact_halves = np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32)
     x = np.concatenate([
-        rng.standard_normal(200000).astype(np.float32) * 10.0 ** rng.integers(-9, 6, 200000),
-        np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32),  # exact halves
+        (rng.standard_normal(200000) * 10.0 ** rng.integers(-9, 6, 200000)).astype(np.float32),
+        exact_halves,
         np.array([0.0, -0.0, 65504.0, 65519.99, 65520.0, 1e9, -1e9, np.inf, -np.inf,
                   2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0000001, 2.0 ** -14, 5.9604645e-08],
                  np.float32),
