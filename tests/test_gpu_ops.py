@@ -1143,7 +1143,9 @@ def test_sample_advance_on_the_reference_samplers_golden_cases(backend, arena, o
         work = t["work"].read()[:B * V].reshape(B, V)
         want = z[f"{c}_logits_after"]
         same = (work == want) | (np.isnan(work) & np.isnan(want))
-        assert np.all(same | (np.abs(work - want) <= 2e-6 * np.abs(want))), c
+        with np.errstate(invalid="ignore"):  # inf - inf on entries `same` already covers
+            close = np.abs(work - want) <= 2e-6 * np.abs(want)
+        assert np.all(same | close), c
         assert np.array_equal(t["hist_len"].read(), hist_len + 1)
 
 
