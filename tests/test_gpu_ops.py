@@ -703,9 +703,9 @@ def test_fused_linear_rms_prologue_and_residual(backend, arena, oracle, M, K, N)
     _close(y.read(), want)
     backend.fused_linear(tx, tw, tb, tr, None, y, True, 2, 0)
     want = oracle.add(res, oracle.linear_nt(x, w, bias))
-    _close(y.read(), want)
+    _close(y.read(), want, through=res)  # the sum may cancel: one rounding step is the residual's size
     backend.fused_linear(tx, tw, None, tr, tn, y, True, 0, 2, 1e-5)
-    _close(y.read(), oracle.add(res, oracle.linear_nt(oracle.rms_norm(x, nw, 1e-5), w)))
+    _close(y.read(), oracle.add(res, oracle.linear_nt(oracle.rms_norm(x, nw, 1e-5), w)), through=res)
 
 
 @pytest.mark.parametrize("M,K,N,nk", [(64, 1536, 512, True), (64, 1536, 512, False), (16, 352, 2048, True), (3, 24, 33, False)])
