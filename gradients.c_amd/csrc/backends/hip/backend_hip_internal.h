@@ -38,6 +38,7 @@ struct gd_backend {
     int m3_simple;        /* 1: MiniMax-M3 operators always take the per-row kernels (tests compare the two paths) */
     int linear_tiles;    /* few-row projections: 16-column tiles per workgroup, 1 / 2 / 4 (0 = automatic) */
     int linear_waves;    /* few-row projections: wavefronts per workgroup = K split, 4 / 8 (0 = automatic) */
+    int linear_no_lds_stream; /* few-row projections: 1 = never stage the weight stream through LDS (tests compare the two paths) */
 };
 
 struct gd_backend_buffer {

@@ -65,6 +65,7 @@ static gd_status project_full(gd_backend *backend, const gd_backend_matrix_view 
     p.rope_freq_scale = 0.0f;
     p.force_tiles = (uint32_t)backend->linear_tiles;
     p.force_waves = (uint32_t)backend->linear_waves;
+    p.no_lds_stream = (uint32_t)backend->linear_no_lds_stream;
     /* 16-byte fragment loads: x rows always, w rows when K-contiguous, the norm weight */
     vec = (K % 8u) == 0u && ((x->offset | x->row_bytes) & 15u) == 0u &&
           (!w_is_nk || ((w->offset | w->row_bytes) & 15u) == 0u) && (norm_w == NULL || (norm_w->offset & 15u) == 0u);
@@ -199,6 +200,7 @@ gd_status gd_backend_fused_qkv_rope_append(gd_backend *backend, const gd_backend
     p.rope_freq_scale = -2.0f * log2f(rope_args->theta) / (float)head_dim;
     p.force_tiles = (uint32_t)backend->linear_tiles;
     p.force_waves = (uint32_t)backend->linear_waves;
+    p.no_lds_stream = (uint32_t)backend->linear_no_lds_stream;
     r.rope_pos = (const int32_t *)gd_hip_view_ptr(pos_ids);
     r.cache_pos = (const int32_t *)gd_hip_view_ptr(cache_pos);
     r.q = gd_hip_view_ptr(q);

@@ -28,6 +28,7 @@ typedef struct gd_hip_linear_params {
     uint32_t rope_heads, rope_head_dim, rope_tmax;
     float rope_freq_scale;
     uint32_t force_tiles, force_waves; /* tunables: 0 = automatic */
+    uint32_t no_lds_stream;            /* tunable: 1 = weights always go straight to registers */
 } gd_hip_linear_params;
 
 /* destinations of the rope + append epilogue: q [M,H,D]; caches [M,Tmax,H,D]; positions I32 [M] */

@@ -39,6 +39,17 @@ __device__ __forceinline__ float gd_lin_silu(float z)
     return z * (z >= 0.0f ? inv : e * inv);
 }
 
+/* 16 bytes per lane from global memory straight into LDS: lane l's data lands at lds_byte_address + 16*l.
+ * Assembly, because the kernel counts these loads itself (s_waitcnt vmcnt) instead of waiting for all of them. */
+__device__ __forceinline__ void gd_lin_load_lds16(const unsigned char *uniform_base, uint32_t lane_byte_offset,
+                                                  uint32_t lds_byte_address)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_byte_address), "v"(lane_byte_offset), "s"(uniform_base)
+                 : "memory");
+}
+
 template <int NT, int WAVES, bool W_NK, int PRO, bool RES>
 __global__ void __launch_bounds__(WAVES * 64)
 gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__ w,
@@ -55,6 +66,17 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
     __shared__ float s_part[WAVES][16];
     /* w stored [K,N]: a 32(k) x COLS(n) tile per wavefront, turned by the transposing LDS read */
     __shared__ __align__(16) gd_half s_tr[W_NK ? 1 : WAVES][W_NK ? 8 : 32 * COLS];
+    /* Weight stream through LDS (long-K [N,K] projections behind an rms_norm whose activation slice is resident:
+     * the qkv, up/gate and LM-head projections of the wide decoders).  A load that goes straight to registers must
+     * follow the MFMA operand layout, 4 lanes = 64 bytes per weight row and instruction, and such half-line requests
+     * stream about a fifth slower than whole lines.  Lane order in LDS is free, so here one instruction fetches
+     * 8 weight rows x 128 bytes (two K steps) into a wavefront-private ring and the fragments are read from there
+     * (16-byte chunks XOR-swizzled by the row so that the reads spread over the banks).  A group = the 16 rows of
+     * one column tile x 128 bytes = two instructions; RING groups are in flight per wavefront.  The MFMAs run in
+     * the order of the register path, so the sums are the same to the bit. */
+    constexpr bool LDSW = W_NK && RES && WAVES == 8 && NT >= 4 && PRO == GD_HIP_PRO_RMS_NORM;
+    constexpr int RING = 6;
+    __shared__ __align__(16) unsigned char s_ring[LDSW ? WAVES * RING * 2048 : 16];
     /* every kernel argument the kernel reads, requested in one batch with one wait (left alone, the compiler puts
      * each load in front of its first use, one dependent round trip after the other) */
     asm volatile("" ::"s"(x), "s"(w), "s"(bias), "s"(residual), "s"(norm_w), "s"(y), "s"(p.M), "s"(p.N), "s"(p.K),
@@ -215,8 +237,35 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
     using gd_s0 = std::integral_constant<int, 0>;
     using gd_s1 = std::integral_constant<int, 1>;
 
-    /* the first weights are requested before anything else so that the row norms below overlap their flight */
-    load_set(gd_s0{}, s_begin);
+    /* LDS path: every step of the wavefront exists (8 steps = 4 line pairs per column tile) */
+    const bool ldsw = LDSW && fast && p.no_lds_stream == 0u && s_begin + (uint32_t)RES_STEPS <= s_end;
+    uint32_t goff[NT][2]; /* bytes from the group's base to the lane's 16 bytes: row 8*half + lane/8, swizzled chunk */
+    const uint32_t ring_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)s_ring + (uint32_t)wave * (RING * 2048u);
+    auto issue_group = [&](uint32_t g) __attribute__((always_inline)) {
+        /* g = pair * NT + j: K steps 2*pair, 2*pair+1 of column tile j */
+        const uint32_t pair = g / NT, j = g % NT, slot = ring_base + (g % RING) * 2048u;
+        const unsigned char *src = wb + (size_t)(s_begin + 2u * pair) * 64u;
+        gd_lin_load_lds16(src, goff[j][0], slot);
+        gd_lin_load_lds16(src, goff[j][1], slot + 1024u);
+    };
+    if (LDSW && ldsw) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint32_t rowi = 8u * h + (uint32_t)lane / 8u;
+                const uint32_t n = (gated && j >= NT / 2)
+                                       ? pair_offset + min(n0 + 16u * (uint32_t)(j - NT / 2) + rowi, p.N - 1u)
+                                       : min(n0 + 16u * (uint32_t)j + rowi, p.N - 1u);
+                goff[j][h] = (n * p.ldw + ((((uint32_t)lane % 8u) ^ ((uint32_t)lane / 8u)) * 8u)) * 2u;
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < RING; ++g) issue_group((uint32_t)g);
+    } else {
+        /* the first weights are requested before anything else so that the row norms below overlap their flight */
+        load_set(gd_s0{}, s_begin);
+    }
 
     if (RES) {
         /* the wavefront's whole activation slice (at most RES_STEPS steps): one batch of loads, and the row's sum of
@@ -240,7 +289,7 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
         }
         /* the second register set is requested here too: behind the barrier of the row norms its round trip would
          * start only when the first one has ended */
-        load_set(gd_s1{}, s_begin + U);
+        if (!(LDSW && ldsw)) load_set(gd_s1{}, s_begin + U);
         if (PRO == GD_HIP_PRO_RMS_NORM) {
 #pragma unroll
             for (int r = 0; r < RES_STEPS; ++r)
@@ -274,7 +323,50 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
     }
 
     /* two register sets alternate: the next U steps are in flight while the current ones are multiplied */
-    if (RES) {
+    if (LDSW && ldsw) {
+        const uint32_t li8 = (uint32_t)li % 8u, half_rows = ((uint32_t)li / 8u) * 1024u;
+        const uint32_t rd0 = half_rows + (li8 * 8u + ((uint32_t)lg ^ li8)) * 16u;
+        const uint32_t rd1 = half_rows + (li8 * 8u + ((4u + (uint32_t)lg) ^ li8)) * 16u;
+        const unsigned char *ring = &s_ring[0] + (size_t)wave * (RING * 2048);
+        constexpr int NG = (RES_STEPS / 2) * NT;
+        /* the normalised activation fragments, rounded to F16 like the separate rms_norm */
+#pragma unroll
+        for (int r = 0; r < RES_STEPS; ++r) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ar[r][e] = (gd_half)((float)ar[r][e] * (float)nr[r][e] * minv);
+        }
+        /* group g is read from its slot while the MFMAs of group g-1 run; the slot of g-1 is refilled only behind
+         * those MFMAs, which could not issue before its reads had returned */
+        gd_half8 f0, f1, pf0 = zero8, pf1 = zero8;
+#pragma unroll
+        for (int g = 0; g <= NG; ++g) {
+            if (g < NG) {
+                /* loads return in order: group g has landed once only the groups requested after it are outstanding */
+                const int issued = g < 2 ? RING - 1 : (g - 2 + RING < NG - 1 ? g - 2 + RING : NG - 1);
+                const int later = issued - g;
+                if (later >= 7) asm volatile("s_waitcnt vmcnt(14)" ::: "memory");
+                else if (later == 6) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+                else if (later == 5) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+                else if (later == 4) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+                else if (later == 3) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+                else if (later == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+                else if (later == 1) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                const unsigned char *slot = ring + (g % RING) * 2048;
+                f0 = *reinterpret_cast<const gd_half8 *>(slot + rd0);
+                f1 = *reinterpret_cast<const gd_half8 *>(slot + rd1);
+            }
+            if (g >= 1) {
+                const int q = g - 1, pair = q / NT, j = q % NT;
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ar[2 * pair], pf0, acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ar[2 * pair + 1], pf1, acc[j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (q + RING < NG) issue_group((uint32_t)(q + RING));
+            }
+            pf0 = f0;
+            pf1 = f1;
+        }
+    } else if (RES) {
         /* at most RES_STEPS steps: fully unrolled so that the resident fragments are indexed statically */
         compute_set(gd_s0{}, std::integral_constant<int, 0>{});
         if (2 * U < RES_STEPS) {

@@ -875,6 +875,39 @@ def test_fused_linear_swiglu_epilogue(backend, arena, oracle, gda, M, K, H):
     assert backend.call("gd_backend_fused_linear", tx.matrix(), wk.matrix(), None, None, None, y.matrix(), C.byref(a)) == gda.UNSUPPORTED
 
 
+@pytest.mark.parametrize("M,N,gated", [(16, 5632, True), (33, 8200, False), (64, 4096, True), (5, 32768, False)])
+def test_few_row_projection_weight_stream_through_lds(backend, arena, oracle, gda, M, N, gated):
+    """rms_norm + projection with K = 2048 and 64 columns per workgroup stages its weight stream through LDS (whole
+    128-byte lines per weight row and load) instead of loading MFMA fragments straight into registers.  Both paths
+    multiply in the same order: the same bits, and both within the bar of the oracle (also where the last workgroup's
+    columns run past N)."""
+    K = 2048
+    x = oracle.normal_f16((M, K), 3000 + M, 1.3)
+    nw = (1.0 + 0.1 * oracle.normal_f16((K,), 3001).astype(np.float32)).astype(np.float16)
+    rows = 2 * N if gated else N
+    w = oracle.normal_f16((rows, K), 3002 + N, 0.05)
+    bias = oracle.normal_f16((rows,), 3003, 0.5)
+    y = arena.alloc((M, N), gda.F16)
+    tx, tw, tb, tn = (arena.from_numpy(a) for a in (x, w, bias, nw))
+    got = {}
+    try:
+        for off in (0, 1):
+            backend.set_tunable("linear_no_lds_stream", off)
+            backend.fill(y, 0x7e00)
+            backend.fused_linear(tx, tw, tb, None, tn, y, True, 2, 2, 1e-5, epilogue=1 if gated else 0)
+            got[off] = y.read()
+    finally:
+        backend.set_tunable("linear_no_lds_stream", 0)
+    assert np.array_equal(got[0].view(np.uint16), got[1].view(np.uint16))
+    u = oracle.linear_nt(oracle.rms_norm(x, nw, 1e-5), w, bias)
+    if gated:
+        through = (np.abs(u[:, :N].astype(np.float64)) + np.abs(bias[:N].astype(np.float64))) * \
+                  (1.0 + np.abs(u[:, N:].astype(np.float64)) + np.abs(bias[N:].astype(np.float64)))
+        _close(got[0], oracle.swiglu_split(u), through=through)
+    else:
+        _close(got[0], u)
+
+
 @pytest.mark.parametrize("B,H,D,K", [(64, 8, 64, 512), (16, 16, 128, 2048), (5, 3, 32, 72), (33, 2, 96, 64)])
 def test_fused_qkv_rope_append_equals_separate_ops(backend, arena, oracle, gda, B, H, D, K):
     """rms_norm -> qkv projection (+F16 bias) -> rope -> cache append in one launch against the fused projection
