@@ -63,8 +63,8 @@ static gd_status project_full(gd_backend *backend, const gd_backend_matrix_view 
     p.swiglu_cols = gated ? y->cols : 0u;
     p.rope_heads = p.rope_head_dim = p.rope_tmax = 0u;
     p.rope_freq_scale = 0.0f;
-    p.force_tiles = (uint32_t)backend->linear_tiles;
-    p.force_waves = (uint32_t)backend->linear_waves;
+    p.force_tiles = (uint16_t)backend->linear_tiles;
+    p.force_waves = (uint16_t)backend->linear_waves;
     p.no_lds_stream = (uint32_t)backend->linear_no_lds_stream;
     /* 16-byte fragment loads: x rows always, w rows when K-contiguous, the norm weight */
     vec = (K % 8u) == 0u && ((x->offset | x->row_bytes) & 15u) == 0u &&
@@ -198,8 +198,8 @@ gd_status gd_backend_fused_qkv_rope_append(gd_backend *backend, const gd_backend
     p.rope_head_dim = head_dim;
     p.rope_tmax = (uint32_t)k_cache->shape[1];
     p.rope_freq_scale = -2.0f * log2f(rope_args->theta) / (float)head_dim;
-    p.force_tiles = (uint32_t)backend->linear_tiles;
-    p.force_waves = (uint32_t)backend->linear_waves;
+    p.force_tiles = (uint16_t)backend->linear_tiles;
+    p.force_waves = (uint16_t)backend->linear_waves;
     p.no_lds_stream = (uint32_t)backend->linear_no_lds_stream;
     r.rope_pos = (const int32_t *)gd_hip_view_ptr(pos_ids);
     r.cache_pos = (const int32_t *)gd_hip_view_ptr(cache_pos);
