@@ -18,6 +18,10 @@
 extern "C" {
 #endif
 
+#define GD_HIP_MAX_RETIRED_WS 16
+#define GD_HIP_GRAPH_STRIDE 8u
+#define GD_HIP_GRAPH_RING 4u
+
 struct gd_backend {
     int device;
     hipStream_t stream;
@@ -30,6 +34,15 @@ struct gd_backend {
     /* scratch for split-KV attention partials, grown on demand outside capture */
     void *attn_ws;
     size_t attn_ws_bytes;
+    /* instantiated graphs hold the workspace address of their capture: blocks replaced while any graph is alive
+     * are kept here and freed when the last graph is destroyed (or with the backend) */
+    int live_graphs;
+    void *retired_ws[GD_HIP_MAX_RETIRED_WS];
+    int retired_ws_count;
+    /* graph launches in flight are bounded: an event after every GD_HIP_GRAPH_STRIDE launches, the host waits
+     * for the one GD_HIP_GRAPH_RING events back */
+    hipEvent_t graph_events[GD_HIP_GRAPH_RING];
+    unsigned graph_launches;
     /* tunables read from the environment once at creation */
     int sdpa_chunk;      /* keys per workgroup in the split-KV decode kernel (0 = automatic) */
     int sdpa_waves;      /* 4 or 8 wavefronts per workgroup (0 = default 8) */
