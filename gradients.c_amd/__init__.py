@@ -142,6 +142,7 @@ _SIGNATURES = {
     "gd_backend_sdpa_decode": [_vp, _TV, _TV, _TV, _TV, _TV, C.POINTER(SdpaDecodeArgs)],
     "gd_backend_sdpa_decode_at": [_vp, _TV, _TV, _TV, _TV, C.POINTER(SdpaDecodeArgs)],
     "gd_backend_sdpa_decode_positions": [_vp, _TV, _TV, _TV, _TV, _TV, C.POINTER(SdpaDecodeArgs)],
+    "gd_backend_sdpa_decode_positions_noalloc": [_vp, _TV, _TV, _TV, _TV, _TV, C.POINTER(SdpaDecodeArgs)],
     "gd_backend_kv_cache_append_at": [_vp, _TV, _TV, _TV, _TV, C.POINTER(KvAppendArgs)],
     "gd_backend_kv_cache_append_positions": [_vp, _TV, _TV, _TV, _TV, _TV, C.POINTER(KvAppendArgs)],
     "gd_backend_kv_cache_append_packed": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, C.POINTER(KvAppendArgs)],
@@ -484,6 +485,11 @@ class Backend:
         a = SdpaDecodeArgs(scale, window, prefix, 0)
         _check(self.call("gd_backend_sdpa_decode_positions", q.view(), k.view(), v.view(), pos.view(), out.view(),
                          C.byref(a)), "gd_backend_sdpa_decode_positions")
+
+    def sdpa_decode_positions_noalloc(self, q, k, v, pos, out, scale, window=0, prefix=0):
+        a = SdpaDecodeArgs(scale, window, prefix, 0)
+        _check(self.call("gd_backend_sdpa_decode_positions_noalloc", q.view(), k.view(), v.view(), pos.view(),
+                         out.view(), C.byref(a)), "gd_backend_sdpa_decode_positions_noalloc")
 
     def kv_cache_append_at(self, k_cache, v_cache, cache_pos, k_new, v_new):
         a = KvAppendArgs(cache_pos)

@@ -18,6 +18,8 @@ int gd_hip_launch_fill(hipStream_t stream, void *dst, size_t count, size_t elem_
 int gd_hip_launch_rand_uniform(hipStream_t stream, void *dst, uint64_t count, uint32_t dtype, uint64_t seed,
                                float low, float high);
 
+int gd_hip_sdpa_decode_scratch_init(int device);
+
 static gd_status status_of(hipError_t e)
 {
     if (e == hipSuccess) return GD_OK;
@@ -46,14 +48,27 @@ gd_status gd_hip_reserve_attn_ws(gd_backend *backend, size_t nbytes)
     /* work already enqueued may still read the old block */
     if (hipStreamSynchronize(backend->stream) != hipSuccess) return GD_ERR_INTERNAL;
     nbytes = (nbytes + ((size_t)1 << 20) - 1u) & ~(((size_t)1 << 20) - 1u);
+    /* a live graph replays kernels that write their partial results into the block it was captured with */
+    if (backend->attn_ws != NULL && backend->live_graphs > 0 && backend->retired_ws_count == GD_HIP_MAX_RETIRED_WS)
+        return GD_ERR_BUSY;
     if (hipMalloc(&p, nbytes) != hipSuccess) {
         (void)hipGetLastError();
         return GD_ERR_OUT_OF_MEMORY;
     }
-    if (backend->attn_ws != NULL) (void)hipFree(backend->attn_ws);
+    if (backend->attn_ws != NULL) {
+        if (backend->live_graphs > 0) backend->retired_ws[backend->retired_ws_count++] = backend->attn_ws;
+        else (void)hipFree(backend->attn_ws);
+    }
     backend->attn_ws = p;
     backend->attn_ws_bytes = nbytes;
     return GD_OK;
+}
+
+static void free_retired_ws(gd_backend *backend)
+{
+    int i;
+    for (i = 0; i < backend->retired_ws_count; ++i) (void)hipFree(backend->retired_ws[i]);
+    backend->retired_ws_count = 0;
 }
 
 static int env_int(const char *name, int fallback, int lo, int hi)
@@ -82,6 +97,9 @@ gd_status gd_backend_create_default(gd_backend **out_backend)
     if (b == NULL) return GD_ERR_OUT_OF_MEMORY;
     b->device = 0;
     if (hipSetDevice(b->device) != hipSuccess || hipGetDeviceProperties(&prop, b->device) != hipSuccess ||
+        /* address of the fixed scratch array of the entry point that allocates nothing: looked up once per
+         * device, with this device current */
+        gd_hip_sdpa_decode_scratch_init(b->device) != (int)hipSuccess ||
         hipStreamCreateWithFlags(&b->stream, hipStreamNonBlocking) != hipSuccess) {
         (void)hipGetLastError();
         free(b);
@@ -107,6 +125,13 @@ void gd_backend_destroy(gd_backend *backend)
     if (backend == NULL) return;
     (void)hipStreamSynchronize(backend->stream);
     if (backend->attn_ws != NULL) (void)hipFree(backend->attn_ws);
+    free_retired_ws(backend);
+    {
+        unsigned i;
+        for (i = 0u; i < GD_HIP_GRAPH_RING; ++i) {
+            if (backend->graph_events[i] != NULL) (void)hipEventDestroy(backend->graph_events[i]);
+        }
+    }
     (void)hipStreamDestroy(backend->stream);
     free(backend);
 }
@@ -424,6 +449,7 @@ gd_status gd_backend_graph_end_capture(gd_backend *backend, gd_backend_graph **o
         free(g);
         return GD_ERR_INTERNAL;
     }
+    backend->live_graphs += 1;
     *out_graph = g;
     return GD_OK;
 }
@@ -432,7 +458,29 @@ gd_status gd_backend_graph_launch(gd_backend *backend, gd_backend_graph *graph)
 {
     if (backend == NULL || graph == NULL || graph->backend != backend) return GD_ERR_INVALID_ARGUMENT;
     if (backend->capturing) return GD_ERR_BAD_STATE;
-    return gd_hip_finish_op(backend, (int)hipGraphLaunch(graph->exec, backend->stream));
+    {
+        /* Keep the launches queued on the stream bounded (GD_HIP_GRAPH_RING * GD_HIP_GRAPH_STRIDE): each one holds
+         * kernel-argument memory and queue packets of every node until it has run, and a caller may enqueue
+         * thousands without a wait in between.  One event per GD_HIP_GRAPH_STRIDE launches keeps the cost of the
+         * bound off the single step. */
+        const unsigned n = backend->graph_launches;
+        hipEvent_t *slot = &backend->graph_events[(n / GD_HIP_GRAPH_STRIDE) % GD_HIP_GRAPH_RING];
+        hipError_t e;
+        if ((n % GD_HIP_GRAPH_STRIDE) == 0u && n / GD_HIP_GRAPH_STRIDE >= GD_HIP_GRAPH_RING && *slot != NULL) {
+            if (hipEventSynchronize(*slot) != hipSuccess) return GD_ERR_INTERNAL;
+        }
+        e = hipGraphLaunch(graph->exec, backend->stream);
+        if (e == hipSuccess && (n % GD_HIP_GRAPH_STRIDE) == GD_HIP_GRAPH_STRIDE - 1u) {
+            if (*slot == NULL && hipEventCreateWithFlags(slot, hipEventDisableTiming) != hipSuccess) {
+                (void)hipGetLastError();
+                *slot = NULL;
+                return GD_ERR_INTERNAL;
+            }
+            e = hipEventRecord(*slot, backend->stream);
+        }
+        backend->graph_launches = n + 1u;
+        return gd_hip_finish_op(backend, (int)e);
+    }
 }
 
 void gd_backend_graph_destroy(gd_backend_graph *graph)
@@ -441,5 +489,7 @@ void gd_backend_graph_destroy(gd_backend_graph *graph)
     (void)hipStreamSynchronize(graph->backend->stream);
     (void)hipGraphExecDestroy(graph->exec);
     (void)hipGraphDestroy(graph->graph);
+    graph->backend->live_graphs -= 1;
+    if (graph->backend->live_graphs == 0) free_retired_ws(graph->backend);
     free(graph);
 }

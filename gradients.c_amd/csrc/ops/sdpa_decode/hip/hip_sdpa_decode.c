@@ -4,6 +4,7 @@
  * limit raised from 64 to 128 for the split-KV kernel (256 for the generic one).
  */
 #include <math.h>
+#include <stdio.h>
 
 #include "../../../backends/hip/backend_hip_internal.h"
 #include "hip_sdpa_decode_types.h"
@@ -14,7 +15,11 @@ int gd_hip_launch_sdpa_decode_split(hipStream_t stream, const void *q, const voi
 int gd_hip_launch_sdpa_decode_generic(hipStream_t stream, const void *q, const void *k, const void *v,
                                       const int32_t *pos, void *out, const gd_hip_sdpa_decode_params *params);
 
+float *gd_hip_sdpa_decode_scratch(int device);
+
 #define GD_HIP_SDPA_MAX_DH 256
+_Static_assert(GD_HIP_SDPA_NOALLOC_SCRATCH_BYTES == GD_BACKEND_SDPA_DECODE_NOALLOC_SCRATCH_BYTES,
+               "public constant and device array differ");
 
 static bool common_ok(const gd_backend_tensor_view *q, const gd_backend_tensor_view *k,
                       const gd_backend_tensor_view *v, const gd_backend_tensor_view *out)
@@ -43,7 +48,7 @@ static bool args_ok(const gd_backend_sdpa_decode_args *a, const gd_backend_tenso
 static gd_status dispatch(gd_backend *backend, const gd_backend_tensor_view *q, const gd_backend_tensor_view *k,
                           const gd_backend_tensor_view *v, const gd_backend_tensor_view *pos,
                           const gd_backend_tensor_view *out, const gd_backend_sdpa_decode_args *args,
-                          uint32_t pos_mode)
+                          uint32_t pos_mode, bool noalloc)
 {
     gd_hip_sdpa_decode_params p;
     const int32_t *pos_ptr = pos != NULL ? (const int32_t *)gd_hip_view_ptr(pos) : NULL;
@@ -95,13 +100,28 @@ static gd_status dispatch(gd_backend *backend, const gd_backend_tensor_view *q, 
         /* about 8 wavefronts per compute unit stream best: 4 per workgroup once there are two workgroups per unit */
         if (backend->sdpa_waves == 0)
             p.waves = (uint64_t)p.batch * p.hkv * p.nsplit >= 2u * (uint64_t)backend->compute_units ? 4u : 8u;
+        float *ws = NULL;
         if (p.nsplit > 1u) {
-            st = gd_hip_reserve_attn_ws(backend, (size_t)p.batch * p.hq * p.nsplit * (p.dh + 2u) * sizeof(float));
-            if (st != GD_OK) return st;
+            const size_t need = (size_t)p.batch * p.hq * p.nsplit * (p.dh + 2u) * sizeof(float);
+            if (noalloc) {
+                /* partial results go to the fixed device array of this library; nothing is allocated */
+                ws = gd_hip_sdpa_decode_scratch(backend->device);
+                if (ws == NULL) return GD_ERR_BAD_STATE;
+                if (need > GD_HIP_SDPA_NOALLOC_SCRATCH_BYTES) {
+                    fprintf(stderr, "gd_backend_sdpa_decode_positions_noalloc: the split-KV partial results of this "
+                                    "call need %zu bytes, the fixed scratch holds %u\n",
+                            need, (unsigned)GD_HIP_SDPA_NOALLOC_SCRATCH_BYTES);
+                    return GD_ERR_OUT_OF_MEMORY;
+                }
+            } else {
+                st = gd_hip_reserve_attn_ws(backend, need);
+                if (st != GD_OK) return st;
+                ws = (float *)backend->attn_ws;
+            }
         }
         return gd_hip_finish_op(backend, gd_hip_launch_sdpa_decode_split(
             backend->stream, gd_hip_view_ptr(q), gd_hip_view_ptr(k), gd_hip_view_ptr(v), pos_ptr,
-            gd_hip_view_ptr(out), (float *)backend->attn_ws, &p));
+            gd_hip_view_ptr(out), ws, &p));
     }
     if ((uint64_t)p.batch * p.hq * p.tq > 0x7fffffffu) return GD_ERR_UNSUPPORTED;
     return gd_hip_finish_op(backend, gd_hip_launch_sdpa_decode_generic(
@@ -118,7 +138,7 @@ gd_status gd_backend_sdpa_decode(gd_backend *backend, const gd_backend_tensor_vi
         cache_pos->dtype != GD_BACKEND_DTYPE_I32 || cache_pos->rank != 0u || cache_pos->count != 1u ||
         (cache_pos->offset & 3u) != 0u || !args_ok(args, k_cache))
         return GD_ERR_INVALID_ARGUMENT;
-    return dispatch(backend, q, k_cache, v_cache, cache_pos, out, args, GD_HIP_SDPA_POS_TENSOR0);
+    return dispatch(backend, q, k_cache, v_cache, cache_pos, out, args, GD_HIP_SDPA_POS_TENSOR0, false);
 }
 
 gd_status gd_backend_sdpa_decode_at(gd_backend *backend, const gd_backend_tensor_view *q,
@@ -129,7 +149,7 @@ gd_status gd_backend_sdpa_decode_at(gd_backend *backend, const gd_backend_tensor
         args->cache_pos < 0 || (int64_t)args->cache_pos > k_cache->shape[1] ||
         q->shape[1] > k_cache->shape[1] - (int64_t)args->cache_pos)
         return GD_ERR_INVALID_ARGUMENT;
-    return dispatch(backend, q, k_cache, v_cache, NULL, out, args, GD_HIP_SDPA_POS_SCALAR);
+    return dispatch(backend, q, k_cache, v_cache, NULL, out, args, GD_HIP_SDPA_POS_SCALAR, false);
 }
 
 gd_status gd_backend_sdpa_decode_positions(gd_backend *backend, const gd_backend_tensor_view *q,
@@ -143,5 +163,22 @@ gd_status gd_backend_sdpa_decode_positions(gd_backend *backend, const gd_backend
         cache_pos->dtype != GD_BACKEND_DTYPE_I32 || cache_pos->rank != 1u || cache_pos->shape[0] != q->shape[0] ||
         (cache_pos->offset & 3u) != 0u || !args_ok(args, k_cache))
         return GD_ERR_INVALID_ARGUMENT;
-    return dispatch(backend, q, k_cache, v_cache, cache_pos, out, args, GD_HIP_SDPA_POS_VECTOR);
+    return dispatch(backend, q, k_cache, v_cache, cache_pos, out, args, GD_HIP_SDPA_POS_VECTOR, false);
+}
+
+/* The per-row-positions form for callers that cannot allocate device memory: same validation, same kernels and
+ * therefore the same bits as gd_backend_sdpa_decode_positions; the split-KV partial results use the library's
+ * fixed device array instead of the backend's grown workspace.  No hipMalloc / hipFree on any path. */
+gd_status gd_backend_sdpa_decode_positions_noalloc(gd_backend *backend, const gd_backend_tensor_view *q,
+                                                   const gd_backend_tensor_view *k_cache,
+                                                   const gd_backend_tensor_view *v_cache,
+                                                   const gd_backend_tensor_view *cache_pos,
+                                                   const gd_backend_tensor_view *out,
+                                                   const gd_backend_sdpa_decode_args *args)
+{
+    if (backend == NULL || !common_ok(q, k_cache, v_cache, out) || !gd_hip_view_ok(cache_pos) ||
+        cache_pos->dtype != GD_BACKEND_DTYPE_I32 || cache_pos->rank != 1u || cache_pos->shape[0] != q->shape[0] ||
+        (cache_pos->offset & 3u) != 0u || !args_ok(args, k_cache))
+        return GD_ERR_INVALID_ARGUMENT;
+    return dispatch(backend, q, k_cache, v_cache, cache_pos, out, args, GD_HIP_SDPA_POS_VECTOR, true);
 }

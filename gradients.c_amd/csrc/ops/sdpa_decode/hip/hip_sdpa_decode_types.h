@@ -6,6 +6,11 @@
 #define GD_HIP_SDPA_POS_TENSOR0 1u /* pos[0] for every batch row */
 #define GD_HIP_SDPA_POS_VECTOR 2u  /* pos[b] */
 
+/* size of the fixed device array behind gd_backend_sdpa_decode_positions_noalloc
+ * (= GD_BACKEND_SDPA_DECODE_NOALLOC_SCRATCH_BYTES of the public header) */
+#define GD_HIP_SDPA_NOALLOC_SCRATCH_BYTES (8u << 20)
+#define GD_HIP_SDPA_MAX_DEVICES 16
+
 typedef struct gd_hip_sdpa_decode_params {
     uint32_t batch, tq, tmax, hq, hkv, dh;
     uint32_t window, prefix_len;

@@ -420,6 +420,34 @@ gd_sdpa_decode_generic_kernel(const T *__restrict__ q, const T *__restrict__ kc,
     }
 }
 
+/* ---- fixed scratch of the entry point that allocates nothing ------------------------------ */
+
+/* Split-KV partial results of gd_backend_sdpa_decode_positions_noalloc live here instead of a hipMalloc'd
+ * workspace.  Every device that loads this code object holds its own copy at its own address until the
+ * process ends; the address is looked up once per device (with that device current) and kept, and host code
+ * uses the kept pointer only: the array's name is a host-side stand-in, not a device address.  The split
+ * kernel writes (max, sum) of every (row, head, split) slot, also of splits without keys, and the combine
+ * kernel skips the accumulator of such a slot, so nothing has to be cleared between calls. */
+static __device__ __align__(256) float scratch[GD_HIP_SDPA_NOALLOC_SCRATCH_BYTES / sizeof(float)];
+static float *gd_scratch_ptr[GD_HIP_SDPA_MAX_DEVICES];
+
+extern "C" int gd_hip_sdpa_decode_scratch_init(int device)
+{
+    float *ptr = nullptr;
+    if (device < 0 || device >= GD_HIP_SDPA_MAX_DEVICES) return (int)hipErrorInvalidDevice;
+    if (gd_scratch_ptr[device] != nullptr) return (int)hipSuccess;
+    const hipError_t e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    gd_scratch_ptr[device] = ptr;
+    return (int)hipSuccess;
+}
+
+/* NULL until gd_hip_sdpa_decode_scratch_init(device) has succeeded. */
+extern "C" float *gd_hip_sdpa_decode_scratch(int device)
+{
+    return device >= 0 && device < GD_HIP_SDPA_MAX_DEVICES ? gd_scratch_ptr[device] : nullptr;
+}
+
 /* ---- launchers ----------------------------------------------------------------------- */
 
 template <int D, int G>

@@ -539,6 +539,24 @@ gd_status gd_backend_device_info(const gd_backend *backend, char *name, size_t n
  * Unknown name -> GD_ERR_INVALID_ARGUMENT. */
 gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t value);
 
+/* gd_backend_sdpa_decode_positions for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * arguments, validation, kernels and result bits as gd_backend_sdpa_decode_positions; the split-KV partial
+ * results (needed when batch * kv heads is below the number of compute units and the key range is split) go to a
+ * fixed device array of GD_BACKEND_SDPA_DECODE_NOALLOC_SCRATCH_BYTES that the library holds on every GPU it runs
+ * on until the process ends, instead of the backend's workspace that grows by hipMalloc.  A call whose partial
+ * results (batch * q heads * splits * (head size + 2) * 4 bytes) exceed that size returns GD_ERR_OUT_OF_MEMORY
+ * and prints the two sizes on stderr; nothing is launched.  The call makes no hipMalloc / hipFree and may be
+ * captured.  All calls on one GPU share the array: calls that overlap on one GPU (two backends, two streams)
+ * race; calls on one backend are ordered by its stream. */
+#define GD_BACKEND_SDPA_DECODE_NOALLOC_SCRATCH_BYTES (8u << 20)
+gd_status gd_backend_sdpa_decode_positions_noalloc(gd_backend *backend, const gd_backend_tensor_view *q,
+                                                   const gd_backend_tensor_view *k_cache,
+                                                   const gd_backend_tensor_view *v_cache,
+                                                   const gd_backend_tensor_view *cache_pos,
+                                                   const gd_backend_tensor_view *out,
+                                                   const gd_backend_sdpa_decode_args *args);
+
 /* Raw device address of a buffer (base of the allocation). */
 void *gd_backend_buffer_device_ptr(gd_backend_buffer *buffer);
 

@@ -37,6 +37,7 @@ GD_NULL_OP(gd_backend_sample_advance)
 GD_NULL_OP(gd_backend_sdpa_decode)
 GD_NULL_OP(gd_backend_sdpa_decode_at)
 GD_NULL_OP(gd_backend_sdpa_decode_positions)
+GD_NULL_OP(gd_backend_sdpa_decode_positions_noalloc)
 GD_NULL_OP(gd_backend_sdpa_varlen)
 GD_NULL_OP(gd_backend_swiglu_split_forward)
 GD_NULL_OP(gd_backend_swiglu_split_linear)
