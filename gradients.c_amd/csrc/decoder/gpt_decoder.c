@@ -48,7 +48,7 @@ struct gd_gpt_decoder {
     bool resident_x0;     /* x0_dev is kept current by the greedy-pick kernel */
     /* open resident session */
     bool resident_open;
-    int32_t resident_max_steps, resident_steps, resident_hold, resident_unfused;
+    int32_t resident_max_steps, resident_steps, resident_hold, resident_unfused, resident_keep_logits;
     gd_backend_graph *resident_graph;
     gd_tensor resident_out_ids, resident_out_gaps;
     /* sampling front end (state arena): what the reference's generation loop keeps on the host */
@@ -303,6 +303,7 @@ gd_tensor *gd_gpt_decoder_tensor(gd_gpt_decoder *d, const char *name, int32_t la
     if (!strcmp(name, "w_down")) return &b->down_proj.weight;
     if (!strcmp(name, "w_down_t")) return &b->down_t;
     if (!strcmp(name, "b_down")) return &b->down_proj.bias;
+    if (!strcmp(name, "last_logits")) return &d->last_logits;
     if (!strcmp(name, "k_cache")) return &d->k_cache[layer];
     if (!strcmp(name, "v_cache")) return &d->v_cache[layer];
     return NULL;
@@ -962,6 +963,15 @@ static gd_status enqueue_sample(gd_gpt_decoder *d, const gd_tensor *logits, int3
     return gd_backend_sample_advance(gd_context_backend(d->ctx), &vl, &t, &a);
 }
 
+/* GD_GPT_RESIDENT_KEEP_LOGITS: the step's logits into the state tensor that outlives the step scope */
+static gd_status keep_logits(gd_gpt_decoder *d, const gd_tensor *logits)
+{
+    return gd_backend_copy(gd_context_backend(d->ctx), (gd_backend_buffer *)d->last_logits.storage.buffer,
+                           d->last_logits.storage.offset + d->last_logits.view_offset,
+                           (gd_backend_buffer *)logits->storage.buffer, logits->storage.offset + logits->view_offset,
+                           (size_t)d->cfg.batch * (size_t)d->cfg.vocab * 2U);
+}
+
 static gd_status enqueue_resident_step(gd_gpt_decoder *d)
 {
     gd_context *ctx = d->ctx;
@@ -992,6 +1002,7 @@ static gd_status enqueue_resident_step(gd_gpt_decoder *d)
         /* greedy pick, token feedback, position and record keeping in one launch */
         gd_backend_tensor_view vl;
         TRY(enqueue_fused_step(d, &logits));
+        if (d->resident_keep_logits) TRY(keep_logits(d, &logits));
         tview(&logits, &vl);
         view1(&d->ids_dev, &vi);
         view1(&d->pos_dev, &vp);
@@ -1008,6 +1019,7 @@ static gd_status enqueue_resident_step(gd_gpt_decoder *d)
         return gd_backend_argmax_advance(gd_context_backend(ctx), &vl, &vi, &vp, &vs, &vo, &vog, d->resident_hold ? 0 : 1,
                                          NULL, NULL);
     }
+    if (d->resident_keep_logits) TRY(keep_logits(d, &logits));
     view1(&next, &vn);
     view1(&gaps, &vg);
     view1(&d->ids_dev, &vi);
@@ -1064,6 +1076,7 @@ static gd_status resident_begin_impl(gd_gpt_decoder *d, const int32_t *first_ids
     if (sampling != NULL) d->sampling = *sampling;
     /* the fused rope + append kernel needs NeoX pairs of a head size that is a multiple of 16 */
     d->resident_unfused = (flags & GD_GPT_RESIDENT_UNFUSED) != 0 || (d->cfg.head_dim % 16) != 0;
+    d->resident_keep_logits = sampling == NULL && (flags & GD_GPT_RESIDENT_KEEP_LOGITS) != 0;
     dims[0] = (int64_t)max_steps * d->cfg.batch;
     st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_I32, gd_shape_make(1U, dims), 256U, &d->resident_out_ids);
     if (st == GD_OK) st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F32, gd_shape_make(1U, dims), 256U, &d->resident_out_gaps);

@@ -328,9 +328,9 @@ class GptDecoder:
         self.ctx.check(st, "gd_gpt_decoder_generate")
         return [out[b, :counts[b]].copy() for b in range(self.cfg.batch)]
 
-    def resident_begin(self, first_ids, max_steps, hold_positions=False, unfused=False):
+    def resident_begin(self, first_ids, max_steps, hold_positions=False, unfused=False, keep_logits=False):
         first = np.ascontiguousarray(first_ids, np.int32)
-        flags = (1 if hold_positions else 0) | (2 if unfused else 0)
+        flags = (1 if hold_positions else 0) | (2 if unfused else 0) | (4 if keep_logits else 0)
         self.ctx.check(lib().gd_gpt_decoder_resident_begin(self.handle, first.ctypes.data_as(_vp), max_steps, flags),
                        "gd_gpt_decoder_resident_begin")
         self._resident_max = max_steps  # only a session that opened sizes what resident_end downloads

@@ -118,9 +118,13 @@ gd_status gd_gpt_decoder_step(gd_gpt_decoder *dec, const int32_t *ids, int32_t *
  *                                   it the step uses the fused backend entry points
  *                                   (gd_backend_fused_linear, gd_backend_qkv_rope_append: 5 launches
  *                                   per layer), which keep every rounding point of the separate
- *                                   operators. */
+ *                                   operators;
+ *   GD_GPT_RESIDENT_KEEP_LOGITS     every step also copies its logits [batch, vocab] into the decoder's
+ *                                   "last_logits" tensor (one more launch per step; greedy sessions only):
+ *                                   after sync it holds the logits of the last step run. */
 #define GD_GPT_RESIDENT_HOLD_POSITIONS 1
 #define GD_GPT_RESIDENT_UNFUSED 2
+#define GD_GPT_RESIDENT_KEEP_LOGITS 4
 gd_status gd_gpt_decoder_resident_begin(gd_gpt_decoder *dec, const int32_t *first_ids, int32_t max_steps,
                                         int32_t flags);
 gd_status gd_gpt_decoder_resident_run(gd_gpt_decoder *dec, int32_t n_steps);
