@@ -43,11 +43,13 @@ struct gd_backend {
      * for the one GD_HIP_GRAPH_RING events back */
     hipEvent_t graph_events[GD_HIP_GRAPH_RING];
     unsigned graph_launches;
+    /* what the last sdpa_decode dispatch launched: 0 none, 1 split, 2 generic; D, G, W, U, streaming, prefix, grid */
+    uint32_t last_sdpa[11];
     /* tunables read from the environment once at creation */
     int sdpa_chunk;      /* keys per workgroup in the split-KV decode kernel (0 = automatic) */
     int sdpa_waves;      /* 4 or 8 wavefronts per workgroup (0 = default 8) */
     int sdpa_unroll;     /* 4 or 8 key-row loads in flight per lane (0 = default 8) */
-    int sdpa_nontemporal; /* 1: streaming hint on the K/V loads */
+    int sdpa_nontemporal; /* streaming hint on the K/V loads: 1 always, 0 never, -1 by the size of the caches */
     int m3_simple;        /* 1: MiniMax-M3 operators always take the per-row kernels (tests compare the two paths) */
     int linear_tiles;    /* few-row projections: 16-column tiles per workgroup, 1 / 2 / 4 (0 = automatic) */
     int linear_waves;    /* few-row projections: wavefronts per workgroup = K split, 4 / 8 (0 = automatic) */

@@ -530,7 +530,8 @@ gd_status gd_backend_device_info(const gd_backend *backend, char *name, size_t n
 /* Kernel tunables, normally left at 0 = automatic.  name "sdpa_chunk": keys per workgroup of
  * the split-KV decode kernel (also read once from the environment variable
  * GD_HIP_SDPA_CHUNK); "sdpa_waves" (4 or 8 wavefronts per workgroup) and "sdpa_unroll" (2, 4 or 8
- * key-row loads per lane and trip) of the same kernel.  "linear_tiles" (1, 2 or 4 column tiles of 16
+ * key-row loads per lane and trip) of the same kernel; "sdpa_nontemporal" (GD_HIP_SDPA_NONTEMPORAL): 1 = mark its
+ * K/V loads streaming, 0 = never, -1 (default) = when the caches of the call exceed 128 MiB.  "linear_tiles" (1, 2 or 4 column tiles of 16
  * per workgroup) and "linear_waves" (4 or 8 wavefronts sharing the K range) of the few-row projection
  * kernel (environment: GD_HIP_LINEAR_TILES, GD_HIP_LINEAR_WAVES).  "m3_simple" = 1: the MiniMax-M3 operators
  * take their per-row kernels also where the matrix-core kernels apply (head size 64, block size a multiple of 64).
@@ -538,6 +539,12 @@ gd_status gd_backend_device_info(const gd_backend *backend, char *name, size_t n
  * also where it would stage the weight stream through LDS (same results to the bit; for comparing the two).
  * Unknown name -> GD_ERR_INVALID_ARGUMENT. */
 gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t value);
+
+/* Name of the kernel instantiation the most recent gd_backend_sdpa_decode{,_at,_positions} call on this backend
+ * launched, as a kernel trace prints it (e.g. "gd_sdpa_decode_split_kernel<64,1,4,2,false>"), followed by its
+ * grid in brackets; written to out as a NUL-terminated string of at most capacity bytes.  No counterpart in the
+ * reference (measurement aid: bench.py labels its roofline with it).  GD_ERR_BAD_STATE before the first call. */
+gd_status gd_backend_sdpa_decode_last_kernel(gd_backend *backend, char *out, size_t capacity);
 
 /* gd_backend_sdpa_decode_positions for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same

@@ -36,6 +36,7 @@ GD_NULL_OP(gd_backend_rms_norm_forward)
 GD_NULL_OP(gd_backend_sample_advance)
 GD_NULL_OP(gd_backend_sdpa_decode)
 GD_NULL_OP(gd_backend_sdpa_decode_at)
+GD_NULL_OP(gd_backend_sdpa_decode_last_kernel)
 GD_NULL_OP(gd_backend_sdpa_decode_positions)
 GD_NULL_OP(gd_backend_sdpa_decode_positions_noalloc)
 GD_NULL_OP(gd_backend_sdpa_varlen)

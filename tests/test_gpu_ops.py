@@ -256,6 +256,33 @@ def test_decode_isolated_config_shape(backend, arena, oracle, chunk):
     _close(out.read(), oracle.sdpa_decode(q, wk, wv, L, 0.125))
 
 
+@pytest.mark.parametrize("D,chunk", [(64, 0), (64, 32), (128, 0), (128, 64)])
+def test_decode_ignores_rows_behind_the_live_range(backend, arena, oracle, D, chunk):
+    """Cache rows behind a sequence's last live key may hold anything (another request's rows, NaN, infinities): the
+    result must not depend on them.  Every row from position + 1 on is filled with NaN (K) and infinities (V); rows
+    with 1, 2, 7, 33 and 300 live keys plus a full one, so that the first loads of a workgroup reach behind the
+    range in every way."""
+    B, H, Tmax = 6, 4, 384
+    pos = np.array([0, 1, 6, 32, 299, Tmax - 1], np.int32)
+    q = oracle.normal_f16((B, 1, H, D), 50)
+    k, v = oracle.normal_f16((B, Tmax, H, D), 51), oracle.normal_f16((B, Tmax, H, D), 52)
+    kd, vd = k.copy(), v.copy()
+    for b in range(B):
+        kd[b, pos[b] + 1:] = np.nan
+        vd[b, pos[b] + 1:] = np.inf
+        vd[b, pos[b] + 1::2] = -np.inf
+    out = arena.from_numpy(np.full(q.shape, 7.0, np.float16))
+    backend.set_tunable("sdpa_chunk", chunk)
+    try:
+        backend.sdpa_decode_positions(arena.from_numpy(q), arena.from_numpy(kd), arena.from_numpy(vd),
+                                      arena.from_numpy(pos), out, 1.0 / np.sqrt(D))
+    finally:
+        backend.set_tunable("sdpa_chunk", 0)
+    got = out.read()
+    assert np.isfinite(got.astype(np.float32)).all()
+    _close(got, oracle.sdpa_decode(q, k, v, pos, 1.0 / np.sqrt(D)))
+
+
 def test_decode_full_size_long_context_sampled(backend, oracle):
     """BASELINE config 3's attention at its full size (B=16, 16 heads of 128, 4096-row caches, live lengths in
     [1024, 4096]: 537 MB of cache filled on the device), checked on sampled batch rows against a float64 softmax of
