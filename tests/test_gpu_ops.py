@@ -283,6 +283,40 @@ def test_decode_ignores_rows_behind_the_live_range(backend, arena, oracle, D, ch
     _close(got, oracle.sdpa_decode(q, k, v, pos, 1.0 / np.sqrt(D)))
 
 
+@pytest.mark.parametrize("B,H,Hkv,D,Tmax,window,per_unit", [
+    (5, 4, 4, 64, 700, 0, 1), (5, 4, 4, 128, 700, 0, 2), (70, 2, 2, 64, 130, 0, 1), (9, 8, 2, 64, 300, 0, 1),
+    (6, 8, 1, 128, 257, 0, 2), (7, 4, 2, 64, 500, 96, 1), (4, 2, 2, 128, 2100, 0, 1), (130, 1, 1, 64, 40, 7, 2)])
+def test_decode_keys_dealt_by_count(backend, arena, oracle, B, H, Hkv, D, Tmax, window, per_unit):
+    """The form of the split-KV kernel that deals the visible keys of all rows to the wavefronts by count (only on
+    request): ragged positions with one-key rows, full rows, rows past the cache end
+    and rows with a negative position (left untouched: the sentinel stays), first and last rows among them; more
+    rows than a wavefront has lanes; grouped query heads; windows.  Rows behind a position hold NaN."""
+    rng = np.random.default_rng(B * 1000 + Tmax)
+    pos = rng.integers(0, Tmax, B).astype(np.int32)
+    pos[0], pos[B - 1], pos[B // 2] = -1, -3, Tmax + 5
+    pos[1], pos[2] = 0, Tmax - 1
+    q = oracle.normal_f16((B, 1, H, D), 60)
+    k, v = oracle.normal_f16((B, Tmax, Hkv, D), 61), oracle.normal_f16((B, Tmax, Hkv, D), 62)
+    kd, vd = k.copy(), v.copy()
+    for b in range(B):
+        if 0 <= pos[b] < Tmax - 1:
+            kd[b, pos[b] + 1:] = np.nan
+            vd[b, pos[b] + 1:] = np.nan
+    sentinel = np.full(q.shape, 7.0, np.float16)
+    out = arena.from_numpy(sentinel)
+    backend.set_tunable("sdpa_balanced", per_unit)
+    try:
+        backend.sdpa_decode_positions(arena.from_numpy(q), arena.from_numpy(kd), arena.from_numpy(vd),
+                                      arena.from_numpy(pos), out, 1.0 / np.sqrt(D), window)
+        assert "balanced" in backend.sdpa_decode_last_kernel()
+    finally:
+        backend.set_tunable("sdpa_balanced", 0)
+    got = out.read()
+    assert np.isfinite(got.astype(np.float32)).all()
+    assert (got[0] == 7.0).all() and (got[B - 1] == 7.0).all()
+    _close(got, oracle.sdpa_decode(q, k, v, pos, 1.0 / np.sqrt(D), window, out_init=sentinel.astype(np.float32)))
+
+
 def test_decode_full_size_long_context_sampled(backend, oracle):
     """BASELINE config 3's attention at its full size (B=16, 16 heads of 128, 4096-row caches, live lengths in
     [1024, 4096]: 537 MB of cache filled on the device), checked on sampled batch rows against a float64 softmax of
@@ -306,6 +340,12 @@ def test_decode_full_size_long_context_sampled(backend, oracle):
                 backend.set_tunable("sdpa_chunk", 0)
             results.append(out.read().astype(np.float32))
         assert np.abs(results[0] - results[1]).max() < 1e-3 and np.abs(results[0] - results[2]).max() < 1e-3
+        backend.set_tunable("sdpa_balanced", 1)    # the keys dealt to the wavefronts by count
+        try:
+            backend.sdpa_decode_positions(tq, k, v, tp, out, scale)
+        finally:
+            backend.set_tunable("sdpa_balanced", 0)
+        assert np.abs(results[0] - out.read().astype(np.float32)).max() < 1e-3
         for b in (0, 7, 15):
             n = int(pos[b]) + 1
             kb = k.rows(b, 1).read()[0, :n].astype(np.float64)  # [n, H, D]
