@@ -113,6 +113,7 @@ gd_status gd_backend_create_default(gd_backend **out_backend)
     b->sdpa_chunk = env_int("GD_HIP_SDPA_CHUNK", 0, 32, 1 << 20);
     b->sdpa_waves = env_int("GD_HIP_SDPA_WAVES", 0, 4, 8);
     b->sdpa_unroll = env_int("GD_HIP_SDPA_UNROLL", 0, 2, 8);
+    b->linear_wide = env_int("GD_HIP_LINEAR_WIDE", -1, -1, 1);
     b->sdpa_balanced = env_int("GD_HIP_SDPA_BALANCED", 0, 0, 2);
     b->sdpa_nontemporal = env_int("GD_HIP_SDPA_NONTEMPORAL", -1, -1, 1);
     b->linear_tiles = env_int("GD_HIP_LINEAR_TILES", 0, 1, 4);
@@ -169,6 +170,11 @@ gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t 
     if (strcmp(name, "m3_simple") == 0) {
         if (value != 0 && value != 1) return GD_ERR_INVALID_ARGUMENT;
         backend->m3_simple = (int)value;
+        return GD_OK;
+    }
+    if (strcmp(name, "linear_wide") == 0) {
+        if (value < -1 || value > 1) return GD_ERR_INVALID_ARGUMENT;
+        backend->linear_wide = (int)value;
         return GD_OK;
     }
     if (strcmp(name, "sdpa_balanced") == 0) {

@@ -8,7 +8,8 @@
 
 int gd_hip_launch_linear(hipStream_t stream, const void *x, const void *w, const void *bias, const void *residual,
                          const void *norm_w, void *y, const gd_hip_linear_params *params, int vector_ok,
-                         int kn_vector_ok, int store_vector_ok, int min_workgroups, const gd_hip_rope_epilogue *rope);
+                         int kn_vector_ok, int store_vector_ok, int min_workgroups, const gd_hip_rope_epilogue *rope,
+                         int wide_mode);
 
 static gd_status project_full(gd_backend *backend, const gd_backend_matrix_view *x, const gd_backend_matrix_view *w,
                               const gd_backend_vector_view *bias, const gd_backend_matrix_view *residual,
@@ -76,7 +77,7 @@ static gd_status project_full(gd_backend *backend, const gd_backend_matrix_view 
     return gd_hip_finish_op(backend, gd_hip_launch_linear(
         backend->stream, gd_hip_matrix_ptr(x), gd_hip_matrix_ptr(w), bias != NULL ? gd_hip_vector_ptr(bias) : NULL,
         residual != NULL ? gd_hip_matrix_ptr(residual) : NULL, norm_w != NULL ? gd_hip_vector_ptr(norm_w) : NULL,
-        gd_hip_matrix_ptr(y), &p, vec, kn_vec, store_vec, 2 * backend->compute_units, NULL));
+        gd_hip_matrix_ptr(y), &p, vec, kn_vec, store_vec, 2 * backend->compute_units, NULL, backend->linear_wide));
 }
 
 static gd_status project(gd_backend *backend, const gd_backend_matrix_view *x, const gd_backend_matrix_view *w,
@@ -208,5 +209,6 @@ gd_status gd_backend_fused_qkv_rope_append(gd_backend *backend, const gd_backend
     r.v_cache = gd_hip_view_ptr(v_cache);
     return gd_hip_finish_op(backend, gd_hip_launch_linear(
         backend->stream, gd_hip_matrix_ptr(x), gd_hip_matrix_ptr(w), bias != NULL ? gd_hip_vector_ptr(bias) : NULL, NULL,
-        norm_weight != NULL ? gd_hip_vector_ptr(norm_weight) : NULL, NULL, &p, 1, 0, 0, 2 * backend->compute_units, &r));
+        norm_weight != NULL ? gd_hip_vector_ptr(norm_weight) : NULL, NULL, &p, 1, 0, 0, 2 * backend->compute_units, &r,
+        backend->linear_wide));
 }

@@ -99,6 +99,12 @@ static void launch_stream(hipStream_t stream, const gd_half *x, const gd_half *w
 #undef GD_GO
 }
 
+/* linear_wide.hip: the projections of the wide decoders (megabytes of [N,K] weights, fewer than 128 rows) */
+extern "C" int gd_hip_try_launch_linear_wide(hipStream_t stream, const void *x, const void *w, const void *bias,
+                                             const void *residual, const void *norm_w, void *y,
+                                             const gd_hip_linear_params *params, const gd_hip_rope_epilogue *rope_epilogue,
+                                             uint64_t min_bytes, uint32_t tiles, uint32_t units);
+
 extern "C" int gd_hip_launch_linear_tile(hipStream_t stream, const void *x, const void *w, const void *bias,
                                          const void *residual, const void *norm_w, void *y,
                                          const gd_hip_linear_params *params, int big_tiles, int vector_store,
@@ -106,11 +112,12 @@ extern "C" int gd_hip_launch_linear_tile(hipStream_t stream, const void *x, cons
 
 /* vector_ok: K % 8 == 0 and every pointer / pitch allows 16-byte fragment loads (for w only when it is [N,K]);
  * kn_vector_ok: w stored [K,N] with N % 8 == 0 and 16-byte aligned rows; store_vector_ok: y (and the residual)
- * rows allow 16-byte accesses.  min_workgroups: about two per compute unit. */
+ * rows allow 16-byte accesses.  min_workgroups: about two per compute unit.  wide_mode: see below. */
 extern "C" int gd_hip_launch_linear(hipStream_t stream, const void *x, const void *w, const void *bias,
                                     const void *residual, const void *norm_w, void *y,
                                     const gd_hip_linear_params *params, int vector_ok, int kn_vector_ok,
-                                    int store_vector_ok, int min_workgroups, const gd_hip_rope_epilogue *rope_epilogue)
+                                    int store_vector_ok, int min_workgroups, const gd_hip_rope_epilogue *rope_epilogue,
+                                    int wide_mode)
 {
     const gd_hip_rope_epilogue no_rope = {nullptr, nullptr, nullptr, nullptr, nullptr};
     const gd_hip_rope_epilogue &rope = rope_epilogue != nullptr ? *rope_epilogue : no_rope;
@@ -129,6 +136,13 @@ extern "C" int gd_hip_launch_linear(hipStream_t stream, const void *x, const voi
         const uint64_t big = (uint64_t)((p.M + 255u) / 256u) * ((p.N + out_cols - 1u) / out_cols);
         const uint32_t units = min_workgroups > 0 ? (uint32_t)min_workgroups / 2u : 256u;
         return gd_hip_launch_linear_tile(stream, x, w, bias, residual, norm_w, y, params, big >= units, store_vector_ok, (int)units);
+    } else if (wide_mode != 0 && p.w_is_nk &&
+               gd_hip_try_launch_linear_wide(stream, x, w, bias, residual, norm_w, y, params, rope_epilogue,
+                                             wide_mode > 0 ? 0u : (4ull << 20), p.force_tiles,
+                                             min_workgroups > 0 ? (uint32_t)min_workgroups / 2u : 256u)) {
+        /* weight matrices of megabytes: the kernel built around the weight stream (wide_mode: 0 never, 1 whenever it
+         * covers the call, -1 from 4 MiB of weights on; below that the launch latency decides and the stream kernel
+         * is shorter) */
     } else {
         /* columns per workgroup: 64, 32 or 16 (rows: always 16, further rows in grid.y; their weight re-reads
          * come from L2).  More columns reuse each activation fragment for more MFMAs and repeat the prologue

@@ -538,6 +538,9 @@ gd_status gd_backend_device_info(const gd_backend *backend, char *name, size_t n
  * per workgroup) and "linear_waves" (4 or 8 wavefronts sharing the K range) of the few-row projection
  * kernel (environment: GD_HIP_LINEAR_TILES, GD_HIP_LINEAR_WAVES).  "m3_simple" = 1: the MiniMax-M3 operators
  * take their per-row kernels also where the matrix-core kernels apply (head size 64, block size a multiple of 64).
+ * "linear_wide" (GD_HIP_LINEAR_WIDE): the kernel built around the weight stream for few-row projections over [N,K]
+ * weights (whole-line loads through an LDS ring, every row tile of up to 64 rows in one workgroup): 1 = wherever it
+ * covers the call, 0 = never, -1 (default) = from 4 MiB of weights on.
  * "linear_no_lds_stream" = 1: the few-row projection always loads its weight fragments straight into registers,
  * also where it would stage the weight stream through LDS (same results to the bit; for comparing the two).
  * Unknown name -> GD_ERR_INVALID_ARGUMENT. */

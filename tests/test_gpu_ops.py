@@ -942,6 +942,43 @@ def test_fused_linear_swiglu_epilogue(backend, arena, oracle, gda, M, K, H):
     assert backend.call("gd_backend_fused_linear", tx.matrix(), wk.matrix(), None, None, None, y.matrix(), C.byref(a)) == gda.UNSUPPORTED
 
 
+def test_few_row_projection_over_weights_on_both_sides_of_a_2_gib_boundary(backend, oracle, gda):
+    """The kernels that stream large weight matrices through LDS take the matrix's address as a scalar base plus
+    32-bit lane offsets.  The same matrix placed twice, 2 GiB apart: one of the two copies has an address whose low
+    word has its top bit set (a sign extension of that word once sent the loads of such a copy to invalid
+    addresses).  rms_norm + up/gate + swiglu (the persistent form) and projection + residual (one tile per
+    workgroup), both copies against the oracle and against each other to the bit."""
+    M, K, H = 16, 2048, 1024
+    big = backend.buffer((2 << 30) + (96 << 20))
+    try:
+        x = oracle.normal_f16((M, K), 3100, 1.3)
+        nw = (1.0 + 0.1 * oracle.normal_f16((K,), 3101).astype(np.float32)).astype(np.float16)
+        w = oracle.normal_f16((2 * H, K), 3102, 0.05)
+        bias = oracle.normal_f16((2 * H,), 3103, 0.5)
+        res = oracle.normal_f16((M, 2 * H), 3104, 1.0)
+        tx, tn, tb, tr = (big.from_numpy(a) for a in (x, nw, bias, res))
+        y1, y2 = big.alloc((M, H), gda.F16), big.alloc((M, 2 * H), gda.F16)
+        first = big.alloc((2 * H, K), gda.F16).write(w)
+        second = gda.Tensor(big, first.offset + (2 << 30), (2 * H, K), gda.F16).write(w)
+        backend.set_tunable("linear_wide", 1)
+        got = []
+        for tw in (first, second):
+            backend.fill(y1, 0x7e00)
+            backend.fill(y2, 0x7e00)
+            backend.fused_linear(tx, tw, tb, None, tn, y1, True, 2, 2, 1e-5, epilogue=1)
+            backend.fused_linear(tx, tw, tb, tr, None, y2, True, 2, 0)
+            got.append((y1.read(), y2.read()))
+        assert np.array_equal(_bits(got[0][0]), _bits(got[1][0])) and np.array_equal(_bits(got[0][1]), _bits(got[1][1]))
+        u = oracle.linear_nt(oracle.rms_norm(x, nw, 1e-5), w, bias)
+        through = (np.abs(u[:, :H].astype(np.float64)) + np.abs(bias[:H].astype(np.float64))) * \
+                  (1.0 + np.abs(u[:, H:].astype(np.float64)) + np.abs(bias[H:].astype(np.float64)))
+        _close(got[0][0], oracle.swiglu_split(u), through=through)
+        _close(got[0][1], oracle.add(res, oracle.linear_nt(x, w, bias)), through=res)
+    finally:
+        backend.set_tunable("linear_wide", -1)
+        backend.free(big)
+
+
 @pytest.mark.parametrize("M,N,gated", [(16, 5632, True), (33, 8200, False), (64, 4096, True), (5, 32768, False)])
 def test_few_row_projection_weight_stream_through_lds(backend, arena, oracle, gda, M, N, gated):
     """rms_norm + projection with K = 2048 and 64 columns per workgroup stages its weight stream through LDS (whole
