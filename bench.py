@@ -322,7 +322,7 @@ def long_context_workload(a, oracle, D, which, steps=None, warmup=None, batches=
                           "prefill_tokens_per_s": round(n_tokens / prefill_s, 1),
                           "prefill_tflops": round(prefill_tflops, 1)}))
         return None
-    steps = (a.steps if steps is None else steps) if which == 3 else 128
+    steps = (a.steps if steps is None else steps) if which == 3 else a.decode_steps
     warmup = (a.warmup if warmup is None else warmup) if which == 3 else 0
     batches = batches if which == 3 else 1
     total = warmup + steps * batches
@@ -353,7 +353,7 @@ def long_context_workload(a, oracle, D, which, steps=None, warmup=None, batches=
         "workload": f"configs[{which}]: scaled decoder (V32768 Dm2048 L24 H16 Dh128 Hm5632, untied head), "
                     + ("B=16, caches of 1024..4095 tokens built by packed prefill, positions held"
                        if which == 3 else
-                       "32 prompts of 64..2048 tokens, packed prefill then 128 greedy steps with growing caches"),
+                       f"32 prompts of 64..2048 tokens, packed prefill then {steps} greedy steps with growing caches"),
         "decode_tokens_per_s": round(B * steps / elapsed, 1), "ms_per_step": round(ms_per_step, 5),
         "steps": steps, "warmup": warmup, "batches": batches, "batch": B, "prompt_tokens": n_tokens,
         "prefill_seconds": round(prefill_s, 4), "prefill_tokens_per_s": round(n_tokens / prefill_s, 1),
@@ -366,7 +366,7 @@ def long_context_workload(a, oracle, D, which, steps=None, warmup=None, batches=
     }
     if which == 4:
         out["end_to_end_tokens_per_s"] = round(B * steps / (elapsed + prefill_s), 1)
-        out["decode_note"] = "first step, graph capture and 127 replays inside the decode clock"
+        out["decode_note"] = f"first step, graph capture and {steps - 1} replays inside the decode clock"
         out["prefill_roofline"] = {"bound": "mfma", "achieved": round(prefill_tflops, 1), "peak": MFMA_F16_PEAK_TFLOPS,
                                    "unit": "TFLOP/s", "frac": round(prefill_tflops / MFMA_F16_PEAK_TFLOPS, 4),
                                    "note": "projection + visible-pair attention flops over the whole prefill call "
@@ -482,6 +482,13 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--batches", type=int, default=0,
+                    help="how many times the K steps are timed (the median batch is reported); default 5 for the headline "
+                         "line, 3 for --workload 3.  Kernel traces use --batches 1: rocprofv3's queue interception "
+                         "crashes the profiled process once the 16384 dispatch packets of a hardware queue's ring have "
+                         "been used and a graph launch wraps around its end")
+    ap.add_argument("--decode-steps", type=int, default=128,
+                    help="--workload 4: greedy steps after the prefill (BASELINE: 128; fewer for kernel traces, see --batches)")
     ap.add_argument("--headline-only", action="store_true",
                     help="skip the other BASELINE.json configs (the 'others' object of the line)")
     ap.add_argument("--workload", type=int, default=2, choices=(2, 3, 4),
@@ -513,7 +520,7 @@ def main():
         return
     from gradients_c_amd import decoder as D
     if a.workload != 2:
-        obj = long_context_workload(a, oracle, D, a.workload, batches=3 if a.workload == 3 else 1)
+        obj = long_context_workload(a, oracle, D, a.workload, batches=(a.batches or 3) if a.workload == 3 else 1)
         if obj is not None:
             print(json.dumps(long_context_line(a, obj, a.workload)))
         return
@@ -523,7 +530,7 @@ def main():
         return
 
     B, T = 64, 512
-    batches = 5
+    batches = a.batches or 5
     shape = (2048, 512, 3, 8, 64, 1536, T, B)
     cfg = D.gpt_config(*shape, window=0, tie_lm_head=False, seed=1002)
     dec = D.GptDecoder(cfg, max_prefill_tokens=B * (T - 1))
