@@ -82,6 +82,34 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
     const uint32_t m0 = blockIdx.y * 16u;
     const uint32_t mrow = min(m0 + (uint32_t)li, p.M - 1u);
 
+    /* What the epilogue will need of other tensors (bias values, the residual, the positions of the rope + append
+     * form) is requested here, in front of everything else: read behind the sum of the wavefronts, each would be one
+     * more dependent round trip at the end of a kernel that is a chain of round trips. */
+    constexpr int NTO_MAX = NT >= 2 ? NT : 1; /* output column tiles of the plain form (the paired forms have NT / 2) */
+    constexpr int EPT = (NTO_MAX * 256 + WAVES * 64 - 1) / (WAVES * 64);
+    gd_half pf_b1[EPT], pf_b2[EPT], pf_res[EPT];
+    int32_t pf_pos[EPT], pf_cpos[EPT];
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) {
+        const int idx = (int)threadIdx.x + i * WAVES * 64;
+        const int j = idx >> 8, rl = idx & 63, rr = (idx >> 6) & 3;
+        const uint32_t col = min(n0 + 16u * j + (rl & 15), p.N - 1u);
+        const uint32_t row = min(m0 + 4u * (rl >> 4) + rr, p.M - 1u);
+        pf_b1[i] = pf_b2[i] = pf_res[i] = (gd_half)0.f;
+        pf_pos[i] = pf_cpos[i] = 0;
+        if (idx < (gated ? NT / 2 : NT) * 256) {
+            if (p.epilogue != GD_HIP_EPI_NONE) {
+                pf_b1[i] = bias[col];
+                if (gated) pf_b2[i] = bias[pair_offset + col];
+            }
+            if (!gated && p.has_residual) pf_res[i] = residual[(size_t)row * p.ldr + col];
+            if (roped) {
+                pf_pos[i] = rope.rope_pos[row];
+                pf_cpos[i] = rope.cache_pos[row];
+            }
+        }
+    }
+
     /* K range of this wavefront, in steps of 32 */
     const uint32_t ksteps = (p.K + 31u) / 32u;
     const uint32_t per_wave = (ksteps + WAVES - 1u) / WAVES;
@@ -374,7 +402,10 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
     }
     __syncthreads();
     if (gated) {
-        for (int idx = threadIdx.x; idx < (NT / 2) * 256; idx += WAVES * 64) {
+#pragma unroll
+        for (int i = 0; i < EPT; ++i) {
+            const int idx = (int)threadIdx.x + i * WAVES * 64;
+            if (idx >= (NT / 2) * 256) break;
             const int j = idx >> 8, rl = idx & 63, rr = (idx >> 6) & 3;
             const uint32_t col = n0 + 16u * j + (rl & 15);
             const uint32_t row = m0 + 4u * (rl >> 4) + rr;
@@ -387,11 +418,11 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
             if (row < p.M && col < p.N) {
                 gd_half h1, h2;
                 if (p.epilogue == GD_HIP_EPI_BIAS_F32) {
-                    h1 = (gd_half)(v1 + (float)bias[col]);
-                    h2 = (gd_half)(v2 + (float)bias[pair_offset + col]);
+                    h1 = (gd_half)(v1 + (float)pf_b1[i]);
+                    h2 = (gd_half)(v2 + (float)pf_b2[i]);
                 } else if (p.epilogue == GD_HIP_EPI_BIAS_F16) {
-                    h1 = (gd_half)v1 + bias[col];
-                    h2 = (gd_half)v2 + bias[pair_offset + col];
+                    h1 = (gd_half)v1 + pf_b1[i];
+                    h2 = (gd_half)v2 + pf_b2[i];
                 } else {
                     h1 = (gd_half)v1;
                     h2 = (gd_half)v2;
@@ -406,7 +437,7 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
                     gd_half o1 = h1, o2 = h2;
                     if (section < 2u) {
                         float c, sn;
-                        gd_rope_cos_sin((float)rope.rope_pos[row], pair, p.rope_freq_scale, &c, &sn);
+                        gd_rope_cos_sin((float)pf_pos[i], pair, p.rope_freq_scale, &c, &sn);
                         gd_rope_rotate((float)h1, (float)h2, c, sn, &o1, &o2);
                     }
                     if (section == 0u) {
@@ -414,7 +445,7 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
                         dst[0] = o1;
                         dst[D / 2u] = o2;
                     } else {
-                        const int32_t cp = rope.cache_pos[row];
+                        const int32_t cp = pf_cpos[i];
                         if (cp >= 0 && (uint32_t)cp < p.rope_tmax) {
                             gd_half *dst = (gd_half *)(section == 1u ? rope.k_cache : rope.v_cache) +
                                            ((size_t)row * p.rope_tmax + (size_t)cp) * area + within;
@@ -428,7 +459,10 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
         return;
     }
     /* (result lane, register) pairs of the NT tiles are spread over the workgroup's threads */
-    for (int idx = threadIdx.x; idx < NT * 256; idx += WAVES * 64) {
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) {
+        const int idx = (int)threadIdx.x + i * WAVES * 64;
+        if (idx >= NT * 256) break;
         const int j = idx >> 8, rl = idx & 63, rr = (idx >> 6) & 3;
         const uint32_t col = n0 + 16u * j + (rl & 15);
         const uint32_t row = m0 + 4u * (rl >> 4) + rr;
@@ -437,10 +471,10 @@ gd_linear_stream_kernel(const gd_half *__restrict__ x, const gd_half *__restrict
         for (int wv = 0; wv < WAVES; ++wv) v += sm[wv][j][rl][rr];
         if (row < p.M && col < p.N) {
             gd_half h;
-            if (p.epilogue == GD_HIP_EPI_BIAS_F32) h = (gd_half)(v + (float)bias[col]);
-            else if (p.epilogue == GD_HIP_EPI_BIAS_F16) h = (gd_half)v + bias[col];
+            if (p.epilogue == GD_HIP_EPI_BIAS_F32) h = (gd_half)(v + (float)pf_b1[i]);
+            else if (p.epilogue == GD_HIP_EPI_BIAS_F16) h = (gd_half)v + pf_b1[i];
             else h = (gd_half)v;
-            if (p.has_residual) h = residual[(size_t)row * p.ldr + col] + h;
+            if (p.has_residual) h = pf_res[i] + h;
             y[(size_t)row * p.ldy + col] = h;
         }
     }

@@ -26,6 +26,8 @@ static void launch_persistent(hipStream_t stream, const void *x, const void *w, 
                               uint32_t units)
 {
     constexpr bool PAIRED = EPI != GD_WIDE_EPI_PLAIN;
+    /* as deep as LDS allows next to the sums of the wavefronts (NT x MT x 8 KB): 8 x RING x 2 KB; an eighth group for
+     * the two-tile forms changed nothing (12.5 against 12.2 us at 16 x 2048 -> 6144) */
     constexpr int RING = NT * MT <= 4 ? 7 : 5;
     const uint32_t cols = PAIRED ? 8u * NT : 16u * NT;
     const uint32_t outs = EPI == GD_WIDE_EPI_ROPE ? p.N / 2u : (EPI == GD_WIDE_EPI_SWIGLU ? p.swiglu_cols : p.N);
@@ -82,6 +84,8 @@ extern "C" int gd_hip_try_launch_linear_wide(hipStream_t stream, const void *x, 
             if (mt == 1u) GD_P(4, 1, GD_WIDE_EPI_PLAIN);
             GD_P(4, 2, GD_WIDE_EPI_PLAIN);
         }
+        /* four row tiles: the sums of 4 x 4 tiles would not fit next to the ring, so 32 columns per tile */
+        if (epi == GD_WIDE_EPI_PLAIN && (p.N % 32u) == 0u) GD_P(2, 4, GD_WIDE_EPI_PLAIN);
         if (epi == GD_WIDE_EPI_SWIGLU && tiles != 2u && (p.swiglu_cols % 32u) == 0u && mt <= 2u) {
             if (mt == 1u) GD_P(4, 1, GD_WIDE_EPI_SWIGLU);
             GD_P(4, 2, GD_WIDE_EPI_SWIGLU);
@@ -94,7 +98,9 @@ extern "C" int gd_hip_try_launch_linear_wide(hipStream_t stream, const void *x, 
         if (epi == GD_WIDE_EPI_ROPE && (p.rope_head_dim % 32u) == 0u && p.N == 3u * p.rope_heads * p.rope_head_dim) {
             if (mt == 1u) GD_P(2, 1, GD_WIDE_EPI_ROPE);
             if (mt == 2u) GD_P(2, 2, GD_WIDE_EPI_ROPE);
-            GD_P(2, 4, GD_WIDE_EPI_ROPE);
+            /* 33 rows or more: the stream kernel's four workgroups per column tile are faster here (20.7 against
+             * 22.3 us at 64 x 2048 -> 6144), the rotation of 64 rows weighs more than the second pass over L2 */
+            return 0;
         }
     }
 #undef GD_P
@@ -103,7 +109,7 @@ extern "C" int gd_hip_try_launch_linear_wide(hipStream_t stream, const void *x, 
         if (tiles != 2u && (p.swiglu_cols % 32u) == 0u) GD_W_MT(4, 4, GD_HIP_PRO_RMS_NORM, GD_WIDE_EPI_SWIGLU);
         if ((p.swiglu_cols % 16u) == 0u) GD_W_MT(2, 4, GD_HIP_PRO_RMS_NORM, GD_WIDE_EPI_SWIGLU);
     }
-    if (epi == GD_WIDE_EPI_ROPE && (p.rope_head_dim % 32u) == 0u && p.N == 3u * p.rope_heads * p.rope_head_dim)
+    if (epi == GD_WIDE_EPI_ROPE && (p.rope_head_dim % 32u) == 0u && p.N == 3u * p.rope_heads * p.rope_head_dim && mt <= 2u)
         GD_W_MT(2, 4, GD_HIP_PRO_RMS_NORM, GD_WIDE_EPI_ROPE);
 #undef GD_W_MT
 #undef GD_W
