@@ -57,7 +57,10 @@ __device__ __forceinline__ uint32_t gd_tile_slot(uint32_t row, uint32_t c)
 __device__ __forceinline__ float gd_tile_silu(float z)
 {
     const float e = __expf(-fabsf(z));
-    const float inv = 1.0f / (1.0f + e);
+    /* 1 / (1 + e) with e in (0, 1]: the reciprocal instruction is good to one unit in the last place of F32, and the
+     * product is rounded to F16 afterwards; the division's dozen instructions per element would make the gated
+     * epilogue of a tile a quarter longer */
+    const float inv = __builtin_amdgcn_rcpf(1.0f + e);
     return z * (z >= 0.0f ? inv : e * inv);
 }
 
@@ -93,15 +96,19 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
     const uint32_t total = tiles_m * tiles_n;
     constexpr bool DIRECT = PRO == GD_HIP_PRO_NONE;
     uint32_t m0 = 0u, n0 = 0u; /* origin of the current tile (rows, output columns) */
-    /* swiglu epilogue ([N,K] weights of 2H rows, H = p.N output columns): the first BN/2 weight rows of a tile are
-     * value rows n0 .., the others the gate rows H + n0 ..; the tile then owns BN/2 output columns */
+    /* swiglu epilogue ([N,K] weights of 2H rows, H = p.N output columns).  The BN weight rows of a tile are two
+     * wavefront columns of BN/2; each holds HW = BN/4 value rows (n0 + wc*HW ..) in its first half and the matching
+     * gate rows (H + n0 + wc*HW ..) in its second half, so a lane finds value and gate of one output column in
+     * its own accumulators (tiles j and j + WN/2).  The tile then owns BN/2 output columns. */
     const bool gated = p.swiglu_cols != 0u;
     const uint32_t out_bn = gated ? BN / 2u : BN;
+    constexpr uint32_t HW = BN / 4u;
     auto wrow = [&](uint32_t tn0, uint32_t r) __attribute__((always_inline)) {
-        return gated ? (r < BN / 2u ? tn0 + r : p.swiglu_cols + tn0 + (r - BN / 2u)) : tn0 + r;
+        const uint32_t wc = r / (BN / 2u), wr = r % (BN / 2u);
+        return gated ? (wr < HW ? tn0 + wc * HW + wr : p.swiglu_cols + tn0 + wc * HW + (wr - HW)) : tn0 + r;
     };
     auto wrow_ok = [&](uint32_t tn0, uint32_t r) __attribute__((always_inline)) {
-        return tn0 + (gated && r >= BN / 2u ? r - BN / 2u : r) < p.N;
+        return (gated ? tn0 + (r / (BN / 2u)) * HW + r % HW : tn0 + r) < p.N;
     };
     auto locate = [&](uint32_t t, uint32_t &tm0, uint32_t &tn0) __attribute__((always_inline)) {
         uint32_t pid = t;
@@ -418,24 +425,28 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
             }
         }
     };
+    /* the four columns of register quad q of accumulator tile a, rounded to F16 with the bias of the mode */
+    auto quad_f16 = [&](auto mode_tag, const gd_float16 &a, int j, int q) __attribute__((always_inline)) {
+        constexpr uint32_t MODE = decltype(mode_tag)::value;
+        gd_half4 h;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float v = a[4 * q + r];
+            if (MODE == GD_HIP_EPI_NONE) h[r] = (gd_half)v;
+            else if (MODE == GD_HIP_EPI_BIAS_F32) h[r] = (gd_half)(v + (float)bq[j][q][r]);
+            else h[r] = (gd_half)v + bq[j][q][r];
+        }
+        return h;
+    };
     auto epilogue_pass = [&](auto pass_tag, auto mode_tag) __attribute__((always_inline)) {
         constexpr int I = decltype(pass_tag)::value;
-        constexpr uint32_t MODE = decltype(mode_tag)::value;
         const uint32_t e = wm * 32u + frag_row;
 #pragma unroll
         for (int j = 0; j < WN; ++j) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const uint32_t lc = wn * (WN * 32u) + (uint32_t)j * 32u + 8u * (uint32_t)q + 4u * frag_c;
-                gd_half4 h;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const float v = acc[I][j][4 * q + r];
-                    if (MODE == GD_HIP_EPI_NONE) h[r] = (gd_half)v;
-                    else if (MODE == GD_HIP_EPI_BIAS_F32) h[r] = (gd_half)(v + (float)bq[j][q][r]);
-                    else h[r] = (gd_half)v + bq[j][q][r];
-                }
-                *reinterpret_cast<gd_half4 *>(epi + (e * EU + ((lc >> 2) ^ (e & 31u))) * 8u) = h;
+                *reinterpret_cast<gd_half4 *>(epi + (e * EU + ((lc >> 2) ^ (e & 31u))) * 8u) = quad_f16(mode_tag, acc[I][j], j, q);
             }
         }
         __syncthreads();
@@ -454,14 +465,16 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
             return h;
         };
         if (gated) {
-            /* value chunk v and gate chunk v + CPRW/2 of the same row make output chunk v */
+            /* a value chunk and the gate chunk HW/8 behind it make one output chunk */
 #pragma unroll
             for (uint32_t idx0 = 0; idx0 < 32u * CPRW; idx0 += 256u) {
                 const uint32_t idx = idx0 + tid;
                 const uint32_t er = idx / (CPRW / 2u), v = idx % (CPRW / 2u);
                 const uint32_t gr = m0 + (er >> 5) * (WM * 32u) + (uint32_t)I * 32u + (er & 31u), gc = n0 + v * 8u;
                 if (gr >= p.M || gc >= p.N) continue;
-                const gd_half8 hv = read_chunk(er, v), hg = read_chunk(er, v + CPRW / 2u);
+                /* staged columns: wavefront column wc holds its HW value columns, then their gates */
+                const uint32_t cv = (v / (HW / 8u)) * (HW / 4u) + v % (HW / 8u);
+                const gd_half8 hv = read_chunk(er, cv), hg = read_chunk(er, cv + HW / 8u);
                 gd_half8 h;
 #pragma unroll
                 for (int t = 0; t < 8; ++t) h[t] = (gd_half)((float)hv[t] * gd_tile_silu((float)hg[t]));
@@ -510,6 +523,118 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
             epilogue_pass(std::integral_constant<int, (WM > 2 ? 2 : 0)>{}, mode_tag);
             epilogue_pass(std::integral_constant<int, (WM > 2 ? 3 : 0)>{}, mode_tag);
         }
+    };
+
+    /* Epilogue of a whole 256-column tile whose rows can take 16-byte stores: no workgroup barriers.  A wavefront
+     * rounds its own 32 x 128 block of a pass, brings the two 8-byte pieces that lanes l and l + 32 hold of one
+     * 16-byte chunk into one lane (v_permlane32_swap), writes whole chunks into its own quarter of the buffer and
+     * reads them back as row pieces (16 lanes x 16 bytes per row, four rows per instruction; gated tiles, whose
+     * wavefront has already multiplied value and gate in registers: 8 lanes per row, eight rows).  LDS operations
+     * of one wavefront are carried out in order, so the next pass overwrites the quarter without a barrier.
+     * Chunk c of row e sits at e*16 + (c ^ (e & 15)) (gated: e*8 + (c ^ ((e >> 1) & 7))): 16 consecutive rows of
+     * one chunk, and the lanes of one read, hit all banks.  The residual rows of a pass are requested before its
+     * accumulators are rounded, so that their latency passes behind that work. */
+    typedef unsigned gd_uint2v __attribute__((ext_vector_type(2)));
+    auto pair_chunk = [&](gd_half4 a, gd_half4 b) __attribute__((always_inline)) {
+        union { gd_half4 h; uint32_t u[2]; } ua, ub;
+        ua.h = a;
+        ub.h = b;
+        /* lanes 32-63 of the first operand change places with lanes 0-31 of the second */
+        const gd_uint2v s0 = __builtin_amdgcn_permlane32_swap(ua.u[0], ub.u[0], false, false);
+        const gd_uint2v s1 = __builtin_amdgcn_permlane32_swap(ua.u[1], ub.u[1], false, false);
+        union { uint32_t u[4]; gd_half8 h; } c;
+        c.u[0] = s0[0];
+        c.u[1] = s1[0];
+        c.u[2] = s0[1];
+        c.u[3] = s1[1];
+        return c.h;
+    };
+    auto epilogue_own = [&](auto mode_tag) __attribute__((always_inline)) {
+        if (decltype(mode_tag)::value != GD_HIP_EPI_NONE) load_bias();
+        unsigned char *own = epi + wave * 8192u;
+        const uint32_t rr = lane >> 4, v = lane & 15u;
+        /* offsets of this lane's piece from the tile's first element; the pass and the row group add a uniform
+         * term */
+        const gd_half *rtile = residual + ((size_t)m0 * p.ldr + n0);
+        gd_half *ytile = y + ((size_t)m0 * p.ldy + n0);
+        const uint32_t y_lane = (wm * (WM * 32u) + rr) * p.ldy + wn * (WN * 32u) + v * 8u;
+        const uint32_t r_lane = (wm * (WM * 32u) + rr) * p.ldr + wn * (WN * 32u) + v * 8u;
+        auto pass = [&](auto pass_tag) __attribute__((always_inline)) {
+            constexpr int I = decltype(pass_tag)::value;
+            gd_half8 res[8];
+            if (p.has_residual) {
+#pragma unroll
+                for (uint32_t it = 0; it < 8u; ++it)
+                    res[it] = *reinterpret_cast<const gd_half8 *>(rtile + ((uint32_t)I * 32u + it * 4u) * p.ldr + r_lane);
+            }
+#pragma unroll
+            for (int j = 0; j < WN; ++j) {
+#pragma unroll
+                for (int pr = 0; pr < 2; ++pr) {
+                    const uint32_t c = (uint32_t)j * 4u + 2u * (uint32_t)pr + frag_c;
+                    *reinterpret_cast<gd_half8 *>(own + (frag_row * 16u + (c ^ (frag_row & 15u))) * 16u) =
+                        pair_chunk(quad_f16(mode_tag, acc[I][j], j, 2 * pr), quad_f16(mode_tag, acc[I][j], j, 2 * pr + 1));
+                }
+            }
+            gd_half8 h[8];
+#pragma unroll
+            for (uint32_t it = 0; it < 8u; ++it) {
+                const uint32_t e = it * 4u + rr;
+                h[it] = *reinterpret_cast<const gd_half8 *>(own + (e * 16u + (v ^ (e & 15u))) * 16u);
+            }
+#pragma unroll
+            for (uint32_t it = 0; it < 8u; ++it) {
+                if (p.has_residual) {
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) h[it][t] = res[it][t] + h[it][t];
+                }
+                *reinterpret_cast<gd_half8 *>(ytile + ((uint32_t)I * 32u + it * 4u) * p.ldy + y_lane) = h[it];
+            }
+        };
+        pass(std::integral_constant<int, 0>{});
+        pass(std::integral_constant<int, 1>{});
+        pass(std::integral_constant<int, (WM > 2 ? 2 : 0)>{});
+        pass(std::integral_constant<int, (WM > 2 ? 3 : 0)>{});
+    };
+    auto epilogue_own_gated = [&](auto mode_tag) __attribute__((always_inline)) {
+        if (decltype(mode_tag)::value != GD_HIP_EPI_NONE) load_bias();
+        unsigned char *own = epi + wave * 8192u;
+        const uint32_t rr = lane >> 3, v = lane & 7u;
+        gd_half *ytile = y + ((size_t)m0 * p.ldy + n0);
+        const uint32_t y_lane = (wm * (WM * 32u) + rr) * p.ldy + wn * HW + v * 8u;
+        auto pass = [&](auto pass_tag) __attribute__((always_inline)) {
+            constexpr int I = decltype(pass_tag)::value;
+#pragma unroll
+            for (int j = 0; j < WN / 2; ++j) {
+#pragma unroll
+                for (int pr = 0; pr < 2; ++pr) {
+                    gd_half4 o[2];
+#pragma unroll
+                    for (int s2 = 0; s2 < 2; ++s2) {
+                        const gd_half4 hv = quad_f16(mode_tag, acc[I][j], j, 2 * pr + s2);
+                        const gd_half4 hg = quad_f16(mode_tag, acc[I][j + WN / 2], j + WN / 2, 2 * pr + s2);
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) o[s2][t] = (gd_half)((float)hv[t] * gd_tile_silu((float)hg[t]));
+                    }
+                    const uint32_t c = (uint32_t)j * 4u + 2u * (uint32_t)pr + frag_c;
+                    *reinterpret_cast<gd_half8 *>(own + (frag_row * 8u + (c ^ ((frag_row >> 1) & 7u))) * 16u) =
+                        pair_chunk(o[0], o[1]);
+                }
+            }
+            gd_half8 h[4];
+#pragma unroll
+            for (uint32_t it = 0; it < 4u; ++it) {
+                const uint32_t e = it * 8u + rr;
+                h[it] = *reinterpret_cast<const gd_half8 *>(own + (e * 8u + (v ^ ((e >> 1) & 7u))) * 16u);
+            }
+#pragma unroll
+            for (uint32_t it = 0; it < 4u; ++it)
+                *reinterpret_cast<gd_half8 *>(ytile + ((uint32_t)I * 32u + it * 8u) * p.ldy + y_lane) = h[it];
+        };
+        pass(std::integral_constant<int, 0>{});
+        pass(std::integral_constant<int, 1>{});
+        pass(std::integral_constant<int, (WM > 2 ? 2 : 0)>{});
+        pass(std::integral_constant<int, (WM > 2 ? 3 : 0)>{});
     };
 
         /* interior tile: every staged chunk is in range, so the main loop carries no guards */
@@ -586,9 +711,17 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
             }
         }
 
-        if (p.epilogue == GD_HIP_EPI_BIAS_F32) epilogue(std::integral_constant<uint32_t, GD_HIP_EPI_BIAS_F32>{});
-        else if (p.epilogue == GD_HIP_EPI_BIAS_F16) epilogue(std::integral_constant<uint32_t, GD_HIP_EPI_BIAS_F16>{});
-        else epilogue(std::integral_constant<uint32_t, GD_HIP_EPI_NONE>{});
+        auto finish = [&](auto mode_tag) __attribute__((always_inline)) {
+            if (WM == 4 && WN == 4 && vector_store && m0 + BM <= p.M && n0 + out_bn <= p.N) {
+                if (gated) epilogue_own_gated(mode_tag);
+                else epilogue_own(mode_tag);
+            } else {
+                epilogue(mode_tag);
+            }
+        };
+        if (p.epilogue == GD_HIP_EPI_BIAS_F32) finish(std::integral_constant<uint32_t, GD_HIP_EPI_BIAS_F32>{});
+        else if (p.epilogue == GD_HIP_EPI_BIAS_F16) finish(std::integral_constant<uint32_t, GD_HIP_EPI_BIAS_F16>{});
+        else finish(std::integral_constant<uint32_t, GD_HIP_EPI_NONE>{});
     }
 }
 

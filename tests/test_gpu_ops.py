@@ -916,7 +916,8 @@ def test_many_row_projection_row_pitches_and_unaligned_output(backend, arena, or
 
 
 @pytest.mark.parametrize("M,K,H", [(64, 512, 1536), (16, 2048, 5632), (5, 136, 24), (33, 64, 40),
-                                   (1024, 512, 1536), (512, 256, 384), (300, 200, 200), (257, 128, 136)])
+                                   (1024, 512, 1536), (512, 256, 384), (300, 200, 200), (257, 128, 136),
+                                   (2304, 160, 4096), (2100, 96, 4100)])
 def test_fused_linear_swiglu_epilogue(backend, arena, oracle, gda, M, K, H):
     """rms_norm -> up/gate projection (+ F16 bias) -> swiglu_split in one launch equals the three separate operators."""
     x = oracle.normal_f16((M, K), 2600 + K, 1.3)
