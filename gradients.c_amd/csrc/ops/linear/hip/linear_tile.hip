@@ -49,6 +49,25 @@
 
 #define GD_TILE_BK 64u
 
+/* Profiling build (make TILE_TIMELINE=1): the first wavefront of every workgroup notes, for its first 32 tiles, the
+ * 100 MHz real-time counter at the start of the tile, after the K loop and after the epilogue, and the shader clock
+ * ticks the K loop took (their ratio is the clock the chip ran at).  gd_hip_linear_tile_timeline copies the notes of
+ * the last launch out; bench.py --probe tile_timeline prints them.  Not part of a normal build. */
+#ifdef GD_TILE_TIMELINE
+__device__ unsigned long long gd_tile_timeline[256 * 32 * 4];
+extern "C" __attribute__((visibility("default"))) int gd_hip_linear_tile_timeline(unsigned long long *host)
+{
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(gd_tile_timeline), sizeof(gd_tile_timeline));
+}
+#define GD_TILE_NOTE(slot, value)                                                                              \
+    do {                                                                                                        \
+        if (threadIdx.x == 0 && blockIdx.x < 256u && timeline_tile < 32u)                                       \
+            gd_tile_timeline[(blockIdx.x * 32u + timeline_tile) * 4u + (slot)] = (value);                       \
+    } while (0)
+#else
+#define GD_TILE_NOTE(slot, value) do { } while (0)
+#endif
+
 __device__ __forceinline__ uint32_t gd_tile_slot(uint32_t row, uint32_t c)
 {
     return row * 8u + (c ^ (row & 7u) ^ ((row >> 3) & 7u));
@@ -125,7 +144,15 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
 
     uint32_t tid_opaque = threadIdx.x;
     bool prefetched = false; /* the first two K tiles of the current output tile are already requested */
+#ifdef GD_TILE_TIMELINE
+    uint32_t timeline_tile = 0xffffffffu;
+#endif
     for (uint32_t tile = blockIdx.x; tile < total; tile += gridDim.x) {
+#ifdef GD_TILE_TIMELINE
+    ++timeline_tile;
+    const unsigned long long timeline_c0 = __builtin_amdgcn_s_memtime();
+    GD_TILE_NOTE(0, __builtin_amdgcn_s_memrealtime());
+#endif
     /* Everything below is derived from the thread id anew for every tile: were it loop-invariant, the
      * compiler would hoist some hundred addresses and offsets out of the tile loop and spill them. */
     asm volatile("" : "+v"(tid_opaque));
@@ -711,6 +738,10 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
             }
         }
 
+#ifdef GD_TILE_TIMELINE
+        GD_TILE_NOTE(1, __builtin_amdgcn_s_memrealtime());
+        GD_TILE_NOTE(3, __builtin_amdgcn_s_memtime() - timeline_c0);
+#endif
         auto finish = [&](auto mode_tag) __attribute__((always_inline)) {
             if (WM == 4 && WN == 4 && vector_store && m0 + BM <= p.M && n0 + out_bn <= p.N) {
                 if (gated) epilogue_own_gated(mode_tag);
@@ -722,6 +753,7 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
         if (p.epilogue == GD_HIP_EPI_BIAS_F32) finish(std::integral_constant<uint32_t, GD_HIP_EPI_BIAS_F32>{});
         else if (p.epilogue == GD_HIP_EPI_BIAS_F16) finish(std::integral_constant<uint32_t, GD_HIP_EPI_BIAS_F16>{});
         else finish(std::integral_constant<uint32_t, GD_HIP_EPI_NONE>{});
+        GD_TILE_NOTE(2, __builtin_amdgcn_s_memrealtime());
     }
 }
 

@@ -5,6 +5,9 @@ BASELINE.json configurations, timed with stream events around graph replays, one
     python bench.py --probe sdpa_decode        split-KV decode attention, caches rotating through HBM
     python bench.py --probe few_row_linear     decode-time projections of the scaled decoder, weights rotating through HBM
     python bench.py --probe tile_gemm          prefill projections on the matrix cores (also the program of the --pmc runs)
+    python bench.py --probe tile_timeline      the same projections in a profiling build of the library
+                                               (make -C gradients.c_amd/csrc TILE_TIMELINE=1): K loop and epilogue
+                                               time per tile and the clock the chip ran at
 
 Every probe reads more distinct bytes between two reads of the same byte than the 256 MB memory-side cache holds, so
 what it times comes from HBM.
@@ -186,4 +189,64 @@ def tile_gemm(pkg, launches=6):
                       "launches_per_shape": launches + 1, "results": results}))
 
 
-PROBES = {"sdpa_decode": sdpa_decode, "few_row_linear": few_row_linear, "tile_gemm": tile_gemm}
+def tile_timeline(pkg):
+    """Per-tile time stamps of the prefill projection kernel (library built with TILE_TIMELINE=1): for each shape of
+    tile_gemm and the up/gate + swiglu projection, microseconds in the K loop and in the epilogue per tile (mean over
+    the workgroups, first full rounds of tiles) and the shader clock during the K loop (s_memtime ticks per
+    nanosecond of the 100 MHz real-time counter)."""
+    import ctypes
+    lib = pkg.lib()
+    if not hasattr(lib, "gd_hip_linear_tile_timeline"):
+        raise SystemExit("this probe needs the profiling build: make -C gradients.c_amd/csrc TILE_TIMELINE=1")
+    be = pkg.Backend()
+    buf = be.buffer(3 << 30)
+    rng = np.random.default_rng(0)
+    timer = pkg.Timer(be)
+    results = []
+    for label, M, K, N, epi, res_on in (("qkv", 30229, 2048, 6144, 0, False),
+                                        ("attention projection + residual", 30229, 2048, 2048, 0, True),
+                                        ("up/gate + swiglu", 30229, 2048, 5632, 1, False),
+                                        ("down projection + residual", 30229, 5632, 2048, 0, True),
+                                        ("square", 8192, 8192, 8192, 0, False)):
+        buf.reset()
+        wrows = N * (2 if epi == 1 else 1)
+        x, w = buf.alloc((M, K), pkg.F16), buf.alloc((wrows, K), pkg.F16)
+        be.rand_uniform(x, 1, -1.0, 1.0)
+        be.rand_uniform(w, 2, -0.05, 0.05)
+        b = buf.from_numpy((rng.standard_normal(wrows) * 0.3).astype(np.float16))
+        r = buf.alloc((M, N), pkg.F16)
+        be.rand_uniform(r, 3, -1.0, 1.0)
+        y = buf.alloc((M, N), pkg.F16)
+        be.scope_begin()
+        call = lambda: be.fused_linear(x, w, b, r if res_on else None, None, y, True, 2, 0, 0.0, epi)
+        for _ in range(3):
+            call()
+        timer.start()
+        call()
+        timer.stop()
+        us = timer.elapsed_ms() * 1e3
+        be.fence_wait(be.record_fence())
+        notes = np.zeros(256 * 32 * 4, np.uint64)
+        rc = lib.gd_hip_linear_tile_timeline(notes.ctypes.data_as(ctypes.c_void_p))
+        if rc != 0:
+            raise SystemExit(f"gd_hip_linear_tile_timeline: {rc}")
+        notes = notes.reshape(256, 32, 4).astype(np.int64)
+        tiles = (M + 255) // 256 * ((wrows + 255) // 256)
+        rounds = min(32, tiles // 256)
+        k_loop = (notes[:, :rounds, 1] - notes[:, :rounds, 0]) / 100.0
+        epilogue = (notes[:, :rounds, 2] - notes[:, :rounds, 1]) / 100.0
+        clock = notes[:, :rounds, 3] / (k_loop * 1e3)
+        k_tiles = K // 64
+        results.append({"projection": label, "M": M, "K": K, "N": wrows, "launch_us": round(us, 1), "tiles": tiles,
+                        "full_rounds": rounds, "k_loop_us_per_tile": round(float(k_loop.mean()), 2),
+                        "epilogue_us_per_tile": round(float(epilogue.mean()), 2),
+                        "shader_clock_ghz_in_k_loop": round(float(clock.mean()), 3),
+                        "clocks_per_64_wide_k_tile": round(float((notes[:, :rounds, 3] / k_tiles).mean()), 0),
+                        "matrix_instruction_clocks_per_k_tile": 2048})
+    timer.close()
+    be.free(buf)
+    be.close()
+    print(json.dumps({"probe": "tile_timeline", "results": results}))
+
+
+PROBES = {"tile_timeline": tile_timeline, "sdpa_decode": sdpa_decode, "few_row_linear": few_row_linear, "tile_gemm": tile_gemm}
