@@ -19,6 +19,17 @@ static void launch_wide(hipStream_t stream, const void *x, const void *w, const 
         (const gd_half *)norm_w, (gd_half *)y, p, n_tiles, rope);
 }
 
+/* 8 columns per workgroup (narrow outputs, one row tile): see gd_linear_wide_half_kernel */
+template <int QMAX>
+static void launch_wide_half(hipStream_t stream, const void *x, const void *w, const void *bias, const void *residual,
+                             void *y, const gd_hip_linear_params &p)
+{
+    const uint32_t n_tiles = p.N / 8u;
+    dim3 grid(n_tiles, (p.M + 15u) / 16u);
+    gd_linear_wide_half_kernel<QMAX, 8><<<grid, 512, 0, stream>>>(
+        (const gd_half *)x, (const gd_half *)w, (const gd_half *)bias, (const gd_half *)residual, (gd_half *)y, p, n_tiles);
+}
+
 /* persistent form: K = 2048 behind an rms_norm, at most 8 tiles per workgroup, one workgroup per compute unit */
 template <int NT, int MT, int EPI>
 static void launch_persistent(hipStream_t stream, const void *x, const void *w, const void *bias, const void *residual,
@@ -44,7 +55,8 @@ static void launch_persistent(hipStream_t stream, const void *x, const void *w, 
  * not cover the call and the caller goes on to the stream kernel.  Covered: [N,K] weights of at least min_bytes
  * whose K is a multiple of 64 and splits over the eight wavefronts into at most 4 (behind an rms_norm) or 12 (no
  * prologue) pairs of steps each, fewer than 128 rows, and
- *   plain epilogue:   no prologue, 16 columns per workgroup; rms_norm prologue, 64 columns per workgroup;
+ *   plain epilogue:   no prologue, 16 columns per workgroup (8 where that leaves compute units without one);
+ *                     rms_norm prologue, 64 columns per workgroup;
  *   swiglu epilogue:  rms_norm prologue, 32 (tiles == 2) or 64 weight rows per workgroup;
  *   rope epilogue:    rms_norm prologue, 32 weight rows per workgroup (head size a multiple of 32). */
 extern "C" int gd_hip_try_launch_linear_wide(hipStream_t stream, const void *x, const void *w, const void *bias,
@@ -71,6 +83,13 @@ extern "C" int gd_hip_try_launch_linear_wide(hipStream_t stream, const void *x, 
         /* 16 columns per workgroup: these are the narrow outputs (N = d_model), where further row tiles are worth
          * more as workgroups of their own (16 x 2048 x 2048 and 32 x ...: 6.0 us with one row tile per workgroup,
          * 8.2 us with both in one; the second reader of a weight line finds it in L2) */
+        /* up to 16 rows and fewer 16-column tiles than compute units: 8 columns per workgroup, so that every unit
+         * streams (16 x 5632 -> 2048: 256 workgroups instead of 128) */
+        if (p.M <= 16u && p.N / 16u < units && tiles != 1u && (p.K % 128u) == 0u && (p.N % 8u) == 0u) {
+            const uint32_t qpw = (p.K / 128u + 7u) / 8u; /* pieces of 128 per wavefront */
+            if (qpw <= 2u) { launch_wide_half<2>(stream, x, w, bias, residual, y, p); return 1; }
+            if (qpw <= 6u) { launch_wide_half<6>(stream, x, w, bias, residual, y, p); return 1; }
+        }
         if (ppw <= 4u) GD_W(1, 1, 4, GD_HIP_PRO_NONE, GD_WIDE_EPI_PLAIN);
         if (ppw <= 12u) GD_W(1, 1, 12, GD_HIP_PRO_NONE, GD_WIDE_EPI_PLAIN);
         return 0;

@@ -305,6 +305,138 @@ gd_linear_wide_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
 }
 
 /*
+ * The plain projection (no prologue; bias, optional residual) for outputs so NARROW that 16 columns per workgroup
+ * leave compute units without one (N = 2048: 128 workgroups on 256 units): 8 columns per workgroup.  A weight group
+ * is still 2 KB in two instructions of 8 rows x 128 bytes, but both cover the same 8 weight rows, at consecutive
+ * 64-wide pieces of K; the matrix instruction takes weight row l % 8 in lanes l % 16 = 0..7 and again in 8..15, so
+ * its output columns 8..15 repeat 0..7 and are dropped (the matrix cores have time to spare: the kernel is bound by
+ * the weight stream).  One row tile of 16 per workgroup (blockIdx.y walks further ones), a wavefront's K range is
+ * at most QMAX pieces of 128.  Host guarantees: K % 128 == 0, ceil(K / 128 / 8) <= QMAX, N % 8 == 0, byte offsets
+ * below 2^31, 16-byte aligned rows.
+ */
+template <int QMAX, int RING>
+__global__ void __launch_bounds__(512)
+gd_linear_wide_half_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__ w, const gd_half *__restrict__ bias,
+                           const gd_half *__restrict__ residual, gd_half *__restrict__ y, gd_hip_linear_params p,
+                           uint32_t n_tiles)
+{
+    constexpr int WAVES = 8;
+    constexpr int SMAX = 4 * QMAX; /* K steps of 32 per wavefront */
+    static_assert(RING >= 2 && RING <= 8, "ring depth");
+    constexpr int RING_BYTES = WAVES * RING * 2048, SUM_BYTES = WAVES * 1024;
+    __shared__ __align__(16) unsigned char s_mem[RING_BYTES > SUM_BYTES ? RING_BYTES : SUM_BYTES];
+
+    asm volatile("" ::"s"(x), "s"(w), "s"(bias), "s"(residual), "s"(y), "s"(p.M), "s"(p.N), "s"(p.K), "s"(p.ldx),
+                 "s"(p.ldw), "s"(p.ldy), "s"(p.epilogue), "s"(p.has_residual), "s"(p.ldr), "s"(n_tiles));
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int li = lane & 15, lg = lane >> 4;
+    uint32_t tile = blockIdx.x;
+    if ((n_tiles & 7u) == 0u) tile = (blockIdx.x & 7u) * (n_tiles >> 3) + (blockIdx.x >> 3);
+    const uint32_t n0 = tile * 8u, m0 = blockIdx.y * 16u;
+
+    /* what the epilogue will need, requested first: thread t < 128 owns output (row 4*(t/32) + (t/8)%4, column t%8) */
+    const uint32_t e_col = n0 + (threadIdx.x & 7u), e_row = m0 + 4u * (threadIdx.x >> 5) + ((threadIdx.x >> 3) & 3u);
+    gd_half pf_b = (gd_half)0.f, pf_res = (gd_half)0.f;
+    if (threadIdx.x < 128u) {
+        if (p.epilogue != GD_HIP_EPI_NONE) pf_b = bias[e_col];
+        if (p.has_residual) pf_res = residual[(size_t)min(e_row, p.M - 1u) * p.ldr + e_col];
+    }
+
+    /* the wavefront's K range in pieces of 128: the first kq % 8 wavefronts take one piece more */
+    const uint32_t kq = p.K / 128u, base = kq / WAVES, rem = kq % WAVES;
+    const uint32_t q_begin = (uint32_t)wave * base + min((uint32_t)wave, rem);
+    const int nq = (int)(base + ((uint32_t)wave < rem ? 1u : 0u)); /* 0..QMAX: groups of this wavefront */
+    const unsigned char *wb = reinterpret_cast<const unsigned char *>(w) + (size_t)q_begin * 256u;
+    const unsigned char *xb = reinterpret_cast<const unsigned char *>(x) + (size_t)q_begin * 256u;
+    const gd_half8 zero8 = (gd_half8)(gd_half)0.f;
+
+    /* lane's 16 bytes of an instruction: weight row n0 + lane/8, chunk (lane%8 ^ lane/8) of the 128-byte piece */
+    const uint32_t goff = ((n0 + (uint32_t)lane / 8u) * p.ldw + ((((uint32_t)lane % 8u) ^ ((uint32_t)lane / 8u)) * 8u)) * 2u;
+    const uint32_t ring_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)s_mem +
+                               (uint32_t)wave * (RING * 2048u);
+    auto issue_group = [&](int g) __attribute__((always_inline)) {
+        const uint32_t slot = ring_base + (uint32_t)(g % RING) * 2048u;
+        const uint64_t sp = (uint64_t)(uintptr_t)(wb + (size_t)g * 256u);
+        const unsigned char *src = reinterpret_cast<const unsigned char *>(
+            ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(sp >> 32)) << 32) |
+            (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)sp));
+        gd_lin_load_lds16(src, goff, slot);
+        gd_lin_load_lds16(src + 128, goff, slot + 1024u);
+    };
+#pragma unroll
+    for (int g = 0; g < RING && g < QMAX; ++g) {
+        if (g < nq) issue_group(g);
+    }
+
+    /* the activation slice of the wavefront, resident */
+    gd_half8 ar[SMAX];
+    {
+        const uint32_t mrow = min(m0 + (uint32_t)li, p.M - 1u);
+        const uint32_t xoff = (mrow * p.ldx + (uint32_t)lg * 8u) * 2u;
+#pragma unroll
+        for (int s = 0; s < SMAX; ++s) {
+            ar[s] = zero8;
+            if (s < 4 * nq) ar[s] = *reinterpret_cast<const gd_half8 *>(xb + (size_t)s * 64u + xoff);
+        }
+    }
+
+    /* the stream: group g is read from its slot while the matrix instructions of group g-1 run; the slot of g-1 is
+     * refilled behind them */
+    gd_float4 acc = (gd_float4){0.f, 0.f, 0.f, 0.f};
+    {
+        const uint32_t li8 = (uint32_t)li % 8u;
+        const uint32_t rd0 = (li8 * 8u + ((uint32_t)lg ^ li8)) * 16u;
+        const uint32_t rd1 = (li8 * 8u + ((4u + (uint32_t)lg) ^ li8)) * 16u;
+        const unsigned char *ring = &s_mem[0] + (size_t)wave * (RING * 2048);
+        gd_half8 f[4] = {zero8, zero8, zero8, zero8}, pf[4] = {zero8, zero8, zero8, zero8};
+#pragma unroll
+        for (int g = 0; g <= QMAX; ++g) {
+            if (g < QMAX && g < nq) {
+                const int issued = g < 2 ? RING - 1 : g - 2 + RING;
+                const int last = issued < nq - 1 ? issued : nq - 1;
+                gd_wide_wait_groups(last - g);
+                const unsigned char *slot = ring + (g % RING) * 2048;
+                f[0] = *reinterpret_cast<const gd_half8 *>(slot + rd0);
+                f[1] = *reinterpret_cast<const gd_half8 *>(slot + rd1);
+                f[2] = *reinterpret_cast<const gd_half8 *>(slot + 1024 + rd0);
+                f[3] = *reinterpret_cast<const gd_half8 *>(slot + 1024 + rd1);
+            }
+            if (g >= 1 && g - 1 < nq) {
+                const int q = g - 1;
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ar[4 * q + t], pf[t], acc, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (q + RING < QMAX && q + RING < nq) issue_group(q + RING);
+            }
+#pragma unroll
+            for (int t = 0; t < 4; ++t) pf[t] = f[t];
+        }
+    }
+
+    /* sum of the wavefronts through LDS (the ring's memory: every wavefront is done reading it) */
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    float *sm = reinterpret_cast<float *>(&s_mem[0]);
+    if (li < 8) *reinterpret_cast<gd_float4 *>(sm + ((wave * 4 + lg) * 8 + li) * 4) = acc;
+    __syncthreads();
+    if (threadIdx.x < 128u) {
+        /* lane (li, lg) of the matrix instruction holds column li, rows 4*lg + 0..3 */
+        const int c = threadIdx.x & 7, r = (threadIdx.x >> 3) & 3, g4 = threadIdx.x >> 5;
+        float v = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < WAVES; ++wv) v += sm[((wv * 4 + g4) * 8 + c) * 4 + r];
+        if (e_row < p.M) {
+            gd_half h;
+            if (p.epilogue == GD_HIP_EPI_BIAS_F32) h = (gd_half)(v + (float)pf_b);
+            else if (p.epilogue == GD_HIP_EPI_BIAS_F16) h = (gd_half)v + pf_b;
+            else h = (gd_half)v;
+            if (p.has_residual) h = pf_res + h;
+            y[(size_t)e_row * p.ldy + e_col] = h;
+        }
+    }
+}
+
+/*
  * The same projection for matrices with MANY column tiles (rms_norm prologue, K = 512 * PMAX: every wavefront owns
  * exactly PMAX pairs of steps): persistent workgroups.  gridDim.x workgroups share the n_tiles column tiles in
  * contiguous runs; a workgroup loads and normalises its activation slice ONCE and then walks its tiles with the

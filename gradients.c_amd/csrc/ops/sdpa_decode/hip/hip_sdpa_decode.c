@@ -84,7 +84,7 @@ static gd_status dispatch(gd_backend *backend, const gd_backend_tensor_view *q, 
     else p.nontemporal = (uint64_t)p.batch * p.tmax * p.hkv * p.dh * 4u > (128ull << 20) ? 1u : 0u;
     group = p.hq / p.hkv;
     if (q->dtype == GD_BACKEND_DTYPE_F16 && p.tq == 1u && (p.dh == 64u || p.dh == 128u) &&
-        (group == 1u || group == 2u || group == 4u || group == 8u) &&
+        (group == 1u || group == 2u || group == 3u || group == 4u || group == 6u || group == 8u) &&
         ((q->offset | k->offset | v->offset | out->offset) & 15u) == 0u && p.batch <= 65535u &&
         /* the kernel addresses the rows of one (batch row, kv head) with 24-bit factors and 32-bit byte offsets */
         p.tmax < (1u << 24) && (uint64_t)p.hkv * p.dh * 2u < (1u << 24) &&
@@ -102,7 +102,7 @@ static gd_status dispatch(gd_backend *backend, const gd_backend_tensor_view *q, 
          * 2048 wavefronts each walking its own stretch of a [T, Hkv, D] cache touch far more DRAM pages at a time
          * than 256 workgroups whose wavefronts read neighbouring rows. */
         if (pos_mode == GD_HIP_SDPA_POS_VECTOR && p.prefix_len == 0u && backend->sdpa_chunk == 0 &&
-            backend->sdpa_balanced > 0 && (uint64_t)p.batch * p.hkv * p.tmax < 0x7fffffffull) {
+            backend->sdpa_balanced > 0 && (group & (group - 1u)) == 0u && (uint64_t)p.batch * p.hkv * p.tmax < 0x7fffffffull) {
             /* a share is what one wavefront streams: 8 (or 16) wavefronts per compute unit */
             const uint32_t shares = (uint32_t)backend->compute_units * (backend->sdpa_balanced > 1 ? 16u : 8u);
             const size_t need = ((size_t)p.batch * p.hkv + shares) * group * (p.dh + 4u) * sizeof(float);

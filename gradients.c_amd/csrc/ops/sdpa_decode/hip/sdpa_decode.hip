@@ -421,8 +421,8 @@ extern "C" int gd_hip_launch_sdpa_decode_split(hipStream_t stream, const void *q
     const gd_hip_sdpa_decode_params &p = *params;
     const uint32_t g = p.hq / p.hkv;
 #define GD_CASE(DD, GG) if (p.dh == DD && g == GG) return launch_split<DD, GG>(stream, q, k, v, pos, out, ws, p)
-    GD_CASE(64, 1); GD_CASE(64, 2); GD_CASE(64, 4); GD_CASE(64, 8);
-    GD_CASE(128, 1); GD_CASE(128, 2); GD_CASE(128, 4); GD_CASE(128, 8);
+    GD_CASE(64, 1); GD_CASE(64, 2); GD_CASE(64, 3); GD_CASE(64, 4); GD_CASE(64, 6); GD_CASE(64, 8);
+    GD_CASE(128, 1); GD_CASE(128, 2); GD_CASE(128, 3); GD_CASE(128, 4); GD_CASE(128, 6); GD_CASE(128, 8);
 #undef GD_CASE
     return (int)hipErrorInvalidValue;
 }

@@ -359,7 +359,9 @@ def test_decode_full_size_long_context_sampled(backend, oracle):
         backend.free(big)
 
 
-@pytest.mark.parametrize("H,Hkv,D", [(8, 8, 64), (16, 16, 128), (8, 2, 64), (8, 1, 128), (6, 3, 64), (6, 2, 64)])
+# query heads per kv head: 1, 4, 8, 2, 3, 6 (the split-KV kernel) and 5 (the generic kernel)
+@pytest.mark.parametrize("H,Hkv,D", [(8, 8, 64), (16, 16, 128), (8, 2, 64), (8, 1, 128), (6, 3, 64), (6, 2, 64),
+                                     (12, 2, 128), (6, 1, 64), (10, 2, 64)])
 def test_decode_head_layouts(backend, arena, oracle, H, Hkv, D):
     pos = np.array([0, 1, 63, 64, 200, 299, -1, 31], np.int32)
     _decode_case(backend, arena, oracle, 8, H, Hkv, D, 300, pos, 1.0 / np.sqrt(D), seed=200 + H + D, chunk=96)
@@ -978,6 +980,35 @@ def test_few_row_projection_over_weights_on_both_sides_of_a_2_gib_boundary(backe
     finally:
         backend.set_tunable("linear_wide", -1)
         backend.free(big)
+
+
+@pytest.mark.parametrize("M,K,N", [(16, 2048, 2048), (16, 5632, 2048), (5, 1152, 1024), (1, 384, 264), (16, 128, 2048)])
+def test_few_row_projection_onto_narrow_outputs(backend, arena, oracle, gda, M, K, N):
+    """Up to 16 rows onto an output with fewer 16-column tiles than the chip has compute units: 8 columns per workgroup
+    (K in pieces of 128 dealt to the eight wavefronts: 16, 44, 9, 3 and 1 pieces here, so wavefronts with one piece more
+    than others and wavefronts with none).  All bias modes, with and without the residual, against the oracle; the
+    16-column form (tunable linear_tiles = 1) must meet the same bar."""
+    x = oracle.normal_f16((M, K), 3300 + K, 1.0)
+    w = oracle.normal_f16((N, K), 3301 + N, 0.05)
+    bias = oracle.normal_f16((N,), 3302, 0.5)
+    res = oracle.normal_f16((M, N), 3303, 1.0)
+    y = arena.alloc((M, N), gda.F16)
+    tx, tw, tb, tr = (arena.from_numpy(a) for a in (x, w, bias, res))
+    try:
+        backend.set_tunable("linear_wide", 1)
+        for tiles in (0, 1):
+            backend.set_tunable("linear_tiles", tiles)
+            backend.fill(y, 0x7e00)
+            backend.fused_linear(tx, tw, None, None, None, y, True, 0, 0)
+            _close(y.read(), oracle.linear_nt(x, w))
+            backend.fused_linear(tx, tw, tb, None, None, y, True, 1, 0)
+            _close(y.read(), oracle.linear(x, np.ascontiguousarray(w.T), bias))
+            backend.fused_linear(tx, tw, tb, tr, None, y, True, 2, 0)
+            inter = oracle.linear_nt(x, w, bias)
+            _close(y.read(), oracle.add(res, inter), through=inter)
+    finally:
+        backend.set_tunable("linear_wide", -1)
+        backend.set_tunable("linear_tiles", 0)
 
 
 @pytest.mark.parametrize("M,N,gated", [(16, 5632, True), (33, 8200, False), (64, 4096, True), (5, 32768, False)])
