@@ -13,7 +13,11 @@
  *     compute unit has 8 x (RING - 1) x 2 KB of weights in flight without spending registers on them;
  *   - the activation slice of a wavefront (its K range of all MT row tiles) is loaded once, up front, into
  *     registers, and the operands the epilogue needs (bias, residual, positions) are requested before
- *     anything else, so no dependent round trip is left behind the stream;
+ *     anything else, so no dependent round trip is left behind the stream; the slice is requested in front of
+ *     the ring with loads the kernel counts itself (gd_wide_request16), because a wait placed by the compiler
+ *     would also wait for the ring: the row sums of the rms_norm and the first matrix instructions then run
+ *     while the first weight groups are still on their way (measured per phase with time stamps: the slice
+ *     usable 3.4 instead of 5.7 us after entry at 16 x 2048 -> 6144);
  *   - the eight wavefronts of a workgroup split K and are summed through LDS (the ring's memory, reused).
  *
  * Reference semantics: src/ops/_shared/gemm/metal_gemm_common.h:161-237 (NT GEMM) with the separate bias add of
@@ -28,10 +32,47 @@
 #define GD_WIDE_EPI_SWIGLU 1 /* value / gate column pairs: y = half(value) * silu(half(gate)) */
 #define GD_WIDE_EPI_ROPE 2   /* qkv of a decode step: rotation pairs, q stored, k / v appended to the caches */
 
-/* waits until at most 2 * later of the wavefront's vector-memory loads are outstanding (later uniform, 0..7) */
+/* Register loads the kernel counts itself.  The compiler does not see the global -> LDS loads of the ring, so a wait
+ * it places for a load of its own is a wait for everything outstanding, the ring included: a wavefront would start
+ * on its activation slice only when all of its first weight groups had crossed the chip.  Loads requested this way,
+ * in front of the ring, are waited for with gd_wide_wait_groups (loads return in order: once only the ring's
+ * instructions are outstanding, everything older has arrived); gd_wide_arrived then hands the registers to the
+ * compiler, which must not touch them before. */
+__device__ __forceinline__ gd_half8 gd_wide_request16(const unsigned char *uniform_base, uint32_t lane_byte_offset)
+{
+    gd_half8 v;
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(v) : "v"(lane_byte_offset), "s"(uniform_base) : "memory");
+    return v;
+}
+__device__ __forceinline__ uint32_t gd_wide_request2(const void *uniform_base, uint32_t lane_byte_offset)
+{
+    uint32_t v;
+    asm volatile("global_load_ushort %0, %1, %2" : "=v"(v) : "v"(lane_byte_offset), "s"(uniform_base) : "memory");
+    return v;
+}
+__device__ __forceinline__ uint32_t gd_wide_request4(const void *uniform_base, uint32_t lane_byte_offset)
+{
+    uint32_t v;
+    asm volatile("global_load_dword %0, %1, %2" : "=v"(v) : "v"(lane_byte_offset), "s"(uniform_base) : "memory");
+    return v;
+}
+template <typename T>
+__device__ __forceinline__ void gd_wide_arrived(T &v)
+{
+    asm volatile("" : "+v"(v) : : "memory");
+}
+__device__ __forceinline__ gd_half gd_wide_half_of(uint32_t bits)
+{
+    union { unsigned short u; gd_half h; } c;
+    c.u = (unsigned short)bits;
+    return c.h;
+}
+
+/* waits until at most 2 * later of the wavefront's vector-memory loads are outstanding (later uniform, 0..8) */
 __device__ __forceinline__ void gd_wide_wait_groups(int later)
 {
     switch (later) {
+    case 8: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
     case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
     case 1: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
     case 2: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
@@ -114,12 +155,11 @@ gd_linear_wide_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
     const int np = (int)(min(p_begin + per_wave, kpairs) - p_begin); /* 0..PMAX */
     const int ng = np * NT;
     const unsigned char *wb = reinterpret_cast<const unsigned char *>(w) + (size_t)p_begin * 128u;
-    const unsigned char *xb = reinterpret_cast<const unsigned char *>(x) + (size_t)p_begin * 128u;
-    const unsigned char *nb = reinterpret_cast<const unsigned char *>(norm_w) + (size_t)p_begin * 128u;
+    /* (a wavefront without a K range requests the first step of the row instead of one past its end) */
+    const unsigned char *xb = reinterpret_cast<const unsigned char *>(x) + (size_t)(np > 0 ? p_begin : 0u) * 128u;
+    const unsigned char *nb = reinterpret_cast<const unsigned char *>(norm_w) + (size_t)(np > 0 ? p_begin : 0u) * 128u;
     const gd_half8 zero8 = (gd_half8)(gd_half)0.f;
-    /* ---- 3. the weight stream: group g = pair * NT + j, two instructions of 8 rows x 128 bytes.  The first RING
-     *         groups are requested before the activation slice: the stream starts one round trip earlier, and the
-     *         slice, which comes from L2, is there long before the first group has crossed the chip ---- */
+    /* ---- 3. the weight stream: group g = pair * NT + j, two instructions of 8 rows x 128 bytes ---- */
     uint32_t goff[NT][2]; /* bytes from the pair's base to the lane's 16 bytes: row 8*half + lane/8, swizzled chunk */
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
@@ -140,28 +180,43 @@ gd_linear_wide_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
         gd_lin_load_lds16(src, goff[j][0], slot);
         gd_lin_load_lds16(src, goff[j][1], slot + 1024u);
     };
-#pragma unroll
-    for (int g = 0; g < RING && g < NGMAX; ++g) {
-        if (g < ng) issue_group(g);
-    }
-
-    /* ---- 3b. the activation slice of the wavefront (and the norm weights of its K range), resident ---- */
+    /* ---- 3a. the activation slice of the wavefront (and the norm weights of its K range), resident: requested in
+     *          front of the ring and counted by hand, so that it is usable while the ring is still on its way.  Steps
+     *          past the wavefront's range re-read its first one (never multiplied with a landed weight group, but the
+     *          row sums of the rms_norm must not see them: zeroed after arrival) ---- */
     gd_half8 ar[MT][SMAX], nr[PRO == GD_HIP_PRO_RMS_NORM ? SMAX : 1];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const uint32_t mrow = min(m0 + 16u * mt + (uint32_t)li, p.M - 1u);
         const uint32_t xoff = (mrow * p.ldx + (uint32_t)lg * 8u) * 2u;
 #pragma unroll
-        for (int s = 0; s < SMAX; ++s) {
-            ar[mt][s] = zero8;
-            if (s < 2 * np) ar[mt][s] = *reinterpret_cast<const gd_half8 *>(xb + (size_t)s * 64u + xoff);
-        }
+        for (int s = 0; s < SMAX; ++s) ar[mt][s] = gd_wide_request16(xb, (s < 2 * np ? (uint32_t)s * 64u : 0u) + xoff);
     }
     if (PRO == GD_HIP_PRO_RMS_NORM) {
 #pragma unroll
+        for (int s = 0; s < SMAX; ++s) nr[s] = gd_wide_request16(nb, (s < 2 * np ? (uint32_t)s * 64u : 0u) + (uint32_t)lg * 16u);
+    }
+    int first_groups = 0;
+#pragma unroll
+    for (int g = 0; g < RING && g < NGMAX; ++g) {
+        if (g < ng) {
+            issue_group(g);
+            first_groups = g + 1;
+        }
+    }
+    gd_wide_wait_groups(first_groups);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
         for (int s = 0; s < SMAX; ++s) {
-            nr[s] = zero8;
-            if (s < 2 * np) nr[s] = *reinterpret_cast<const gd_half8 *>(nb + (size_t)s * 64u + (uint32_t)lg * 16u);
+            gd_wide_arrived(ar[mt][s]);
+            if (s >= 2 * np) ar[mt][s] = zero8;
+        }
+    if (PRO == GD_HIP_PRO_RMS_NORM) {
+#pragma unroll
+        for (int s = 0; s < SMAX; ++s) {
+            gd_wide_arrived(nr[s]);
+            if (s >= 2 * np) nr[s] = zero8;
         }
     }
 
@@ -347,7 +402,8 @@ gd_linear_wide_half_kernel(const gd_half *__restrict__ x, const gd_half *__restr
     const uint32_t q_begin = (uint32_t)wave * base + min((uint32_t)wave, rem);
     const int nq = (int)(base + ((uint32_t)wave < rem ? 1u : 0u)); /* 0..QMAX: groups of this wavefront */
     const unsigned char *wb = reinterpret_cast<const unsigned char *>(w) + (size_t)q_begin * 256u;
-    const unsigned char *xb = reinterpret_cast<const unsigned char *>(x) + (size_t)q_begin * 256u;
+    /* (a wavefront without a K range requests the first piece of the row instead of one past its end) */
+    const unsigned char *xb = reinterpret_cast<const unsigned char *>(x) + (size_t)(nq > 0 ? q_begin : 0u) * 256u;
     const gd_half8 zero8 = (gd_half8)(gd_half)0.f;
 
     /* lane's 16 bytes of an instruction: weight row n0 + lane/8, chunk (lane%8 ^ lane/8) of the 128-byte piece */
@@ -363,22 +419,26 @@ gd_linear_wide_half_kernel(const gd_half *__restrict__ x, const gd_half *__restr
         gd_lin_load_lds16(src, goff, slot);
         gd_lin_load_lds16(src + 128, goff, slot + 1024u);
     };
-#pragma unroll
-    for (int g = 0; g < RING && g < QMAX; ++g) {
-        if (g < nq) issue_group(g);
-    }
-
-    /* the activation slice of the wavefront, resident */
+    /* the activation slice of the wavefront, resident: requested in front of the ring and counted by hand (see
+     * gd_wide_request16), so that the first weight group can be multiplied as soon as it lands */
     gd_half8 ar[SMAX];
     {
         const uint32_t mrow = min(m0 + (uint32_t)li, p.M - 1u);
         const uint32_t xoff = (mrow * p.ldx + (uint32_t)lg * 8u) * 2u;
 #pragma unroll
-        for (int s = 0; s < SMAX; ++s) {
-            ar[s] = zero8;
-            if (s < 4 * nq) ar[s] = *reinterpret_cast<const gd_half8 *>(xb + (size_t)s * 64u + xoff);
+        for (int s = 0; s < SMAX; ++s) ar[s] = gd_wide_request16(xb, (s < 4 * nq ? (uint32_t)s * 64u : 0u) + xoff);
+    }
+    int first_groups = 0;
+#pragma unroll
+    for (int g = 0; g < RING && g < QMAX; ++g) {
+        if (g < nq) {
+            issue_group(g);
+            first_groups = g + 1;
         }
     }
+    gd_wide_wait_groups(first_groups);
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s) gd_wide_arrived(ar[s]);
 
     /* the stream: group g is read from its slot while the matrix instructions of group g-1 run; the slot of g-1 is
      * refilled behind them */
@@ -511,24 +571,23 @@ gd_linear_wide_persistent_kernel(const gd_half *__restrict__ x, const gd_half *_
         gd_lin_load_lds16(src, (nbase + lrow[0]) * p.ldw * 2u + lchunk, a);
         gd_lin_load_lds16(src, (nbase + lrow[1]) * p.ldw * 2u + lchunk, a + 1024u);
     };
-#pragma unroll
-    for (int g = 0; g < RING; ++g) {
-        if (g < total_groups) issue_group(g, g);
+    /* ---- requested in front of the ring and counted by hand (gd_wide_request16): the bias values and positions of
+     *      all tiles of this workgroup (TPW * OUT_COLS <= 512: at most one column per thread) and the activation
+     *      slice with its norm weights.  They are usable while the ring's first groups are still crossing the chip,
+     *      so the row sums, their barrier and the scaling pass behind the weight stream, not in front of it ---- */
+    static_assert(TPW * OUT_COLS <= 512, "one bias column per thread");
+    uint32_t rq_b1 = 0u, rq_b2 = 0u, rq_pos = 0u, rq_cpos = 0u;
+    const bool has_col = (int)threadIdx.x < tiles * (int)OUT_COLS;
+    const uint32_t b_col = tile_n0(t_begin + (has_col ? threadIdx.x / OUT_COLS : 0u)) + threadIdx.x % OUT_COLS;
+    if (p.epilogue != GD_HIP_EPI_NONE) {
+        rq_b1 = gd_wide_request2(bias, b_col * 2u);
+        if (PAIRED) rq_b2 = gd_wide_request2(bias, (pair_offset + b_col) * 2u);
     }
-
-    /* ---- bias values and positions of all tiles of this workgroup into LDS ---- */
-    for (int i = (int)threadIdx.x; i < tiles * (int)OUT_COLS; i += 512) {
-        const uint32_t col = tile_n0(t_begin + (uint32_t)i / OUT_COLS) + (uint32_t)i % OUT_COLS;
-        s_bias[0][i] = p.epilogue != GD_HIP_EPI_NONE ? bias[col] : (gd_half)0.f;
-        s_bias[1][i] = (PAIRED && p.epilogue != GD_HIP_EPI_NONE) ? bias[pair_offset + col] : (gd_half)0.f;
+    if (EPI == GD_WIDE_EPI_ROPE) {
+        const uint32_t row = min(m0 + (threadIdx.x & (16u * MT - 1u)), p.M - 1u);
+        rq_pos = gd_wide_request4(rope.rope_pos, row * 4u);
+        rq_cpos = gd_wide_request4(rope.cache_pos, row * 4u);
     }
-    if (EPI == GD_WIDE_EPI_ROPE && threadIdx.x < 16u * MT) {
-        const uint32_t row = min(m0 + threadIdx.x, p.M - 1u);
-        s_pos[0][threadIdx.x] = rope.rope_pos[row];
-        s_pos[1][threadIdx.x] = rope.cache_pos[row];
-    }
-
-    /* ---- the activation slice, resident and normalised once ---- */
     const unsigned char *xb = reinterpret_cast<const unsigned char *>(x) + (size_t)p_begin * 128u;
     const unsigned char *nb = reinterpret_cast<const unsigned char *>(norm_w) + (size_t)p_begin * 128u;
     gd_half8 ar[MT][SMAX];
@@ -539,10 +598,37 @@ gd_linear_wide_persistent_kernel(const gd_half *__restrict__ x, const gd_half *_
             const uint32_t mrow = min(m0 + 16u * mt + (uint32_t)li, p.M - 1u);
             const uint32_t xoff = (mrow * p.ldx + (uint32_t)lg * 8u) * 2u;
 #pragma unroll
-            for (int s = 0; s < SMAX; ++s) ar[mt][s] = *reinterpret_cast<const gd_half8 *>(xb + (size_t)s * 64u + xoff);
+            for (int s = 0; s < SMAX; ++s) ar[mt][s] = gd_wide_request16(xb, (uint32_t)s * 64u + xoff);
         }
 #pragma unroll
-        for (int s = 0; s < SMAX; ++s) nr[s] = *reinterpret_cast<const gd_half8 *>(nb + (size_t)s * 64u + (uint32_t)lg * 16u);
+        for (int s = 0; s < SMAX; ++s) nr[s] = gd_wide_request16(nb, (uint32_t)s * 64u + (uint32_t)lg * 16u);
+    int first_groups = 0;
+#pragma unroll
+        for (int g = 0; g < RING; ++g) {
+            if (g < total_groups) {
+                issue_group(g, g);
+                first_groups = g + 1;
+            }
+        }
+        gd_wide_wait_groups(first_groups);
+        gd_wide_arrived(rq_b1);
+        gd_wide_arrived(rq_b2);
+        gd_wide_arrived(rq_pos);
+        gd_wide_arrived(rq_cpos);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int s = 0; s < SMAX; ++s) gd_wide_arrived(ar[mt][s]);
+#pragma unroll
+        for (int s = 0; s < SMAX; ++s) gd_wide_arrived(nr[s]);
+        if (has_col) {
+            s_bias[0][threadIdx.x] = gd_wide_half_of(rq_b1);
+            s_bias[1][threadIdx.x] = gd_wide_half_of(rq_b2);
+        }
+        if (EPI == GD_WIDE_EPI_ROPE && threadIdx.x < 16u * MT) {
+            s_pos[0][threadIdx.x] = (int32_t)rq_pos;
+            s_pos[1][threadIdx.x] = (int32_t)rq_cpos;
+        }
         float ss[MT];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
