@@ -516,7 +516,7 @@ def main():
     ap.add_argument("--minimax-kernels", action="store_true",
                     help="time the MiniMax-M3 block picker and block-sparse attention next to dense causal attention on "
                          "packed sequences (auxiliary: prints its own JSON line, not the headline metric)")
-    ap.add_argument("--probe", choices=("sdpa_decode", "sdpa_decode_balanced", "few_row_linear", "tile_gemm", "tile_timeline"),
+    ap.add_argument("--probe", choices=("sdpa_decode", "sdpa_decode_balanced", "few_row_linear", "tile_gemm", "tile_timeline", "prefill_attention"),
                     help="operator-local performance probe (gradients.c_amd/perf_probes.py): one operator at the shapes of "
                          "the BASELINE.json configurations, operands rotating through HBM; prints its own JSON line. "
                          "sdpa_decode_balanced also times the form that deals the keys to the wavefronts by count")

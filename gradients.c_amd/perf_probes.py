@@ -5,6 +5,8 @@ BASELINE.json configurations, timed with stream events around graph replays, one
     python bench.py --probe sdpa_decode        split-KV decode attention, caches rotating through HBM
     python bench.py --probe few_row_linear     decode-time projections of the scaled decoder, weights rotating through HBM
     python bench.py --probe tile_gemm          prefill projections on the matrix cores (also the program of the --pmc runs)
+    python bench.py --probe prefill_attention  packed causal attention of the prefill (gd_backend_sdpa_varlen) at the
+                                               prompt mixes of configs[3] and [4] and at equal lengths
     python bench.py --probe tile_timeline      the same projections in a profiling build of the library
                                                (make -C gradients.c_amd/csrc TILE_TIMELINE=1): K loop and epilogue
                                                time per tile and the clock the chip ran at
@@ -189,6 +191,50 @@ def tile_gemm(pkg, launches=6):
                       "launches_per_shape": launches + 1, "results": results}))
 
 
+def prefill_attention(pkg, launches=5):
+    """gd_backend_sdpa_varlen (packed causal attention, 16 heads of 128, F16) over the prompt mixes of configs[3]
+    (16 prompts of 1024..4095 tokens) and configs[4] (32 prompts of 64..2048 tokens), at equal lengths, and with 8
+    heads of 64 (64 prompts of 511 tokens: the prefill of configs[2]).  Flops are counted on the visible
+    (query, key) pairs only: 4 * D per pair and head."""
+    be = pkg.Backend()
+    buf = be.buffer(3 << 30)
+    timer = pkg.Timer(be)
+    results = []
+    rng = np.random.default_rng(1004)
+    for label, H, D, lens in (("configs[3] prompts: 16 x 1024..4095", 16, 128, rng.integers(1024, 4096, 16)),
+                              ("configs[4] prompts: 32 x 64..2048", 16, 128, rng.integers(64, 2049, 32)),
+                              ("16 x 2560 (equal lengths)", 16, 128, np.full(16, 2560)),
+                              ("4 x 8192 (equal lengths)", 16, 128, np.full(4, 8192)),
+                              ("configs[2] prompts: 64 x 511, 8 heads of 64", 8, 64, np.full(64, 511))):
+        buf.reset()
+        n = int(lens.sum())
+        cu = np.zeros(len(lens) + 1, np.int32)
+        cu[1:] = np.cumsum(lens)
+        q, k, v, out = (buf.alloc((n, H, D), pkg.F16) for _ in range(4))
+        for t, seed in ((q, 11), (k, 12), (v, 13)):
+            be.rand_uniform(t, seed, -1.0, 1.0)
+        tcu = buf.from_numpy(cu)
+        be.scope_begin()
+        call = lambda: be.sdpa_varlen(q, k, v, tcu, out, 1.0 / np.sqrt(D))
+        call()
+        timer.start()
+        for _ in range(launches):
+            call()
+        timer.stop()
+        us = timer.elapsed_ms() * 1e3 / launches
+        be.fence_wait(be.record_fence())
+        pairs = int(sum(int(t) * (int(t) + 1) // 2 for t in lens))
+        flops = 4.0 * D * H * pairs
+        results.append({"prompts": label, "tokens": n, "heads": H, "head_dim": D, "us_per_launch": round(us, 1),
+                        "tflops_on_visible_pairs": round(flops / us / 1e6, 1),
+                        "frac_of_mfma_peak": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4)})
+    timer.close()
+    be.free(buf)
+    be.close()
+    print(json.dumps({"probe": "prefill_attention", "unit": "us per launch (stream events)",
+                      "peak_tflops_f16_mfma": MFMA_F16_PEAK_TFLOPS, "results": results}))
+
+
 def tile_timeline(pkg):
     """Per-tile time stamps of the prefill projection kernel (library built with TILE_TIMELINE=1): for each shape of
     tile_gemm and the up/gate + swiglu projection, microseconds in the K loop and in the epilogue per tile (mean over
@@ -249,4 +295,4 @@ def tile_timeline(pkg):
     print(json.dumps({"probe": "tile_timeline", "results": results}))
 
 
-PROBES = {"tile_timeline": tile_timeline, "sdpa_decode": sdpa_decode, "few_row_linear": few_row_linear, "tile_gemm": tile_gemm}
+PROBES = {"tile_timeline": tile_timeline, "prefill_attention": prefill_attention, "sdpa_decode": sdpa_decode, "few_row_linear": few_row_linear, "tile_gemm": tile_gemm}
