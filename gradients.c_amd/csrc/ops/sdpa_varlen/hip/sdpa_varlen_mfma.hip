@@ -90,16 +90,37 @@ gd_sdpa_varlen_mfma_kernel(const gd_half *__restrict__ q, const gd_half *__restr
     const uint32_t hq = blockIdx.x % p.hq, pair = blockIdx.x / p.hq;
     const uint32_t hkv = hq / (p.hq / p.hkv);
 
-    /* (segment, 128-row block) number `pair` */
+    /* (segment, 128-row block) number `pair`: lane t of the wavefront takes segment t of a run of 64 segments (one
+     * load of cu per lane instead of a chain of dependent scalar loads, which cost a workgroup of a short prompt as
+     * much as its attention), the blocks of the run are summed across the lanes, and the first lane whose running
+     * count passes `pair` names the segment */
     if (cu[0] < 0) return;
-    uint32_t seen = 0u, b = 0u;
+    uint32_t seen = 0u, b = p.batch;
     int start = 0, end = 0;
-    for (; b < p.batch; ++b) {
-        start = cu[b];
-        end = cu[b + 1u];
-        const uint32_t nb = end > start ? ((uint32_t)(end - start) + BQ - 1u) / BQ : 0u;
-        if (pair < seen + nb) break;
-        seen += nb;
+    for (uint32_t b0 = 0u; b0 < p.batch; b0 += 64u) {
+        const uint32_t bl = b0 + lane;
+        int s0 = 0, e0 = 0;
+        if (bl < p.batch) {
+            s0 = cu[bl];
+            e0 = cu[bl + 1u];
+        }
+        const uint32_t nb = e0 > s0 ? ((uint32_t)(e0 - s0) + BQ - 1u) / BQ : 0u;
+        uint32_t incl = nb; /* inclusive sum over the lanes below and this one */
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const uint32_t up = (uint32_t)__shfl_up((int)incl, off, 64);
+            if ((int)lane >= off) incl += up;
+        }
+        const unsigned long long hit = __builtin_amdgcn_ballot_w64(seen + incl > pair);
+        if (hit != 0ull) {
+            const int src = __builtin_ctzll(hit);
+            b = b0 + (uint32_t)src;
+            start = __shfl(s0, src, 64);
+            end = __shfl(e0, src, 64);
+            seen += (uint32_t)__shfl((int)(incl - nb), src, 64);
+            break;
+        }
+        seen += (uint32_t)__shfl((int)incl, 63, 64);
     }
     if (b == p.batch || end > (int)p.n_rows) return;
     const int T_len = end - start;
@@ -151,6 +172,8 @@ gd_sdpa_varlen_mfma_kernel(const gd_half *__restrict__ q, const gd_half *__restr
         for (int e = 0; e < 16; ++e) o[t][e] = 0.f;
     float m = GD_VL_NEG_INF, l = 0.f;
     const float scale2 = p.scale * 1.4426950408889634f;
+    const bool plain_causal = causal != 0 && window == 0 && prefix == 0;
+    const int jmax = min(i, T_len - 1); /* last visible key of this lane's row under plain causal attention */
 
     /* transposing read coordinates of this lane: group g = lane/16 -> channel block 16*(g&1), key half g/2 == h;
      * lane q + 4e of a group addresses key row e, channels 4q .. 4q+3 */
@@ -204,7 +227,9 @@ gd_sdpa_varlen_mfma_kernel(const gd_half *__restrict__ q, const gd_half *__restr
                 float s = st[t][e] * scale2;
                 if (!full) {
                     const int j = jb + 32 * t + 8 * (e >> 2) + 4 * (int)h + (e & 3);
-                    if (j >= T_len || !gd_vl_allowed(i, j, causal, window, prefix)) s = GD_VL_NEG_INF;
+                    /* plain causal attention (no window, no prefix): one comparison against min(i, T_len - 1) */
+                    if (plain_causal ? j > jmax : (j >= T_len || !gd_vl_allowed(i, j, causal, window, prefix)))
+                        s = GD_VL_NEG_INF;
                 }
                 st[t][e] = s;
                 mloc = fmaxf(mloc, s);

@@ -494,6 +494,20 @@ def test_varlen_many_blocks_matches_oracle(backend, arena, oracle, H, Hkv, D, ca
     _close(out.read(), oracle.sdpa_varlen(q, k, v, cu, scale, causal, window, prefix, 0))
 
 
+def test_varlen_many_segments(backend, arena, oracle):
+    """150 segments of 0..200 tokens (empty ones among them, some longer than a 128-row query block): a workgroup
+    finds its segment by a search over runs of 64 segments, so the segment index crosses two run boundaries."""
+    lens = oracle.uniform_i32(150, 741, 0, 201)
+    lens[[0, 63, 64, 127, 128, 149]] = [0, 130, 0, 129, 200, 1]
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    N = int(cu[-1])
+    q, k, v = (oracle.normal_f16((N, 2, 64), sd) for sd in (742, 743, 744))
+    out = arena.from_numpy(np.full(q.shape, 5.0, np.float16))
+    backend.sdpa_varlen(arena.from_numpy(q), arena.from_numpy(k), arena.from_numpy(v), arena.from_numpy(cu), out,
+                        0.125, True, 0, 0, 0)
+    _close(out.read(), oracle.sdpa_varlen(q, k, v, cu, 0.125, True, 0, 0, 0))
+
+
 def test_varlen_ignores_values_of_the_next_segment(backend, arena, oracle):
     """Keys past a segment's end are never used, even if the neighbouring segment holds infinities."""
     cu = np.array([0, 70, 140], np.int32)
