@@ -174,7 +174,10 @@ def tile_gemm(pkg, launches=6):
         y = buf.alloc((M, N), pkg.F16)
         be.scope_begin()
         call = lambda: be.fused_linear(x, w, b, r if res_on else None, None, y, True, 2, 0, 0.0, epi)
-        call()
+        # the first matrix work of a process runs at a lower clock than what follows (about 15 % on the first shape):
+        # the chip is given some ten milliseconds of it before anything is timed
+        for _ in range(12 if not results else 1):
+            call()
         timer.start()
         for _ in range(launches):
             call()
