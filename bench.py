@@ -519,10 +519,9 @@ def main():
     ap.add_argument("--minimax-kernels", action="store_true",
                     help="time the MiniMax-M3 block picker and block-sparse attention next to dense causal attention on "
                          "packed sequences (auxiliary: prints its own JSON line, not the headline metric)")
-    ap.add_argument("--probe", choices=("sdpa_decode", "sdpa_decode_balanced", "few_row_linear", "tile_gemm", "tile_timeline", "prefill_attention"),
+    ap.add_argument("--probe", choices=("sdpa_decode", "few_row_linear", "tile_gemm", "tile_timeline", "prefill_attention"),
                     help="operator-local performance probe (gradients.c_amd/perf_probes.py): one operator at the shapes of "
-                         "the BASELINE.json configurations, operands rotating through HBM; prints its own JSON line. "
-                         "sdpa_decode_balanced also times the form that deals the keys to the wavefronts by count")
+                         "the BASELINE.json configurations, operands rotating through HBM; prints its own JSON line")
     ap.add_argument("--kernel-only", action="store_true",
                     help="only launch sdpa_decode at the benchmark shape plus calibration copies (for --pmc runs)")
     a = ap.parse_args()
@@ -537,9 +536,7 @@ def main():
         return
     if a.probe:
         from gradients_c_amd import perf_probes
-        if a.probe == "sdpa_decode_balanced":
-            perf_probes.sdpa_decode(pkg, balanced=(0, 1))
-        elif a.probe == "tile_gemm":
+        if a.probe == "tile_gemm":
             perf_probes.tile_gemm(pkg, launches=max(1, min(a.steps, 6)))
         else:
             perf_probes.PROBES[a.probe](pkg)

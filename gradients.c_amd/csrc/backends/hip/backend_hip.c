@@ -114,7 +114,6 @@ gd_status gd_backend_create_default(gd_backend **out_backend)
     b->sdpa_waves = env_int("GD_HIP_SDPA_WAVES", 0, 4, 8);
     b->sdpa_unroll = env_int("GD_HIP_SDPA_UNROLL", 0, 2, 8);
     b->linear_wide = env_int("GD_HIP_LINEAR_WIDE", -1, -1, 1);
-    b->sdpa_balanced = env_int("GD_HIP_SDPA_BALANCED", 0, 0, 2);
     b->sdpa_nontemporal = env_int("GD_HIP_SDPA_NONTEMPORAL", -1, -1, 1);
     b->linear_tiles = env_int("GD_HIP_LINEAR_TILES", 0, 1, 4);
     b->linear_waves = env_int("GD_HIP_LINEAR_WAVES", 0, 4, 8);
@@ -175,11 +174,6 @@ gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t 
     if (strcmp(name, "linear_wide") == 0) {
         if (value < -1 || value > 1) return GD_ERR_INVALID_ARGUMENT;
         backend->linear_wide = (int)value;
-        return GD_OK;
-    }
-    if (strcmp(name, "sdpa_balanced") == 0) {
-        if (value < 0 || value > 2) return GD_ERR_INVALID_ARGUMENT;
-        backend->sdpa_balanced = (int)value;
         return GD_OK;
     }
     if (strcmp(name, "sdpa_nontemporal") == 0) {

@@ -50,7 +50,6 @@ struct gd_backend {
     int sdpa_waves;      /* 4 or 8 wavefronts per workgroup (0 = default 8) */
     int sdpa_unroll;     /* 4 or 8 key-row loads in flight per lane (0 = default 8) */
     int linear_wide;      /* few-row projections over large [N,K] weights: 1 always the wide kernel, 0 never, -1 from 4 MiB */
-    int sdpa_balanced;    /* keys dealt to wavefronts by count: 0 no (default), 1 / 2 yes (8 / 16 wavefronts per unit) */
     int sdpa_nontemporal; /* streaming hint on the K/V loads: 1 always, 0 never, -1 by the size of the caches */
     int m3_simple;        /* 1: MiniMax-M3 operators always take the per-row kernels (tests compare the two paths) */
     int linear_tiles;    /* few-row projections: 16-column tiles per workgroup, 1 / 2 / 4 (0 = automatic) */

@@ -13,9 +13,6 @@
 int gd_hip_launch_sdpa_decode_split(hipStream_t stream, const void *q, const void *k, const void *v,
                                     const int32_t *pos, void *out, float *ws,
                                     const gd_hip_sdpa_decode_params *params);
-int gd_hip_launch_sdpa_decode_balanced(hipStream_t stream, const void *q, const void *k, const void *v,
-                                       const int32_t *pos, void *out, float *ws,
-                                       const gd_hip_sdpa_decode_params *params, uint32_t shares);
 int gd_hip_launch_sdpa_decode_generic(hipStream_t stream, const void *q, const void *k, const void *v,
                                       const int32_t *pos, void *out, const gd_hip_sdpa_decode_params *params);
 
@@ -94,41 +91,6 @@ static gd_status dispatch(gd_backend *backend, const gd_backend_tensor_view *q, 
         if (p.window > 0u && p.prefix_len > 0u) span = span + p.prefix_len < p.tmax ? span + p.prefix_len : p.tmax;
         uint32_t chunk = (uint32_t)backend->sdpa_chunk;
         gd_status st;
-        /* On request (tunable "sdpa_balanced"): the keys of all rows are dealt to the wavefronts by count
-         * (sdpa_decode_balanced.hip), so that the longest row does not decide the time of the launch.  Not chosen
-         * automatically: measured on MI355X with caches rotating through HBM it is slower than one workgroup per
-         * (row, kv head) at every shape tried (16 x 16 heads of 128, 1024..4095 keys: 64 against 60 us, the same
-         * bytes in equal rows: 61 against 54 us; 32 x 8 heads of 64, 1..4096 keys: 42 against 37 us), because
-         * 2048 wavefronts each walking its own stretch of a [T, Hkv, D] cache touch far more DRAM pages at a time
-         * than 256 workgroups whose wavefronts read neighbouring rows. */
-        if (pos_mode == GD_HIP_SDPA_POS_VECTOR && p.prefix_len == 0u && backend->sdpa_chunk == 0 &&
-            backend->sdpa_balanced > 0 && (group & (group - 1u)) == 0u && (uint64_t)p.batch * p.hkv * p.tmax < 0x7fffffffull) {
-            /* a share is what one wavefront streams: 8 (or 16) wavefronts per compute unit */
-            const uint32_t shares = (uint32_t)backend->compute_units * (backend->sdpa_balanced > 1 ? 16u : 8u);
-            const size_t need = ((size_t)p.batch * p.hkv + shares) * group * (p.dh + 4u) * sizeof(float);
-            float *ws;
-            if (noalloc) {
-                ws = gd_hip_sdpa_decode_scratch(backend->device);
-                if (ws == NULL) return GD_ERR_BAD_STATE;
-                if (need > GD_HIP_SDPA_NOALLOC_SCRATCH_BYTES) {
-                    fprintf(stderr, "gd_backend_sdpa_decode_positions_noalloc: the partial results of this call "
-                                    "need %zu bytes, the fixed scratch holds %u\n",
-                            need, (unsigned)GD_HIP_SDPA_NOALLOC_SCRATCH_BYTES);
-                    return GD_ERR_OUT_OF_MEMORY;
-                }
-            } else {
-                st = gd_hip_reserve_attn_ws(backend, need);
-                if (st != GD_OK) return st;
-                ws = (float *)backend->attn_ws;
-            }
-            {
-                const uint32_t rec[11] = {3u, p.dh, group, 8u, 2u, p.nontemporal, 0u, shares, 1u, 1u, 0u};
-                memcpy(backend->last_sdpa, rec, sizeof(rec));
-            }
-            return gd_hip_finish_op(backend, gd_hip_launch_sdpa_decode_balanced(
-                backend->stream, gd_hip_view_ptr(q), gd_hip_view_ptr(k), gd_hip_view_ptr(v), pos_ptr,
-                gd_hip_view_ptr(out), ws, &p, shares));
-        }
         if (chunk == 0u) {
             /* one workgroup per (batch row, kv head) as soon as that gives every compute unit one (a single pass, no
              * combine kernel: measured 6 % faster than two splits at 256 pairs x 4096 keys); below that, split the
@@ -251,9 +213,6 @@ gd_status gd_backend_sdpa_decode_last_kernel(gd_backend *backend, char *out, siz
     if (r[0] == 1u)
         snprintf(out, capacity, "gd_sdpa_decode_split_kernel<%u,%u,%u,%u,%s%s> [grid %u x %u x %u, %u keys per workgroup]",
                  r[1], r[2], r[3], r[4], r[5] ? "true" : "false", r[6] ? ",true" : "", r[7], r[8], r[9], r[10]);
-    else if (r[0] == 3u)
-        snprintf(out, capacity, "gd_sdpa_decode_balanced_kernel<%u,%u,%s> [%u wavefronts, keys dealt by count]", r[1], r[2],
-                 r[5] ? "true" : "false", r[7]);
     else if (r[0] == 2u)
         snprintf(out, capacity, "gd_sdpa_decode_generic_kernel<%s> [grid %u]", r[5] == 1u ? "gd_half" : "float", r[7]);
     else

@@ -1,5 +1,5 @@
 /*
- * Device helpers shared by the sdpa_decode kernels (sdpa_decode.hip, sdpa_decode_balanced.hip): the reference's
+ * Device helpers shared by the sdpa_decode kernels (sdpa_decode.hip): the reference's
  * visibility mask, the position lookup, and the lane-group reductions of the split-KV kernels.
  */
 #ifndef GD_SDPA_DECODE_DEVICE_H

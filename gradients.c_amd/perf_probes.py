@@ -46,9 +46,9 @@ def _timed(pkg, be, fns, replays=4, repeats=3):
     return sorted(res)[len(res) // 2]
 
 
-def sdpa_decode(pkg, balanced=(0,)):
+def sdpa_decode(pkg):
     """gd_backend_sdpa_decode_positions at the shapes of configs[2], [1], [3], [4] and at equal rows of the same total
-    size (what raggedness costs).  `balanced`: values of the tunable "sdpa_balanced" to time."""
+    size (what raggedness costs)."""
     be = pkg.Backend()
     shapes = [("configs[2]: B64 H8 D64, 512 keys", 64, 8, 64, 512, None),
               ("configs[1]: B32 H8 D64, 1..4096 keys", 32, 8, 64, 4352, (1, 4097)),
@@ -74,20 +74,16 @@ def sdpa_decode(pkg, balanced=(0,)):
         out = buf.alloc((B, 1, H, Dh), pkg.F16)
         pos = buf.from_numpy(lens)
         algo = int(np.sum(lens.astype(np.int64) + 1)) * H * Dh * 4 + 2 * B * H * Dh * 2 + 4 * B
-        for bal in balanced:
+        for _ in (0,):
             for nt in (-1, 0, 1):
-                if bal and nt != 1:
-                    continue
-                be.set_tunable("sdpa_balanced", bal)
                 be.set_tunable("sdpa_nontemporal", nt)
                 fns = [(lambda kv=kv: be.sdpa_decode_positions(q, kv[0], kv[1], pos, out, 1.0 / np.sqrt(Dh)))
                        for _ in range(3) for kv in sets]   # consecutive launches read different caches
                 us = _timed(pkg, be, fns)
-                rows.append({"shape": label, "streaming_loads": {-1: "auto", 0: "off", 1: "on"}[nt], "keys_by_count": bal,
+                rows.append({"shape": label, "streaming_loads": {-1: "auto", 0: "off", 1: "on"}[nt],
                              "kernel": be.sdpa_decode_last_kernel(), "us_per_launch": round(us, 2),
                              "gbs": round(algo / us / 1e3, 1), "frac_of_hbm_peak": round(algo / us / 1e3 / HBM_PEAK_GBS, 4),
                              "algorithmic_bytes": algo, "distinct_cache_sets": nsets})
-        be.set_tunable("sdpa_balanced", 0)
         be.set_tunable("sdpa_nontemporal", -1)
         be.free(buf)
     be.close()

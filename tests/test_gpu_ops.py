@@ -256,6 +256,29 @@ def test_decode_isolated_config_shape(backend, arena, oracle, chunk):
     _close(out.read(), oracle.sdpa_decode(q, wk, wv, L, 0.125))
 
 
+def test_decode_isolated_config_full_size(backend, oracle):
+    """BASELINE config 1 at its full size: B=32, H=8, DH=64, caches of 4097 rows, lengths uniform in [1, 4096]; one
+    token appended per sequence (bit-exact), then the decode over L+1 keys against the oracle.  At this size (275 MB
+    of caches) the dispatch picks the 8-wavefront form with streaming loads, which no smaller case reaches."""
+    B, H, D, Tmax = 32, 8, 64, 4097
+    big = backend.buffer(640 << 20)
+    try:
+        L = oracle.uniform_i32(B, 1101, 1, 4096)
+        k0, v0 = oracle.normal_f16((B, Tmax, H, D), 1102), oracle.normal_f16((B, Tmax, H, D), 1103)
+        q, kn, vn = (oracle.normal_f16((B, 1, H, D), sd) for sd in (1104, 1105, 1106))
+        tk, tv, tp = big.from_numpy(k0), big.from_numpy(v0), big.from_numpy(L)
+        backend.kv_cache_append_positions(tk, tv, tp, big.from_numpy(kn), big.from_numpy(vn))
+        oracle.kv_cache_append(k0, v0, kn, vn, L)
+        assert np.array_equal(_bits(tk.read()), _bits(k0)) and np.array_equal(_bits(tv.read()), _bits(v0))
+        out = big.from_numpy(np.full(q.shape, 7.0, np.float16))
+        backend.sdpa_decode_positions(big.from_numpy(q), tk, tv, tp, out, 0.125)
+        name = backend.sdpa_decode_last_kernel()
+        assert name.startswith("gd_sdpa_decode_split_kernel<64,1,8,") and ",true>" in name, name
+        _close(out.read(), oracle.sdpa_decode(q, k0, v0, L, 0.125))
+    finally:
+        backend.free(big)
+
+
 @pytest.mark.parametrize("D,chunk", [(64, 0), (64, 32), (128, 0), (128, 64)])
 def test_decode_ignores_rows_behind_the_live_range(backend, arena, oracle, D, chunk):
     """Cache rows behind a sequence's last live key may hold anything (another request's rows, NaN, infinities): the
@@ -283,40 +306,6 @@ def test_decode_ignores_rows_behind_the_live_range(backend, arena, oracle, D, ch
     _close(got, oracle.sdpa_decode(q, k, v, pos, 1.0 / np.sqrt(D)))
 
 
-@pytest.mark.parametrize("B,H,Hkv,D,Tmax,window,per_unit", [
-    (5, 4, 4, 64, 700, 0, 1), (5, 4, 4, 128, 700, 0, 2), (70, 2, 2, 64, 130, 0, 1), (9, 8, 2, 64, 300, 0, 1),
-    (6, 8, 1, 128, 257, 0, 2), (7, 4, 2, 64, 500, 96, 1), (4, 2, 2, 128, 2100, 0, 1), (130, 1, 1, 64, 40, 7, 2)])
-def test_decode_keys_dealt_by_count(backend, arena, oracle, B, H, Hkv, D, Tmax, window, per_unit):
-    """The form of the split-KV kernel that deals the visible keys of all rows to the wavefronts by count (only on
-    request): ragged positions with one-key rows, full rows, rows past the cache end
-    and rows with a negative position (left untouched: the sentinel stays), first and last rows among them; more
-    rows than a wavefront has lanes; grouped query heads; windows.  Rows behind a position hold NaN."""
-    rng = np.random.default_rng(B * 1000 + Tmax)
-    pos = rng.integers(0, Tmax, B).astype(np.int32)
-    pos[0], pos[B - 1], pos[B // 2] = -1, -3, Tmax + 5
-    pos[1], pos[2] = 0, Tmax - 1
-    q = oracle.normal_f16((B, 1, H, D), 60)
-    k, v = oracle.normal_f16((B, Tmax, Hkv, D), 61), oracle.normal_f16((B, Tmax, Hkv, D), 62)
-    kd, vd = k.copy(), v.copy()
-    for b in range(B):
-        if 0 <= pos[b] < Tmax - 1:
-            kd[b, pos[b] + 1:] = np.nan
-            vd[b, pos[b] + 1:] = np.nan
-    sentinel = np.full(q.shape, 7.0, np.float16)
-    out = arena.from_numpy(sentinel)
-    backend.set_tunable("sdpa_balanced", per_unit)
-    try:
-        backend.sdpa_decode_positions(arena.from_numpy(q), arena.from_numpy(kd), arena.from_numpy(vd),
-                                      arena.from_numpy(pos), out, 1.0 / np.sqrt(D), window)
-        assert "balanced" in backend.sdpa_decode_last_kernel()
-    finally:
-        backend.set_tunable("sdpa_balanced", 0)
-    got = out.read()
-    assert np.isfinite(got.astype(np.float32)).all()
-    assert (got[0] == 7.0).all() and (got[B - 1] == 7.0).all()
-    _close(got, oracle.sdpa_decode(q, k, v, pos, 1.0 / np.sqrt(D), window, out_init=sentinel.astype(np.float32)))
-
-
 def test_decode_full_size_long_context_sampled(backend, oracle):
     """BASELINE config 3's attention at its full size (B=16, 16 heads of 128, 4096-row caches, live lengths in
     [1024, 4096]: 537 MB of cache filled on the device), checked on sampled batch rows against a float64 softmax of
@@ -340,12 +329,6 @@ def test_decode_full_size_long_context_sampled(backend, oracle):
                 backend.set_tunable("sdpa_chunk", 0)
             results.append(out.read().astype(np.float32))
         assert np.abs(results[0] - results[1]).max() < 1e-3 and np.abs(results[0] - results[2]).max() < 1e-3
-        backend.set_tunable("sdpa_balanced", 1)    # the keys dealt to the wavefronts by count
-        try:
-            backend.sdpa_decode_positions(tq, k, v, tp, out, scale)
-        finally:
-            backend.set_tunable("sdpa_balanced", 0)
-        assert np.abs(results[0] - out.read().astype(np.float32)).max() < 1e-3
         for b in (0, 7, 15):
             n = int(pos[b]) + 1
             kb = k.rows(b, 1).read()[0, :n].astype(np.float64)  # [n, H, D]
@@ -365,6 +348,29 @@ def test_decode_full_size_long_context_sampled(backend, oracle):
 def test_decode_head_layouts(backend, arena, oracle, H, Hkv, D):
     pos = np.array([0, 1, 63, 64, 200, 299, -1, 31], np.int32)
     _decode_case(backend, arena, oracle, 8, H, Hkv, D, 300, pos, 1.0 / np.sqrt(D), seed=200 + H + D, chunk=96)
+
+
+@pytest.mark.parametrize("H,Hkv,D", [(8, 8, 64), (16, 16, 128), (8, 2, 64), (6, 1, 64)])
+@pytest.mark.parametrize("waves", [4, 8])
+def test_decode_streaming_loads_give_the_same_bits(backend, arena, oracle, H, Hkv, D, waves):
+    """The instantiations with streaming (non-temporal) K/V loads, which the dispatch picks by itself only above
+    128 MiB of caches, forced on at a size the oracle covers: within the bar of the oracle, and the same bits as the
+    cacheable form (the hint changes the cache policy of a load, not its value)."""
+    pos = np.array([0, 1, 63, 64, 200, 299, -1, 31], np.int32)
+    backend.set_tunable("sdpa_waves", waves)
+    try:
+        plain = _decode_case(backend, arena, oracle, 8, H, Hkv, D, 300, pos, 1.0 / np.sqrt(D), seed=230 + H + D, chunk=96)
+        assert ",false>" in backend.sdpa_decode_last_kernel()
+        backend.set_tunable("sdpa_nontemporal", 1)
+        try:
+            hinted = _decode_case(backend, arena, oracle, 8, H, Hkv, D, 300, pos, 1.0 / np.sqrt(D), seed=230 + H + D, chunk=96)
+            name = backend.sdpa_decode_last_kernel()
+        finally:
+            backend.set_tunable("sdpa_nontemporal", -1)
+    finally:
+        backend.set_tunable("sdpa_waves", 0)
+    assert ",true>" in name and (H != Hkv or f",{waves}," in name), name
+    assert np.array_equal(_bits(plain), _bits(hinted))
 
 
 @pytest.mark.parametrize("window", [1, 7, 256, 1000])
@@ -492,6 +498,44 @@ def test_varlen_many_blocks_matches_oracle(backend, arena, oracle, H, Hkv, D, ca
     backend.sdpa_varlen(arena.from_numpy(q), arena.from_numpy(k), arena.from_numpy(v), arena.from_numpy(cu), out,
                         scale, causal, window, prefix, 0)
     _close(out.read(), oracle.sdpa_varlen(q, k, v, cu, scale, causal, window, prefix, 0))
+
+
+@pytest.mark.parametrize("H,Hkv,D,causal,window,prefix", [(4, 2, 64, True, 0, 0), (2, 2, 128, True, 9, 3), (3, 1, 20, False, 0, 0),
+                                                          (2, 1, 32, True, 40, 0)])
+def test_varlen_f32_tensors(backend, arena, oracle, H, Hkv, D, causal, window, prefix):
+    """F32 q/k/v/out (the reference accepts F16 and F32: src/ops/sdpa_varlen/core_sdpa_varlen.c:12-122).  Two checks:
+    inputs that are exactly representable in F16 against the oracle (which then computes the same problem), and
+    arbitrary F32 inputs against a float64 softmax over the visible set, the in-test model of the reference
+    (tests/test_sdpa_varlen.c:158-230); bar 1e-5 relative + 2e-6 absolute, F32 accumulation."""
+    lens = np.array([70, 1, 0, 131, 33], np.int32)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    N = int(cu[-1])
+    qh, kh, vh = oracle.normal_f16((N, H, D), 760), oracle.normal_f16((N, Hkv, D), 761), oracle.normal_f16((N, Hkv, D), 762)
+    tcu = arena.from_numpy(cu)
+    out = arena.from_numpy(np.full(qh.shape, 3.0, np.float32))
+    backend.sdpa_varlen(arena.from_numpy(qh.astype(np.float32)), arena.from_numpy(kh.astype(np.float32)),
+                        arena.from_numpy(vh.astype(np.float32)), tcu, out, 0.15, causal, window, prefix, 0)
+    _close(out.read(), oracle.sdpa_varlen(qh, kh, vh, cu, 0.15, causal, window, prefix, 0), 2e-5, 4e-6)
+    rng = np.random.default_rng(763)
+    q, k, v = (rng.standard_normal(sh).astype(np.float32) for sh in ((N, H, D), (N, Hkv, D), (N, Hkv, D)))
+    out = arena.from_numpy(np.full(q.shape, 3.0, np.float32))
+    backend.sdpa_varlen(arena.from_numpy(q), arena.from_numpy(k), arena.from_numpy(v), tcu, out, 0.15, causal, window, prefix, 0)
+    got = out.read()
+    want = np.zeros(q.shape, np.float64)
+    for b in range(len(lens)):
+        s0, T = int(cu[b]), int(lens[b])
+        i, j = np.arange(T)[:, None], np.arange(T)[None, :]
+        vis = np.ones((T, T), bool)   # the mask of tests/test_sdpa_varlen.c:122-148 of the reference, as array logic
+        if causal:
+            vis &= np.where(i < prefix, j < prefix, j <= i) if prefix > 0 else (j <= i)
+        if window > 0:
+            vis &= ~((i >= prefix) & (j >= prefix) & (i - j >= window)) if prefix > 0 else (i - j < window)
+        for h in range(H):
+            sc = q[s0:s0 + T, h].astype(np.float64) @ k[s0:s0 + T, h // (H // Hkv)].astype(np.float64).T * 0.15
+            sc = np.where(vis, sc, -np.inf)
+            w = np.exp(sc - sc.max(axis=1, keepdims=True)) if T else sc
+            want[s0:s0 + T, h] = (w / w.sum(axis=1, keepdims=True)) @ v[s0:s0 + T, h // (H // Hkv)].astype(np.float64)
+    _close(got, want, 2e-5, 4e-6)
 
 
 def test_varlen_many_segments(backend, arena, oracle):

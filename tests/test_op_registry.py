@@ -63,6 +63,11 @@ def test_unsupported_table_is_the_boundary_minus_what_the_backend_defines(gda):
     for must_be_real in ("gd_backend_sdpa_decode", "gd_backend_kv_cache_append_positions", "gd_backend_matmul_nt",
                          "gd_backend_rms_norm_forward", "gd_backend_add", "gd_backend_concat_to_full"):
         assert must_be_real in listed and must_be_real not in stubs
+    # declared at the reference's boundary (src/core/backend.h:259,772,776) although its core calls only the batched
+    # forms: a build that pulls them in must fail at run time with GD_ERR_UNSUPPORTED, not at link time
+    for declared_only in ("gd_backend_adamw", "gd_backend_amp_unscale", "gd_backend_broadcast_to"):
+        assert declared_only in stubs
+    assert len(listed) >= 109
 
 
 def test_lookups_of_the_library(gda):
