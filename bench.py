@@ -39,6 +39,80 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # published dense F16 matrix rate
 SDPA_TRAFFIC_BYTES = 67300600
 
 
+# A hardware queue's ring holds 16384 dispatch packets.  rocprofv3's queue interception has ended the profiled process
+# with a segmentation fault inside hipGraphLaunch whenever a graph launch wrapped around the end of that ring, so a
+# profiled run must stay below it.  Unprofiled runs are not affected.
+QUEUE_RING_PACKETS = 16384
+
+
+def profiler_attached(env=None):
+    """True when a rocprofiler tool library rides in this process (rocprofv3 sets these for the program it starts)."""
+    env = os.environ if env is None else env
+    if any(k.startswith(("ROCPROF_", "ROCPROFILER_", "ROCP_TOOL")) for k in env):
+        return True
+    return "rocprofiler" in env.get("LD_PRELOAD", "") or "rocprofiler" in env.get("HSA_TOOLS_LIB", "")
+
+
+def planned_dispatches(a):
+    """Upper estimate of the dispatch packets the chosen flags put on the backend's queue, as (total, parts): pure
+    arithmetic on the flags.  A fused decode step is 5 launches per layer + 2; weight initialisation and a packed
+    prefill are priced at 12 launches per layer + 8 each (more than either issues); a step through the public
+    operators (step 0 of a resident session) at 14 per layer + 6."""
+    def init(layers):
+        return 12 * layers + 8
+
+    def step(layers):
+        return 5 * layers + 2
+
+    def eager_step(layers):
+        return 14 * layers + 6
+
+    def long_context(which, steps, warmup, batches):
+        if a.prefill_only:
+            return init(24) + 2 * init(24)
+        if which == 4:
+            steps, warmup, batches = a.decode_steps, 0, 1
+        return init(24) + 2 * init(24) + eager_step(24) + (warmup + steps * batches) * step(24)
+
+    parts = {}
+    if a.kernel_only:
+        parts["kernel_only"] = 40
+    elif a.probe:
+        # graphs of at most a few dozen launches, replayed 13 times per timing (perf_probes._timed)
+        parts["probe"] = {"sdpa_decode": 7 * 3 * (2 + 13) * 30, "few_row_linear": 3 * 10 * (2 + 13) * 24}.get(a.probe, 400)
+    elif a.minimax_kernels:
+        parts["minimax_kernels"] = 2 * (8 + 4 * (1 + 10 + 20))
+    elif a.workload != 2:
+        parts[f"configs[{a.workload}]"] = long_context(a.workload, a.steps, a.warmup, (a.batches or 3) if a.workload == 3 else 1)
+    elif a.sampled:
+        parts["sampled"] = 2 * init(3) + eager_step(3) + (a.warmup + a.steps) * (step(3) + 2)
+    else:
+        batches = a.batches or 5
+        parts["configs[2]"] = 2 * init(3) + eager_step(3) + (a.warmup + batches * a.steps) * step(3)
+        parts["roofline"] = 12 + 2 * (1 + 24 * (4 + max(1, 200 // 24)))
+        if not a.headline_only:
+            parts["configs[0]"] = init(3) + 6 * init(3) + 5 * (eager_step(3) + 63 * (step(3) + 1))
+            parts["configs[1]"] = 8 + 2 * (2 + 24 * (2 + 120 // 12))
+            parts["configs[3]"] = long_context(3, 20, 3, 3)
+            parts["configs[4]"] = long_context(4, 0, 0, 1)
+    return sum(parts.values()), parts
+
+
+def refuse_if_profiled_run_would_wrap_the_queue(a, env=None):
+    """Exits non-zero, before anything touches the GPU, when a profiler is attached and the flags would queue more
+    dispatch packets than the ring holds."""
+    if not profiler_attached(env):
+        return
+    total, parts = planned_dispatches(a)
+    if total >= QUEUE_RING_PACKETS:
+        sys.exit(f"bench.py: refusing to run under the profiler: these flags queue about {total} dispatch packets "
+                 f"({parts}), the hardware queue's ring holds {QUEUE_RING_PACKETS}, and rocprofv3's queue interception "
+                 "has crashed the profiled process (segmentation fault inside hipGraphLaunch) whenever a graph launch "
+                 "wrapped around the ring's end.  Profile one workload per process with fewer steps, e.g. "
+                 "--headline-only --no-cpu-baseline --batches 1, --workload 3 --steps 40 --warmup 5 --batches 1, "
+                 "--workload 4 --decode-steps 80.")
+
+
 def _package():
     import __graft_entry__ as entry
     return entry._package(), entry._oracle()
@@ -492,7 +566,7 @@ def sampled_workload(a, oracle, D):
     }))
 
 
-def main():
+def build_parser():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
@@ -500,9 +574,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--batches", type=int, default=0,
                     help="how many times the K steps are timed (the median batch is reported); default 5 for the headline "
-                         "line, 3 for --workload 3.  Kernel traces use --batches 1: rocprofv3's queue interception "
-                         "crashes the profiled process once the 16384 dispatch packets of a hardware queue's ring have "
-                         "been used and a graph launch wraps around its end")
+                         "line, 3 for --workload 3.  Kernel traces use --batches 1: a profiled run that would "
+                         "queue more dispatch packets than a hardware queue's ring holds is refused (QUEUE_RING_PACKETS)")
     ap.add_argument("--decode-steps", type=int, default=128,
                     help="--workload 4: greedy steps after the prefill (BASELINE: 128; fewer for kernel traces, see --batches)")
     ap.add_argument("--headline-only", action="store_true",
@@ -524,11 +597,16 @@ def main():
                          "the BASELINE.json configurations, operands rotating through HBM; prints its own JSON line")
     ap.add_argument("--kernel-only", action="store_true",
                     help="only launch sdpa_decode at the benchmark shape plus calibration copies (for --pmc runs)")
-    a = ap.parse_args()
+    return ap
+
+
+def main():
+    a = build_parser().parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU: the decode path holds every sequence, its K/V cache and a full "
                  "weight replica on a single device (sequences are independent, so more GPUs would only add "
                  "replicas); run with --gpus 1")
+    refuse_if_profiled_run_would_wrap_the_queue(a)
     pkg, oracle = _package()
     pkg.lib()
     if a.kernel_only:
