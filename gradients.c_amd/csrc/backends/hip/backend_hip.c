@@ -55,6 +55,12 @@ gd_status gd_hip_reserve_attn_ws(gd_backend *backend, size_t nbytes)
         (void)hipGetLastError();
         return GD_ERR_OUT_OF_MEMORY;
     }
+    /* the block starts with arrival counters that the kernels find at zero and leave at zero */
+    if (hipMemset(p, 0, nbytes) != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipFree(p);
+        return GD_ERR_INTERNAL;
+    }
     if (backend->attn_ws != NULL) {
         if (backend->live_graphs > 0) backend->retired_ws[backend->retired_ws_count++] = backend->attn_ws;
         else (void)hipFree(backend->attn_ws);
@@ -114,6 +120,7 @@ gd_status gd_backend_create_default(gd_backend **out_backend)
     b->sdpa_waves = env_int("GD_HIP_SDPA_WAVES", 0, 4, 8);
     b->sdpa_unroll = env_int("GD_HIP_SDPA_UNROLL", 0, 2, 8);
     b->linear_wide = env_int("GD_HIP_LINEAR_WIDE", -1, -1, 1);
+    b->sdpa_merge = env_int("GD_HIP_SDPA_MERGE", 1, 0, 2);
     b->sdpa_nontemporal = env_int("GD_HIP_SDPA_NONTEMPORAL", -1, -1, 1);
     b->linear_tiles = env_int("GD_HIP_LINEAR_TILES", 0, 1, 4);
     b->linear_waves = env_int("GD_HIP_LINEAR_WAVES", 0, 4, 8);
@@ -174,6 +181,11 @@ gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t 
     if (strcmp(name, "linear_wide") == 0) {
         if (value < -1 || value > 1) return GD_ERR_INVALID_ARGUMENT;
         backend->linear_wide = (int)value;
+        return GD_OK;
+    }
+    if (strcmp(name, "sdpa_merge") == 0) {
+        if (value < 0 || value > 2) return GD_ERR_INVALID_ARGUMENT;
+        backend->sdpa_merge = (int)value;
         return GD_OK;
     }
     if (strcmp(name, "sdpa_nontemporal") == 0) {

@@ -44,12 +44,13 @@ struct gd_backend {
     hipEvent_t graph_events[GD_HIP_GRAPH_RING];
     unsigned graph_launches;
     /* what the last sdpa_decode dispatch launched: 0 none, 1 split, 2 generic; D, G, W, U, streaming, prefix, grid */
-    uint32_t last_sdpa[11];
+    uint32_t last_sdpa[12];
     /* tunables read from the environment once at creation */
     int sdpa_chunk;      /* keys per workgroup in the split-KV decode kernel (0 = automatic) */
     int sdpa_waves;      /* 4 or 8 wavefronts per workgroup (0 = default 8) */
     int sdpa_unroll;     /* 4 or 8 key-row loads in flight per lane (0 = default 8) */
     int linear_wide;      /* few-row projections over large [N,K] weights: 1 always the wide kernel, 0 never, -1 from 4 MiB */
+    int sdpa_merge;       /* ragged batches in pieces merged inside the kernel: 1 (default) where it pays, 0 never, 2 wherever it applies */
     int sdpa_nontemporal; /* streaming hint on the K/V loads: 1 always, 0 never, -1 by the size of the caches */
     int m3_simple;        /* 1: MiniMax-M3 operators always take the per-row kernels (tests compare the two paths) */
     int linear_tiles;    /* few-row projections: 16-column tiles per workgroup, 1 / 2 / 4 (0 = automatic) */

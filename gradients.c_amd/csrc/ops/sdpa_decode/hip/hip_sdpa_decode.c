@@ -13,12 +13,17 @@
 int gd_hip_launch_sdpa_decode_split(hipStream_t stream, const void *q, const void *k, const void *v,
                                     const int32_t *pos, void *out, float *ws,
                                     const gd_hip_sdpa_decode_params *params);
+int gd_hip_launch_sdpa_decode_pieces(hipStream_t stream, const void *q, const void *k, const void *v,
+                                     const int32_t *pos, void *out, float *ws,
+                                     const gd_hip_sdpa_decode_params *params);
 int gd_hip_launch_sdpa_decode_generic(hipStream_t stream, const void *q, const void *k, const void *v,
                                       const int32_t *pos, void *out, const gd_hip_sdpa_decode_params *params);
 
 float *gd_hip_sdpa_decode_scratch(int device);
 
 #define GD_HIP_SDPA_MAX_DH 256
+/* keys per piece of a ragged batch (PIECES form) */
+#define GD_HIP_SDPA_PIECE_KEYS 256u
 _Static_assert(GD_HIP_SDPA_NOALLOC_SCRATCH_BYTES == GD_BACKEND_SDPA_DECODE_NOALLOC_SCRATCH_BYTES,
                "public constant and device array differ");
 
@@ -91,6 +96,54 @@ static gd_status dispatch(gd_backend *backend, const gd_backend_tensor_view *q, 
         if (p.window > 0u && p.prefix_len > 0u) span = span + p.prefix_len < p.tmax ? span + p.prefix_len : p.tmax;
         uint32_t chunk = (uint32_t)backend->sdpa_chunk;
         gd_status st;
+        /* Ragged batches: rows cut into pieces, one workgroup each, the last piece of a row to arrive merges it
+         * (sdpa_decode_pieces.hip).  Taken by itself when there is a (row, kv head) pair for every compute unit
+         * (below that the key range is split to fill the device, as before) and rows can be long enough for
+         * raggedness to matter; tunable "sdpa_merge": 0 never, 2 whenever the form applies.  The kernel keeps rows of
+         * about one length whole, so an even batch costs about what one workgroup per row costs. */
+        {
+            const uint64_t pairs = (uint64_t)p.batch * p.hkv;
+            uint32_t piece = chunk != 0u ? ((chunk + 31u) & ~31u) : GD_HIP_SDPA_PIECE_KEYS;
+            uint32_t pieces;
+            size_t need;
+            if ((uint64_t)piece * GD_HIP_SDPA_MAX_PIECES < span)
+                piece = ((span + GD_HIP_SDPA_MAX_PIECES - 1u) / GD_HIP_SDPA_MAX_PIECES + 31u) & ~31u;
+            pieces = (span + piece - 1u) / piece;
+            need = ((size_t)GD_HIP_SDPA_COUNTER_SLOTS + (size_t)p.batch * p.hq * pieces * (p.dh + 2u)) * sizeof(float);
+            const bool applies = pos_mode == GD_HIP_SDPA_POS_VECTOR && p.batch <= GD_HIP_SDPA_PIECES_MAX_BATCH &&
+                                 pairs <= GD_HIP_SDPA_COUNTER_SLOTS && pieces > 1u &&
+                                 (!noalloc || need <= GD_HIP_SDPA_NOALLOC_SCRATCH_BYTES);
+            const bool wanted = backend->sdpa_merge == 2 ||
+                                (backend->sdpa_merge == 1 && chunk == 0u && pairs >= (uint64_t)backend->compute_units &&
+                                 span >= 4u * GD_HIP_SDPA_PIECE_KEYS);
+            if (applies && wanted) {
+                float *ws;
+                /* 4 wavefronts per workgroup; a requested chunk is taken literally, otherwise even rows stay whole
+                 * when that leaves two workgroups per compute unit and are halved below that */
+                p.waves = 4u;
+                p.even_pieces = chunk != 0u ? 0u : (pairs >= 2u * (uint64_t)backend->compute_units ? 1u : 2u);
+                p.chunk = piece;
+                p.nsplit = pieces;
+                if (noalloc) {
+                    ws = gd_hip_sdpa_decode_scratch(backend->device);
+                    if (ws == NULL) return GD_ERR_BAD_STATE;
+                } else {
+                    st = gd_hip_reserve_attn_ws(backend, need);
+                    if (st != GD_OK) return st;
+                    ws = (float *)backend->attn_ws;
+                }
+                {
+                    const bool pfx = p.prefix_len > 0u;
+                    const uint32_t rec[12] = {4u, p.dh, group, p.waves, group == 1u ? 2u : 4u, pfx ? 0u : p.nontemporal,
+                                              pfx ? 1u : 0u, p.nsplit, p.hkv, p.batch, p.chunk, p.even_pieces};
+                    memcpy(backend->last_sdpa, rec, sizeof(rec));
+                }
+                return gd_hip_finish_op(backend, gd_hip_launch_sdpa_decode_pieces(
+                    backend->stream, gd_hip_view_ptr(q), gd_hip_view_ptr(k), gd_hip_view_ptr(v), pos_ptr,
+                    gd_hip_view_ptr(out), ws, &p));
+            }
+            p.even_pieces = 0u;
+        }
         if (chunk == 0u) {
             /* one workgroup per (batch row, kv head) as soon as that gives every compute unit one (a single pass, no
              * combine kernel: measured 6 % faster than two splits at 256 pairs x 4096 keys); below that, split the
@@ -109,7 +162,8 @@ static gd_status dispatch(gd_backend *backend, const gd_backend_tensor_view *q, 
             p.waves = (uint64_t)p.batch * p.hkv * p.nsplit >= 2u * (uint64_t)backend->compute_units ? 4u : 8u;
         float *ws = NULL;
         if (p.nsplit > 1u) {
-            const size_t need = (size_t)p.batch * p.hq * p.nsplit * (p.dh + 2u) * sizeof(float);
+            const size_t need = ((size_t)GD_HIP_SDPA_COUNTER_SLOTS +
+                                 (size_t)p.batch * p.hq * p.nsplit * (p.dh + 2u)) * sizeof(float);
             if (noalloc) {
                 /* partial results go to the fixed device array of this library; nothing is allocated */
                 ws = gd_hip_sdpa_decode_scratch(backend->device);
@@ -132,8 +186,8 @@ static gd_status dispatch(gd_backend *backend, const gd_backend_tensor_view *q, 
             const uint32_t w = pfx ? ((group == 1u && p.waves == 8u) ? 8u : 4u) : (group == 1u ? p.waves : 4u);
             const uint32_t u = pfx ? (group == 1u ? 2u : 4u)
                                    : (group == 1u ? ((p.unroll == 8u || p.unroll == 2u) ? p.unroll : 4u) : 4u);
-            const uint32_t rec[11] = {1u, p.dh, group, w, u, pfx ? 0u : p.nontemporal, pfx ? 1u : 0u,
-                                      p.nsplit, p.hkv, p.batch, p.chunk};
+            const uint32_t rec[12] = {1u, p.dh, group, w, u, pfx ? 0u : p.nontemporal, pfx ? 1u : 0u,
+                                      p.nsplit, p.hkv, p.batch, p.chunk, 0u};
             memcpy(backend->last_sdpa, rec, sizeof(rec));
         }
         return gd_hip_finish_op(backend, gd_hip_launch_sdpa_decode_split(
@@ -142,7 +196,7 @@ static gd_status dispatch(gd_backend *backend, const gd_backend_tensor_view *q, 
     }
     if ((uint64_t)p.batch * p.hq * p.tq > 0x7fffffffu) return GD_ERR_UNSUPPORTED;
     {
-        const uint32_t rec[11] = {2u, p.dh, group, 1u, 0u, 0u, 0u, p.batch * p.hq * p.tq, 1u, 1u, 0u};
+        const uint32_t rec[12] = {2u, p.dh, group, 1u, 0u, 0u, 0u, p.batch * p.hq * p.tq, 1u, 1u, 0u, 0u};
         memcpy(backend->last_sdpa, rec, sizeof(rec));
         backend->last_sdpa[5] = p.dtype;
     }
@@ -211,8 +265,14 @@ gd_status gd_backend_sdpa_decode_last_kernel(gd_backend *backend, char *out, siz
     if (backend == NULL || out == NULL || capacity == 0u) return GD_ERR_INVALID_ARGUMENT;
     r = backend->last_sdpa;
     if (r[0] == 1u)
-        snprintf(out, capacity, "gd_sdpa_decode_split_kernel<%u,%u,%u,%u,%s%s> [grid %u x %u x %u, %u keys per workgroup]",
-                 r[1], r[2], r[3], r[4], r[5] ? "true" : "false", r[6] ? ",true" : "", r[7], r[8], r[9], r[10]);
+        snprintf(out, capacity, "gd_sdpa_decode_split_kernel<%u,%u,%u,%u,%s%s> [grid %u x %u x %u, %u keys per workgroup%s]",
+                 r[1], r[2], r[3], r[4], r[5] ? "true" : "false", r[6] ? ",true" : "", r[7], r[8], r[9], r[10],
+                 r[7] > 1u ? ", combine kernel" : "");
+    else if (r[0] == 4u)
+        snprintf(out, capacity, "gd_sdpa_decode_split_kernel<%u,%u,%u,%u,%s,%s,true> [grid %u x %u x %u, pieces of %u keys, "
+                                "rows merged by the last piece%s]",
+                 r[1], r[2], r[3], r[4], r[5] ? "true" : "false", r[6] ? "true" : "false", r[8], r[9], r[7], r[10],
+                 r[11] == 1u ? ", even rows whole" : r[11] == 2u ? ", even rows halved" : "");
     else if (r[0] == 2u)
         snprintf(out, capacity, "gd_sdpa_decode_generic_kernel<%s> [grid %u]", r[5] == 1u ? "gd_half" : "float", r[7]);
     else

@@ -10,6 +10,13 @@
  * (= GD_BACKEND_SDPA_DECODE_NOALLOC_SCRATCH_BYTES of the public header) */
 #define GD_HIP_SDPA_NOALLOC_SCRATCH_BYTES (8u << 20)
 #define GD_HIP_SDPA_MAX_DEVICES 16
+/* The split-KV workspace starts with one arrival counter per (batch row, kv head) (zero between launches: the
+ * piece that merges a row puts its counter back), the partial results follow.  A row is cut into at most
+ * GD_HIP_SDPA_MAX_PIECES pieces when the last piece to arrive merges them inside the kernel. */
+#define GD_HIP_SDPA_COUNTER_SLOTS 16384u
+#define GD_HIP_SDPA_MAX_PIECES 16u
+/* rows the PIECES form handles: every lane keeps the positions of its rows in registers */
+#define GD_HIP_SDPA_PIECES_MAX_BATCH 256
 
 typedef struct gd_hip_sdpa_decode_params {
     uint32_t batch, tq, tmax, hq, hkv, dh;
@@ -23,6 +30,7 @@ typedef struct gd_hip_sdpa_decode_params {
     uint32_t waves;  /* wavefronts per workgroup of the split-KV kernel: 4 or 8 */
     uint32_t unroll; /* key-row loads in flight per lane: 4 or 8 */
     uint32_t nontemporal; /* 1: K/V loads carry the streaming hint */
+    uint32_t even_pieces; /* PIECES form: parts a row is cut into when all rows are about one length; 0: always at chunk */
 } gd_hip_sdpa_decode_params;
 
 #endif

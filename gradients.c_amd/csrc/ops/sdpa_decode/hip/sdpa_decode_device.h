@@ -36,6 +36,19 @@ __device__ __forceinline__ int gd_decode_pos(const int32_t *pos, const gd_hip_sd
     return pos[p.pos_mode == GD_HIP_SDPA_POS_VECTOR ? b : 0];
 }
 
+/* Device-scope relaxed store / load: the store is written through this XCD's L2, the load is served from behind
+ * it, so workgroups on different XCDs (whose L2s do not snoop each other) can hand data over without writing
+ * back or invalidating whole caches.  Ordering against other accesses is the caller's business. */
+__device__ __forceinline__ void gd_agent_store(float *p, float v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ float gd_agent_load(const float *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 /* ---- split-KV kernel ----------------------------------------------------------- */
 
 /* Sum over aligned groups of N (8 or 16) consecutive lanes; every lane of a group receives the total.
@@ -70,6 +83,22 @@ __device__ __forceinline__ float gd_slot_reduce(float x, OP op)
     x = op(__uint_as_float(r[0]), __uint_as_float(r[1]));
     r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
     return op(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+/* Reduction over the 64 lanes of a wavefront, every lane receives the result: swaps inside the 16-lane row, then
+ * the row and half swaps. */
+template <typename OP>
+__device__ __forceinline__ int gd_wave_reduce_i32(int x, OP op)
+{
+    typedef unsigned gd_uint2 __attribute__((ext_vector_type(2)));
+    x = op(x, __builtin_amdgcn_update_dpp(0, x, 0xB1, 0xf, 0xf, false));  /* quad_perm [1,0,3,2] */
+    x = op(x, __builtin_amdgcn_update_dpp(0, x, 0x4E, 0xf, 0xf, false));  /* quad_perm [2,3,0,1] */
+    x = op(x, __builtin_amdgcn_update_dpp(0, x, 0x141, 0xf, 0xf, false)); /* row_half_mirror */
+    x = op(x, __builtin_amdgcn_update_dpp(0, x, 0x140, 0xf, 0xf, false)); /* row_mirror */
+    gd_uint2 r = __builtin_amdgcn_permlane16_swap((unsigned)x, (unsigned)x, false, false);
+    x = op((int)r[0], (int)r[1]);
+    r = __builtin_amdgcn_permlane32_swap((unsigned)x, (unsigned)x, false, false);
+    return op((int)r[0], (int)r[1]);
 }
 
 template <int N>

@@ -48,7 +48,9 @@ def _timed(pkg, be, fns, replays=4, repeats=3):
 
 def sdpa_decode(pkg):
     """gd_backend_sdpa_decode_positions at the shapes of configs[2], [1], [3], [4] and at equal rows of the same total
-    size (what raggedness costs)."""
+    size (what raggedness costs); with cacheable and streaming K/V loads, and with the rows of a ragged batch cut into
+    pieces that the last piece to arrive merges (the dispatch's choice where it applies) or left whole, one workgroup
+    per (row, kv head)."""
     be = pkg.Backend()
     shapes = [("configs[2]: B64 H8 D64, 512 keys", 64, 8, 64, 512, None),
               ("configs[1]: B32 H8 D64, 1..4096 keys", 32, 8, 64, 4352, (1, 4097)),
@@ -74,17 +76,20 @@ def sdpa_decode(pkg):
         out = buf.alloc((B, 1, H, Dh), pkg.F16)
         pos = buf.from_numpy(lens)
         algo = int(np.sum(lens.astype(np.int64) + 1)) * H * Dh * 4 + 2 * B * H * Dh * 2 + 4 * B
-        for _ in (0,):
-            for nt in (-1, 0, 1):
+        for pieces in (1, 0):
+            for nt in ((-1, 0, 1) if pieces else (1,)):
+                be.set_tunable("sdpa_merge", pieces)
                 be.set_tunable("sdpa_nontemporal", nt)
                 fns = [(lambda kv=kv: be.sdpa_decode_positions(q, kv[0], kv[1], pos, out, 1.0 / np.sqrt(Dh)))
                        for _ in range(3) for kv in sets]   # consecutive launches read different caches
                 us = _timed(pkg, be, fns)
                 rows.append({"shape": label, "streaming_loads": {-1: "auto", 0: "off", 1: "on"}[nt],
+                             "ragged_rows_in_pieces": "dispatch's choice" if pieces else "off",
                              "kernel": be.sdpa_decode_last_kernel(), "us_per_launch": round(us, 2),
                              "gbs": round(algo / us / 1e3, 1), "frac_of_hbm_peak": round(algo / us / 1e3 / HBM_PEAK_GBS, 4),
                              "algorithmic_bytes": algo, "distinct_cache_sets": nsets})
         be.set_tunable("sdpa_nontemporal", -1)
+        be.set_tunable("sdpa_merge", 1)
         be.free(buf)
     be.close()
     print(json.dumps({"probe": "sdpa_decode", "unit": "us per launch, stream events around graph replays",
@@ -125,18 +130,22 @@ def few_row_linear(pkg, rows_list=(16, 32, 64)):
                 cpos = buf.from_numpy(rng.integers(0, Tmax, M).astype(np.int32))
                 qo = buf.alloc((M, H, D), pkg.F16)
                 kc, vc = buf.alloc((M, Tmax, H, D), pkg.F16), buf.alloc((M, Tmax, H, D), pkg.F16)
-            for wide in (0, -1):
+            # third variant: every launch reads the same copy, which then stays in the 256 MB memory-side cache: what a
+            # projection would gain if its weights had been brought there ahead of time
+            for wide, resident in ((0, False), (-1, False), (-1, True)):
                 be.set_tunable("linear_wide", wide)
+                wl = [ws[0]] * len(ws) if resident else ws
                 if epi == 2:
-                    fns = [(lambda w=w: be.fused_qkv_rope_append(x, w, b, nw, pos, cpos, qo, kc, vc, H, D, 2, 2, 1e-5)) for w in ws]
+                    fns = [(lambda w=w: be.fused_qkv_rope_append(x, w, b, nw, pos, cpos, qo, kc, vc, H, D, 2, 2, 1e-5)) for w in wl]
                 else:
                     fns = [(lambda w=w: be.fused_linear(x, w, b, r if res_on else None, nw if pro == 2 else None, y, True, 2,
-                                                        pro, 1e-5, epi)) for w in ws]
+                                                        pro, 1e-5, epi)) for w in wl]
                 us = _timed(pkg, be, fns)
                 results.append({"projection": label, "rows": M, "K": K, "N": N, "kernel_family": "stream" if wide == 0 else "wide",
+                                "weights_from": "memory-side cache (one copy re-read)" if resident else "HBM (copies rotated)",
                                 "us_per_launch": round(us, 2), "weight_gbs": round(wbytes / us / 1e3, 1),
                                 "frac_of_hbm_peak": round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4), "weight_bytes": wbytes,
-                                "weight_copies_rotated": len(ws)})
+                                "weight_copies_rotated": 1 if resident else len(ws)})
             be.set_tunable("linear_wide", -1)
     be.free(buf)
     be.close()

@@ -531,7 +531,11 @@ gd_status gd_backend_device_info(const gd_backend *backend, char *name, size_t n
  * the split-KV decode kernel (also read once from the environment variable
  * GD_HIP_SDPA_CHUNK); "sdpa_waves" (4 or 8 wavefronts per workgroup) and "sdpa_unroll" (2, 4 or 8
  * key-row loads per lane and trip) of the same kernel; "sdpa_nontemporal" (GD_HIP_SDPA_NONTEMPORAL): 1 = mark its
- * K/V loads streaming, 0 = never, -1 (default) = when the caches of the call exceed 128 MiB.  "linear_tiles" (1, 2 or 4 column tiles of 16
+ * K/V loads streaming, 0 = never, -1 (default) = when the caches of the call exceed 128 MiB; "sdpa_merge"
+ * (GD_HIP_SDPA_MERGE): the per-row-positions form over at most 256 rows can cut the rows into pieces of 256 keys
+ * (or "sdpa_chunk"), one workgroup each, and let the last piece of a row to arrive merge it, so that a ragged batch
+ * spreads over the compute units; rows of about one length stay whole: 1 (default) = where there is a (row, kv head)
+ * pair per compute unit and caches of 1024 rows or more, 0 = never, 2 = wherever the form applies.  "linear_tiles" (1, 2 or 4 column tiles of 16
  * per workgroup) and "linear_waves" (4 or 8 wavefronts sharing the K range) of the few-row projection
  * kernel (environment: GD_HIP_LINEAR_TILES, GD_HIP_LINEAR_WAVES).  "m3_simple" = 1: the MiniMax-M3 operators
  * take their per-row kernels also where the matrix-core kernels apply (head size 64, block size a multiple of 64).

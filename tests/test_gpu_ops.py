@@ -259,7 +259,9 @@ def test_decode_isolated_config_shape(backend, arena, oracle, chunk):
 def test_decode_isolated_config_full_size(backend, oracle):
     """BASELINE config 1 at its full size: B=32, H=8, DH=64, caches of 4097 rows, lengths uniform in [1, 4096]; one
     token appended per sequence (bit-exact), then the decode over L+1 keys against the oracle.  At this size (275 MB
-    of caches) the dispatch picks the 8-wavefront form with streaming loads, which no smaller case reaches."""
+    of caches) the dispatch marks the K/V loads streaming and cuts long rows into pieces that the last piece to arrive
+    merges; with that switched off it picks the 8-wavefront form, one workgroup per (row, head): neither is reached
+    by a smaller case."""
     B, H, D, Tmax = 32, 8, 64, 4097
     big = backend.buffer(640 << 20)
     try:
@@ -270,13 +272,77 @@ def test_decode_isolated_config_full_size(backend, oracle):
         backend.kv_cache_append_positions(tk, tv, tp, big.from_numpy(kn), big.from_numpy(vn))
         oracle.kv_cache_append(k0, v0, kn, vn, L)
         assert np.array_equal(_bits(tk.read()), _bits(k0)) and np.array_equal(_bits(tv.read()), _bits(v0))
-        out = big.from_numpy(np.full(q.shape, 7.0, np.float16))
-        backend.sdpa_decode_positions(big.from_numpy(q), tk, tv, tp, out, 0.125)
-        name = backend.sdpa_decode_last_kernel()
-        assert name.startswith("gd_sdpa_decode_split_kernel<64,1,8,") and ",true>" in name, name
-        _close(out.read(), oracle.sdpa_decode(q, k0, v0, L, 0.125))
+        want = oracle.sdpa_decode(q, k0, v0, L, 0.125)
+        tq = big.from_numpy(q)
+        for merge, form in ((1, "rows merged by the last piece"), (0, "<64,1,8,")):
+            out = big.from_numpy(np.full(q.shape, 7.0, np.float16))
+            backend.set_tunable("sdpa_merge", merge)
+            try:
+                backend.sdpa_decode_positions(tq, tk, tv, tp, out, 0.125)
+            finally:
+                backend.set_tunable("sdpa_merge", 1)
+            name = backend.sdpa_decode_last_kernel()
+            assert form in name and ",true>" in name, name
+            _close(out.read(), want)
     finally:
         backend.free(big)
+
+
+@pytest.mark.parametrize("H,Hkv,D", [(8, 8, 64), (16, 4, 128), (6, 3, 64)])
+def test_decode_long_rows_in_pieces_merged_in_the_kernel(backend, arena, oracle, H, Hkv, D):
+    """Rows cut into pieces whose partial results the last piece to arrive merges (one launch), against the oracle and
+    against the form with a combine kernel behind the split kernel: a ragged batch (one-key rows, full rows, a row
+    past the cache end, untouched rows, NaN behind every live range), cut at 64, 96 and 1024 keys; then the dispatch's
+    own choice on 40 x Hkv (row, head) pairs with 1100-row caches, which is the merging form when there is a pair for
+    every compute unit: ragged rows are cut at 256 keys, rows of about one length stay whole or are halved."""
+    B, Tmax = 40, 1100
+    rng = np.random.default_rng(77 + H)
+    pos = rng.integers(0, Tmax, B).astype(np.int32)
+    pos[[0, 1, 2, 3, 4, 5]] = [-1, 0, Tmax - 1, Tmax + 7, 255, 256]
+    pos[B - 1] = -5
+    q = oracle.normal_f16((B, 1, H, D), 70)
+    k, v = oracle.normal_f16((B, Tmax, Hkv, D), 71), oracle.normal_f16((B, Tmax, Hkv, D), 72)
+    kd, vd = k.copy(), v.copy()
+    for b in range(B):
+        if 0 <= pos[b] < Tmax - 1:
+            kd[b, pos[b] + 1:] = np.nan
+            vd[b, pos[b] + 1:] = np.nan
+    sentinel = np.full(q.shape, 7.0, np.float16)
+    tq, tk, tv = arena.from_numpy(q), arena.from_numpy(kd), arena.from_numpy(vd)
+    scale = 1.0 / np.sqrt(D)
+
+    def run(positions, merge, chunk, caches=None):
+        out = arena.from_numpy(sentinel)
+        ck, cv = caches or (tk, tv)
+        backend.set_tunable("sdpa_merge", merge)
+        backend.set_tunable("sdpa_chunk", chunk)
+        try:
+            backend.sdpa_decode_positions(tq, ck, cv, arena.from_numpy(positions), out, scale)
+        finally:
+            backend.set_tunable("sdpa_merge", 1)
+            backend.set_tunable("sdpa_chunk", 0)
+        return out.read(), backend.sdpa_decode_last_kernel()
+
+    want = oracle.sdpa_decode(q, k, v, pos, scale, out_init=sentinel.astype(np.float32))
+    for chunk in (64, 96, 1024):
+        merged, name = run(pos, 2, chunk)
+        assert "rows merged by the last piece" in name, name
+        combined, name = run(pos, 0, chunk)
+        assert "combine kernel" in name, name
+        for got in (merged, combined):
+            assert np.isfinite(got.astype(np.float32)).all()
+            assert (got[0] == 7.0).all() and (got[B - 1] == 7.0).all()
+            _close(got, want)
+        assert np.abs(merged.astype(np.float32) - combined.astype(np.float32)).max() < 1e-3
+    # twice in a row: the arrival counters are back at zero after a launch
+    for _ in range(2):
+        got, name = run(pos, 1, 0)
+        assert ("rows merged by the last piece" in name) == (B * Hkv >= backend.device_info()[1]), name
+        _close(got, want)
+    even = rng.integers(1000, Tmax, B).astype(np.int32)
+    even[7] = -1
+    got, _ = run(even, 1, 0, (arena.from_numpy(k), arena.from_numpy(v)))
+    _close(got, oracle.sdpa_decode(q, k, v, even, scale, out_init=sentinel.astype(np.float32)))
 
 
 @pytest.mark.parametrize("D,chunk", [(64, 0), (64, 32), (128, 0), (128, 64)])

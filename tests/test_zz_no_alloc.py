@@ -83,11 +83,13 @@ def test_noalloc_rejects_what_the_fixed_scratch_cannot_hold(backend, gda):
         pos = arena.from_numpy(np.full(B, Tmax - 1, np.int32))
         a = gda.SdpaDecodeArgs(0.1, 0, 0, 0)
         backend.set_tunable("sdpa_chunk", 32)  # 2048 splits x 16 (row, head) pairs x 130 floats = 17 MB
+        backend.set_tunable("sdpa_merge", 0)   # (rows merged inside the kernel are cut into 16 pieces at most)
         try:
             st = backend.call("gd_backend_sdpa_decode_positions_noalloc", q.view(), k.view(), v.view(), pos.view(),
                               out.view(), C.byref(a))
         finally:
             backend.set_tunable("sdpa_chunk", 0)
+            backend.set_tunable("sdpa_merge", 1)
         assert st == -2  # GD_ERR_OUT_OF_MEMORY
         assert np.all(out.read().view(np.uint16) == 0x4700)
         # bad arguments are still bad arguments
