@@ -173,6 +173,7 @@ _SIGNATURES = {
     "gd_backend_device_info": [_vp, C.c_char_p, C.c_size_t, C.POINTER(C.c_int32), C.POINTER(C.c_uint64)],
     "gd_backend_set_tunable": [_vp, C.c_char_p, C.c_int64],
     "gd_backend_sdpa_decode_last_kernel": [_vp, C.c_char_p, C.c_size_t],
+    "gd_backend_linear_last_kernel": [_vp, C.c_char_p, C.c_size_t],
 }
 _OTHER_RESTYPE = {
     "gd_backend_destroy": (None, [_vp]),
@@ -370,6 +371,11 @@ class Backend:
 
     def set_tunable(self, name, value):
         _check(lib().gd_backend_set_tunable(self.handle, name.encode(), value), "gd_backend_set_tunable")
+
+    def linear_last_kernel(self):
+        out = C.create_string_buffer(32)
+        _check(lib().gd_backend_linear_last_kernel(self.handle, out, 32), "gd_backend_linear_last_kernel")
+        return out.value.decode()
 
     def sdpa_decode_last_kernel(self):
         out = C.create_string_buffer(160)

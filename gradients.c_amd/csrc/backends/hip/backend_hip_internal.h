@@ -45,6 +45,7 @@ struct gd_backend {
     unsigned graph_launches;
     /* what the last sdpa_decode dispatch launched: 0 none, 1 split, 2 generic; D, G, W, U, streaming, prefix, grid */
     uint32_t last_sdpa[12];
+    int last_linear_family; /* GD_HIP_LINEAR_FAMILY_* of the last projection call, 0 before the first */
     /* tunables read from the environment once at creation */
     int sdpa_chunk;      /* keys per workgroup in the split-KV decode kernel (0 = automatic) */
     int sdpa_waves;      /* 4 or 8 wavefronts per workgroup (0 = default 8) */

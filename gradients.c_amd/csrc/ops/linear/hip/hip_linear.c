@@ -9,7 +9,7 @@
 int gd_hip_launch_linear(hipStream_t stream, const void *x, const void *w, const void *bias, const void *residual,
                          const void *norm_w, void *y, const gd_hip_linear_params *params, int vector_ok,
                          int kn_vector_ok, int store_vector_ok, int min_workgroups, const gd_hip_rope_epilogue *rope,
-                         int wide_mode);
+                         int wide_mode, int *family);
 
 static gd_status project_full(gd_backend *backend, const gd_backend_matrix_view *x, const gd_backend_matrix_view *w,
                               const gd_backend_vector_view *bias, const gd_backend_matrix_view *residual,
@@ -77,7 +77,8 @@ static gd_status project_full(gd_backend *backend, const gd_backend_matrix_view 
     return gd_hip_finish_op(backend, gd_hip_launch_linear(
         backend->stream, gd_hip_matrix_ptr(x), gd_hip_matrix_ptr(w), bias != NULL ? gd_hip_vector_ptr(bias) : NULL,
         residual != NULL ? gd_hip_matrix_ptr(residual) : NULL, norm_w != NULL ? gd_hip_vector_ptr(norm_w) : NULL,
-        gd_hip_matrix_ptr(y), &p, vec, kn_vec, store_vec, 2 * backend->compute_units, NULL, backend->linear_wide));
+        gd_hip_matrix_ptr(y), &p, vec, kn_vec, store_vec, 2 * backend->compute_units, NULL, backend->linear_wide,
+        &backend->last_linear_family));
 }
 
 static gd_status project(gd_backend *backend, const gd_backend_matrix_view *x, const gd_backend_matrix_view *w,
@@ -134,6 +135,7 @@ gd_status gd_backend_fused_linear(gd_backend *backend, const gd_backend_matrix_v
 }
 
 #include <math.h>
+#include <stdio.h>
 
 /* qkv projection of a decode step with the rotation and the cache append in its epilogue */
 gd_status gd_backend_fused_qkv_rope_append(gd_backend *backend, const gd_backend_matrix_view *x,
@@ -210,5 +212,15 @@ gd_status gd_backend_fused_qkv_rope_append(gd_backend *backend, const gd_backend
     return gd_hip_finish_op(backend, gd_hip_launch_linear(
         backend->stream, gd_hip_matrix_ptr(x), gd_hip_matrix_ptr(w), bias != NULL ? gd_hip_vector_ptr(bias) : NULL, NULL,
         norm_weight != NULL ? gd_hip_vector_ptr(norm_weight) : NULL, NULL, &p, 1, 0, 0, 2 * backend->compute_units, &r,
-        backend->linear_wide));
+        backend->linear_wide, &backend->last_linear_family));
+}
+
+/* Which kernel family the last projection call on this backend took: "stream", "wide", "tile" or "scalar". */
+gd_status gd_backend_linear_last_kernel(gd_backend *backend, char *out, size_t capacity)
+{
+    static const char *const names[] = {NULL, "stream", "wide", "tile", "scalar"};
+    if (backend == NULL || out == NULL || capacity == 0u) return GD_ERR_INVALID_ARGUMENT;
+    if (backend->last_linear_family < 1 || backend->last_linear_family > 4) return GD_ERR_BAD_STATE;
+    snprintf(out, capacity, "%s", names[backend->last_linear_family]);
+    return GD_OK;
 }

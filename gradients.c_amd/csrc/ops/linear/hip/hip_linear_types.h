@@ -39,6 +39,12 @@ static_assert(sizeof(gd_hip_linear_params) == 76, "the few-row kernel's argument
 _Static_assert(sizeof(gd_hip_linear_params) == 76, "the few-row kernel's arguments must stay within one 128-byte line");
 #endif
 
+/* kernel family that took a projection call */
+#define GD_HIP_LINEAR_FAMILY_STREAM 1 /* few rows, MFMA fragments from global memory (linear_stream_kernel.h) */
+#define GD_HIP_LINEAR_FAMILY_WIDE 2   /* few rows, whole-line weight stream through an LDS ring (linear_wide_kernel.h) */
+#define GD_HIP_LINEAR_FAMILY_TILE 3   /* 128 rows and more, LDS-tiled MFMA kernel (linear_tile.hip) */
+#define GD_HIP_LINEAR_FAMILY_SCALAR 4 /* unaligned operands */
+
 /* destinations of the rope + append epilogue: q [M,H,D]; caches [M,Tmax,H,D]; positions I32 [M] */
 typedef struct gd_hip_rope_epilogue {
     const int32_t *rope_pos, *cache_pos;

@@ -117,8 +117,10 @@ extern "C" int gd_hip_launch_linear(hipStream_t stream, const void *x, const voi
                                     const void *residual, const void *norm_w, void *y,
                                     const gd_hip_linear_params *params, int vector_ok, int kn_vector_ok,
                                     int store_vector_ok, int min_workgroups, const gd_hip_rope_epilogue *rope_epilogue,
-                                    int wide_mode)
+                                    int wide_mode, int *family)
 {
+    /* *family: which kernel family took the call (GD_HIP_LINEAR_FAMILY_*), for logs and tests */
+    *family = GD_HIP_LINEAR_FAMILY_STREAM;
     const gd_hip_rope_epilogue no_rope = {nullptr, nullptr, nullptr, nullptr, nullptr};
     const gd_hip_rope_epilogue &rope = rope_epilogue != nullptr ? *rope_epilogue : no_rope;
     const gd_hip_linear_params &p = *params;
@@ -129,12 +131,14 @@ extern "C" int gd_hip_launch_linear(hipStream_t stream, const void *x, const voi
     if (!vector_ok || p.K == 0 || (!p.w_is_nk && !kn_vector_ok)) {
         const uint64_t total = (uint64_t)p.M * p.N;
         gd_linear_scalar_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(xp, wp, bp, rp, np, yp, p);
+        *family = GD_HIP_LINEAR_FAMILY_SCALAR;
     } else if (p.M >= 128u && (p.w_is_nk || kn_vector_ok) && p.rope_head_dim == 0u) {
         /* matrix-core bound: LDS-tiled kernel; the 256 x 256 tile once it still gives every compute unit
          * a workgroup, the 128 x 128 tile below that */
         const uint32_t out_cols = p.swiglu_cols != 0u ? 128u : 256u; /* output columns of a 256-wide weight tile */
         const uint64_t big = (uint64_t)((p.M + 255u) / 256u) * ((p.N + out_cols - 1u) / out_cols);
         const uint32_t units = min_workgroups > 0 ? (uint32_t)min_workgroups / 2u : 256u;
+        *family = GD_HIP_LINEAR_FAMILY_TILE;
         return gd_hip_launch_linear_tile(stream, x, w, bias, residual, norm_w, y, params, big >= units, store_vector_ok, (int)units);
     } else if (wide_mode != 0 && p.w_is_nk &&
                gd_hip_try_launch_linear_wide(stream, x, w, bias, residual, norm_w, y, params, rope_epilogue,
@@ -143,6 +147,7 @@ extern "C" int gd_hip_launch_linear(hipStream_t stream, const void *x, const voi
         /* weight matrices of megabytes: the kernel built around the weight stream (wide_mode: 0 never, 1 whenever it
          * covers the call, -1 from 4 MiB of weights on; below that the launch latency decides and the stream kernel
          * is shorter) */
+        *family = GD_HIP_LINEAR_FAMILY_WIDE;
     } else {
         /* columns per workgroup: 64, 32 or 16 (rows: always 16, further rows in grid.y; their weight re-reads
          * come from L2).  More columns reuse each activation fragment for more MFMAs and repeat the prologue

@@ -552,6 +552,10 @@ gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t 
  * grid in brackets; written to out as a NUL-terminated string of at most capacity bytes.  No counterpart in the
  * reference (measurement aid: bench.py labels its roofline with it).  GD_ERR_BAD_STATE before the first call. */
 gd_status gd_backend_sdpa_decode_last_kernel(gd_backend *backend, char *out, size_t capacity);
+/* Kernel family the last projection call (matmul / linear / fused_linear / fused_qkv_rope_append) took: "stream" (few
+ * rows, fragments from global memory), "wide" (few rows over large [N,K] weights, weight stream through LDS), "tile"
+ * (128 rows and more) or "scalar" (unaligned operands).  No reference counterpart. */
+gd_status gd_backend_linear_last_kernel(gd_backend *backend, char *out, size_t capacity);
 
 /* gd_backend_sdpa_decode_positions for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same

@@ -24,6 +24,7 @@ GD_NULL_OP(gd_backend_kv_cache_append_at)
 GD_NULL_OP(gd_backend_kv_cache_append_packed)
 GD_NULL_OP(gd_backend_kv_cache_append_positions)
 GD_NULL_OP(gd_backend_linear)
+GD_NULL_OP(gd_backend_linear_last_kernel)
 GD_NULL_OP(gd_backend_linear_nt)
 GD_NULL_OP(gd_backend_matmul)
 GD_NULL_OP(gd_backend_matmul_nt)

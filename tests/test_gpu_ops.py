@@ -1168,6 +1168,74 @@ def test_few_row_projection_weight_stream_through_lds(backend, arena, oracle, gd
         _close(got[0], u)
 
 
+# (33 rows or more with the rotation take the stream kernel by design)
+@pytest.mark.parametrize("kind,K,tiles,M", [(kind, K, tiles, M) for kind in ("plain", "swiglu", "rope")
+                                            for (K, tiles) in ((1024, 0), (1536, 0), (2048, 1), (2048, 0))
+                                            for M in (5, 32, 64) if not (kind == "rope" and M == 64)])
+def test_few_row_projection_wide_kernel_forms(backend, arena, oracle, gda, M, K, tiles, kind):
+    """Every form of the kernels built around the weight stream through LDS that sits behind an rms_norm: one, two and
+    four row tiles of 16 in a workgroup (5, 32, 64 rows), K = 1024 and 1536 (one tile per workgroup), K = 2048 in the
+    one-tile form (tunable linear_tiles = 1) and in the persistent form, with the plain, gated and rotate-and-append
+    epilogues.  Against the oracle, and bit for bit against the kernel that loads its fragments straight from global
+    memory with the same eight-way split of K (same products, same order of sums)."""
+    H, D, Tmax = 4, 64, 12
+    N = {"plain": 4096 if (K, M) == (2048, 64) else 320, "swiglu": 160, "rope": 3 * H * D}[kind]
+    rows = 2 * N if kind == "swiglu" else N
+    x = oracle.normal_f16((M, K), 5200 + M + K, 1.2)
+    nw = (1.0 + 0.1 * oracle.normal_f16((K,), 5201).astype(np.float32)).astype(np.float16)
+    w = oracle.normal_f16((rows, K), 5202 + K, 0.05)
+    bias = oracle.normal_f16((rows,), 5203, 0.4)
+    tx, tw, tb, tn = (arena.from_numpy(a) for a in (x, w, bias, nw))
+    pos = oracle.uniform_i32(M, 5204, 0, 3000)
+    cpos = oracle.uniform_i32(M, 5205, 0, Tmax - 1)
+    cpos[0] = -1
+    tp, tc = arena.from_numpy(pos), arena.from_numpy(cpos)
+    k0, v0 = oracle.normal_f16((M, Tmax, H, D), 5206), oracle.normal_f16((M, Tmax, H, D), 5207)
+
+    def run(wide):
+        backend.set_tunable("linear_wide", wide)
+        backend.set_tunable("linear_tiles", tiles if wide else 0)
+        backend.set_tunable("linear_waves", 0 if wide else 8)
+        try:
+            if kind == "rope":
+                q, kc, vc = arena.alloc((M, H, D), gda.F16), arena.from_numpy(k0), arena.from_numpy(v0)
+                backend.fill(q, 0x7e00)
+                backend.fused_qkv_rope_append(tx, tw, tb, tn, tp, tc, q, kc, vc, H, D, 2, 2, 1e-5)
+                out = (q.read(), kc.read(), vc.read())
+            else:
+                y = arena.alloc((M, N), gda.F16)
+                backend.fill(y, 0x7e00)
+                backend.fused_linear(tx, tw, tb, None, tn, y, True, 2, 2, 1e-5, epilogue=1 if kind == "swiglu" else 0)
+                out = (y.read(),)
+            return out, backend.linear_last_kernel()
+        finally:
+            backend.set_tunable("linear_wide", -1)
+            backend.set_tunable("linear_tiles", 0)
+            backend.set_tunable("linear_waves", 0)
+
+    wide, family = run(1)
+    assert family == "wide", family
+    stream, family = run(0)
+    assert family == "stream", family
+    for a, b in zip(wide, stream):
+        assert np.array_equal(_bits(a), _bits(b))
+    u = oracle.linear_nt(oracle.rms_norm(x, nw, 1e-5), w, bias)
+    if kind == "plain":
+        _close(wide[0], u)
+    elif kind == "swiglu":
+        through = (np.abs(u[:, :N].astype(np.float64)) + np.abs(bias[:N].astype(np.float64))) * \
+                  (1.0 + np.abs(u[:, N:].astype(np.float64)) + np.abs(bias[N:].astype(np.float64)))
+        _close(wide[0], oracle.swiglu_split(u), through=through)
+    else:
+        qo, ko, vo = oracle.qkv_split_rope(u, pos, H, D)
+        _close(wide[0], qo, atol=4e-3)
+        for b in range(M):
+            if 0 <= cpos[b] < Tmax:
+                _close(wide[1][b, cpos[b]], ko[b], atol=4e-3)
+                _close(wide[2][b, cpos[b]], vo[b])
+        assert np.array_equal(_bits(wide[1][0]), _bits(k0[0])) and np.array_equal(_bits(wide[2][0]), _bits(v0[0]))
+
+
 @pytest.mark.parametrize("B,H,D,K", [(64, 8, 64, 512), (16, 16, 128, 2048), (5, 3, 32, 72), (33, 2, 96, 64)])
 def test_fused_qkv_rope_append_equals_separate_ops(backend, arena, oracle, gda, B, H, D, K):
     """rms_norm -> qkv projection (+F16 bias) -> rope -> cache append in one launch against the fused projection
