@@ -67,6 +67,13 @@ gd_argmax_rows_kernel(const T *__restrict__ logits, int32_t *__restrict__ ids, f
     t.second = GD_NEG_INF;
     t.idx = -1;
     const uint32_t threads = blockDim.x;
+    /* the row's step counter and position are requested here, in front of the scan, so that the pick at the end is not
+     * followed by two more dependent round trips */
+    int32_t counter = 0, position = 0;
+    if (ADVANCE && threadIdx.x == 0) {
+        counter = adv.step_counters[blockIdx.x];
+        position = adv.positions[blockIdx.x];
+    }
     uint64_t done = 0; /* columns covered by the vector part */
     if (sizeof(T) == 2 && (reinterpret_cast<uintptr_t>(row) & 15u) == 0u) {
         /* 8 halfs per lane and trip; lane-major order keeps the lowest-index rule: pushes of one lane ascend */
@@ -97,8 +104,8 @@ gd_argmax_rows_kernel(const T *__restrict__ logits, int32_t *__restrict__ ids, f
         ids[blockIdx.x] = token;
         if (gap != nullptr) gap[blockIdx.x] = g;
         if (ADVANCE) {
-            const int32_t s = adv.step_counters[blockIdx.x];
-            adv.positions[blockIdx.x] += adv.pos_delta;
+            const int32_t s = counter;
+            adv.positions[blockIdx.x] = position + adv.pos_delta;
             if (s >= 0 && (uint32_t)s < adv.max_steps) {
                 adv.out_ids[(size_t)s * gridDim.x + blockIdx.x] = token;
                 if (adv.out_gaps != nullptr) adv.out_gaps[(size_t)s * gridDim.x + blockIdx.x] = g;

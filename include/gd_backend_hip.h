@@ -559,14 +559,17 @@ gd_status gd_backend_linear_last_kernel(gd_backend *backend, char *out, size_t c
 
 /* gd_backend_sdpa_decode_positions for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
- * arguments, validation, kernels and result bits as gd_backend_sdpa_decode_positions; the split-KV partial
- * results (needed when batch * kv heads is below the number of compute units and the key range is split) go to a
- * fixed device array of GD_BACKEND_SDPA_DECODE_NOALLOC_SCRATCH_BYTES that the library holds on every GPU it runs
- * on until the process ends, instead of the backend's workspace that grows by hipMalloc.  A call whose partial
- * results (batch * q heads * splits * (head size + 2) * 4 bytes) exceed that size returns GD_ERR_OUT_OF_MEMORY
- * and prints the two sizes on stderr; nothing is launched.  The call makes no hipMalloc / hipFree and may be
- * captured.  All calls on one GPU share the array: calls that overlap on one GPU (two backends, two streams)
- * race; calls on one backend are ordered by its stream. */
+ * arguments, validation, kernels and result bits as gd_backend_sdpa_decode_positions; what the kernels keep beside
+ * inputs and outputs (64 KiB of arrival counters, then the partial results of rows that are cut: batch * q heads *
+ * pieces * (head size + 2) * 4 bytes; needed when batch * kv heads is below the number of compute units and the key
+ * range is split, and when the rows of a ragged batch are cut into pieces) goes to a fixed device array of
+ * GD_BACKEND_SDPA_DECODE_NOALLOC_SCRATCH_BYTES that the library holds on every GPU it runs on until the process
+ * ends, instead of the backend's workspace that grows by hipMalloc.  A ragged batch whose pieces would not fit is
+ * run with one workgroup per (row, kv head) instead; a split of the key range that does not fit returns
+ * GD_ERR_OUT_OF_MEMORY and prints the two sizes on stderr; nothing is launched.  The call makes no hipMalloc /
+ * hipFree and may be captured into a graph.  All calls on one GPU share the array: calls that overlap on one GPU
+ * (two backends, two streams, a graph replay next to an eager call on another stream) race; calls on one backend
+ * are ordered by its stream. */
 #define GD_BACKEND_SDPA_DECODE_NOALLOC_SCRATCH_BYTES (8u << 20)
 gd_status gd_backend_sdpa_decode_positions_noalloc(gd_backend *backend, const gd_backend_tensor_view *q,
                                                    const gd_backend_tensor_view *k_cache,

@@ -58,13 +58,78 @@ def test_noalloc_equals_the_allocating_entry_point_on_two_calls_in_a_row(backend
 
 
 def test_noalloc_without_a_split_and_generic_shapes(backend, gda, oracle):
-    """Shapes that need no partial results (one workgroup per (row, head); F32 / Tq > 1 generic kernel)."""
+    """Shapes that need no partial results: one workgroup per (row, head), and the generic kernel (F32 tensors with
+    two query tokens per row)."""
     arena = backend.buffer(256 << 20)
     try:
         pos = list(oracle.uniform_i32(64, 4400, 1, 511))
         n, r, w = _pair(backend, arena, oracle, 64, 8, 8, 64, 512, pos, 4401)
+        assert "split_kernel" in backend.sdpa_decode_last_kernel()
         assert np.array_equal(_bits(n), _bits(r))
         assert np.abs(n.astype(np.float64) - w).max() < 2e-3
+        arena.reset()
+        B, Tq, H, Hkv, D, Tmax = 3, 2, 4, 2, 40, 70
+        q = oracle.normal_f16((B, Tq, H, D), 4410).astype(np.float32)
+        k = oracle.normal_f16((B, Tmax, Hkv, D), 4411).astype(np.float32)
+        v = oracle.normal_f16((B, Tmax, Hkv, D), 4412).astype(np.float32)
+        pos = np.array([0, 33, 60], np.int32)
+        tq, tk, tv, tp = (arena.from_numpy(a) for a in (q, k, v, pos))
+        out_n, out_r = arena.from_numpy(np.zeros(q.shape, np.float32)), arena.from_numpy(np.zeros(q.shape, np.float32))
+        backend.sdpa_decode_positions_noalloc(tq, tk, tv, tp, out_n, 0.2)
+        assert "generic" in backend.sdpa_decode_last_kernel()
+        backend.sdpa_decode_positions(tq, tk, tv, tp, out_r, 0.2)
+        assert np.array_equal(out_n.read().view(np.uint32), out_r.read().view(np.uint32))
+        want = oracle.sdpa_decode(q.astype(np.float16), k.astype(np.float16), v.astype(np.float16), pos, 0.2)
+        assert np.abs(out_n.read().astype(np.float64) - want).max() < 1e-5
+    finally:
+        backend.free(arena)
+
+
+def test_noalloc_ragged_rows_in_pieces_and_under_graph_capture(backend, gda, oracle):
+    """The form that cuts the rows of a ragged batch into pieces keeps its arrival counters and partial results in
+    the fixed array too (counters are back at zero after every launch).  Then the entry point is captured into a
+    graph, as a caller that cannot allocate would use it, and replayed three times with eager calls of other sizes
+    in between: every replay must give the bits of the eager call."""
+    arena = backend.buffer(256 << 20)
+    try:
+        B, H, D, Tmax = 40, 8, 64, 1100
+        pos = oracle.uniform_i32(B, 4500, 0, Tmax - 1)
+        pos[3], pos[7] = -1, Tmax + 3
+        for _ in range(2):
+            arena.reset()
+            n, r, w = _pair(backend, arena, oracle, B, H, H, D, Tmax, pos, 4501)
+            if B * H >= backend.device_info()[1]:
+                assert "rows merged by the last piece" in backend.sdpa_decode_last_kernel()
+            assert np.array_equal(_bits(n), _bits(r))
+            assert np.abs(n.astype(np.float64) - w).max() < 2e-3
+        arena.reset()
+        # split partials (4 rows x 8 heads over 6000 keys) under capture
+        q = oracle.normal_f16((4, 1, 8, 64), 4600)
+        k, v = oracle.normal_f16((4, 6000, 8, 64), 4601), oracle.normal_f16((4, 6000, 8, 64), 4602)
+        tq, tk, tv = arena.from_numpy(q), arena.from_numpy(k), arena.from_numpy(v)
+        tp = arena.from_numpy(np.array([5999, 3000, -1, 17], np.int32))
+        eager, out = arena.from_numpy(np.full(q.shape, 7.0, np.float16)), arena.from_numpy(np.full(q.shape, 7.0, np.float16))
+        backend.sdpa_decode_positions_noalloc(tq, tk, tv, tp, eager, 0.125)
+        assert "combine kernel" in backend.sdpa_decode_last_kernel()
+        backend.scope_begin()
+        backend.graph_begin_capture()
+        backend.sdpa_decode_positions_noalloc(tq, tk, tv, tp, out, 0.125)
+        graph = backend.graph_end_capture()
+        try:
+            for i in range(3):
+                backend.fill(out, 0x4700)
+                backend.graph_launch(graph)
+                backend.fence_wait(backend.record_fence())
+                assert np.array_equal(_bits(out.read()), _bits(eager.read())), i
+                # an eager call of another size dirties the shared array between the replays
+                other = arena.from_numpy(np.zeros((2, 1, 8, 64), np.float16))
+                backend.sdpa_decode_positions_noalloc(arena.from_numpy(q[:2]), arena.from_numpy(k[:2, :3000]),
+                                                      arena.from_numpy(v[:2, :3000]),
+                                                      arena.from_numpy(np.array([2999, 100], np.int32)), other, 0.125)
+                backend.scope_begin()
+        finally:
+            backend.fence_wait(backend.record_fence())
+            backend.graph_destroy(graph)
     finally:
         backend.free(arena)
 
