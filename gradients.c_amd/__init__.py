@@ -151,6 +151,8 @@ _SIGNATURES = {
     "gd_backend_linear_nt": [_vp, _MV, _MV, _VV, _MV],
     "gd_backend_fused_linear": [_vp, _MV, _MV, _VV, _MV, _VV, _MV, C.POINTER(FusedLinearArgs)],
     "gd_backend_qkv_rope_append": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, C.c_uint32, C.c_uint32, C.POINTER(RopeArgs)],
+    "gd_backend_qkv_rope_append_packed": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, _TV, _TV, _TV, C.c_uint32, C.c_uint32,
+                                          C.POINTER(RopeArgs)],
     "gd_backend_rand_uniform": [_vp, _vp, C.c_size_t, C.c_size_t, C.c_uint32, C.c_uint64, C.c_float, C.c_float],
     "gd_backend_concat_to_full": [_vp, _TV, _TV, C.POINTER(ConcatArgs)],
     "gd_backend_gather_rows": [_vp, _TV, _TV, _TV],
@@ -466,6 +468,12 @@ class Backend:
         a = RopeArgs(theta, head_dim, 0)
         _check(self.call("gd_backend_qkv_rope_append", qkv.view(), pos.view(), cache_pos.view(), q.view(),
                          k_cache.view(), v_cache.view(), n_heads, head_dim, C.byref(a)), "gd_backend_qkv_rope_append")
+
+    def qkv_rope_append_packed(self, qkv, pos, cache_pos, cu, q, k, v, k_cache, v_cache, n_heads, head_dim, theta=10000.0):
+        a = RopeArgs(theta, head_dim, 0)
+        _check(self.call("gd_backend_qkv_rope_append_packed", qkv.view(), pos.view(), cache_pos.view(), cu.view(), q.view(),
+                         k.view(), v.view(), k_cache.view(), v_cache.view(), n_heads, head_dim, C.byref(a)),
+               "gd_backend_qkv_rope_append_packed")
 
     def fused_qkv_rope_append(self, x, w, bias, norm_weight, pos, cache_pos, q, k_cache, v_cache, n_heads, head_dim,
                               bias_mode, prologue, eps=0.0, theta=10000.0):

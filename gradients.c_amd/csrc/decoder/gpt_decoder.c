@@ -545,6 +545,7 @@ static gd_status linear_forward(gd_context *ctx, const gpt_linear *l, const gd_t
     return gd_linear(ctx, x, &l->weight, &l->bias, out);
 }
 
+static void tview(const gd_tensor *t, gd_backend_tensor_view *v);
 static gd_status fused_project_rows(gd_gpt_decoder *d, int64_t B, const gd_tensor *x, int64_t x_cols,
                                     const gpt_linear *lin, const gd_tensor *w_override, const gd_tensor *bias,
                                     const gd_tensor *residual, const gd_tensor *norm_w, uint32_t prologue,
@@ -622,8 +623,29 @@ static gd_status block_prefill(gd_gpt_decoder *d, int32_t l, const gd_tensor *x,
     int64_t flat_shape[2] = {x->shape[0], c->d_model};
     TRY(gd_rms_norm(ctx, x, &b->attn_norm_w, c->rms_eps, &normed));
     TRY(linear_forward(ctx, &b->qkv_proj, &normed, &qkv));
-    TRY(gd_qkv_split_rope(ctx, &qkv, positions, c->n_heads, c->head_dim, &rope, &q, &k, &v));
-    TRY(gd_kv_cache_append_packed(ctx, &d->k_cache[l], &d->v_cache[l], cache_positions, cu, &k, &v));
+    if ((c->head_dim % 16) == 0 && qkv.dtype == GD_DTYPE_F16) {
+        /* rotation, split and cache append in one pass over the projection: the appended rows are not read back */
+        const gd_backend_rope_args ra = {c->rope_theta, (uint32_t)c->head_dim, 0U};
+        int64_t dims[3] = {x->shape[0], c->n_heads, c->head_dim};
+        gd_backend_tensor_view vqkv, vpos, vcp, vcu, vq, vk, vv, vkc, vvc;
+        TRY(gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F16, gd_shape_make(3U, dims), 256U, &q));
+        TRY(gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F16, gd_shape_make(3U, dims), 256U, &k));
+        TRY(gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F16, gd_shape_make(3U, dims), 256U, &v));
+        tview(&qkv, &vqkv);
+        tview(positions, &vpos);
+        tview(cache_positions, &vcp);
+        tview(cu, &vcu);
+        tview(&q, &vq);
+        tview(&k, &vk);
+        tview(&v, &vv);
+        tview(&d->k_cache[l], &vkc);
+        tview(&d->v_cache[l], &vvc);
+        TRY(gd_backend_qkv_rope_append_packed(gd_context_backend(ctx), &vqkv, &vpos, &vcp, &vcu, &vq, &vk, &vv, &vkc, &vvc,
+                                              (uint32_t)c->n_heads, (uint32_t)c->head_dim, &ra));
+    } else {
+        TRY(gd_qkv_split_rope(ctx, &qkv, positions, c->n_heads, c->head_dim, &rope, &q, &k, &v));
+        TRY(gd_kv_cache_append_packed(ctx, &d->k_cache[l], &d->v_cache[l], cache_positions, cu, &k, &v));
+    }
     /* MiniMax-M3: picked blocks when the context is long enough for that to matter (reference :588-600, 918-933) */
     if (c->m3_block_size > 0 && c->m3_topk_blocks > 0 && (int64_t)c->max_seq > (int64_t)c->m3_block_size * 8 &&
         (int64_t)c->m3_block_size * c->m3_topk_blocks * 2 < (int64_t)c->max_seq) {

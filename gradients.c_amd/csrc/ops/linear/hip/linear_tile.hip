@@ -807,9 +807,41 @@ extern "C" int gd_hip_launch_linear_tile(hipStream_t stream, const void *x, cons
 {
     const gd_hip_linear_params &p = *params;
     const uint32_t units = ((uint32_t)(compute_units > 0 ? compute_units : 256) + 7u) & ~7u;
-    if (big_tiles)
-        return launch_tile<4, 4>(stream, (const gd_half *)x, (const gd_half *)w, (const gd_half *)bias,
-                                 (const gd_half *)residual, (const gd_half *)norm_w, (gd_half *)y, p, (uint32_t)vector_store, units);
-    return launch_tile<2, 2>(stream, (const gd_half *)x, (const gd_half *)w, (const gd_half *)bias,
-                             (const gd_half *)residual, (const gd_half *)norm_w, (gd_half *)y, p, (uint32_t)vector_store, 2u * units);
+    const gd_half *xp = (const gd_half *)x, *rp = (const gd_half *)residual;
+    gd_half *yp = (gd_half *)y;
+    if (big_tiles) {
+        /* The persistent workgroups walk whole rounds of 256 x 256 tiles; a last round that fills only part of the
+         * compute units costs a full tile time.  When that costs more than it would with small tiles, the rows of
+         * the last, partial round are left to a second launch with 128 x 128 tiles (rows are independent; two such
+         * workgroups fit a compute unit).  A small tile is priced at 0.35 of a big one (a quarter of the work, less
+         * reuse of the staged operands). */
+        const uint32_t out_bn = p.swiglu_cols != 0u ? 128u : 256u;
+        const uint32_t tiles_m = (p.M + 255u) / 256u, tiles_n = (p.N + out_bn - 1u) / out_bn;
+        const uint64_t tiles = (uint64_t)tiles_m * tiles_n, rem = tiles % units;
+        const uint32_t head_m = (uint32_t)((tiles - rem) / tiles_n); /* row tiles that fill whole rounds */
+        if (rem != 0u && head_m != 0u && head_m < tiles_m) {
+            const uint32_t head_rows = head_m * 256u, tail_rows = p.M - head_rows;
+            const uint64_t small = (uint64_t)((tail_rows + 127u) / 128u) * ((p.N + out_bn / 2u - 1u) / (out_bn / 2u));
+            const double whole = (double)((tiles + units - 1u) / units);
+            const double cut = (double)(((uint64_t)head_m * tiles_n + units - 1u) / units) +
+                               0.35 * (double)((small + 2u * units - 1u) / (2u * units));
+            if (cut + 0.1 < whole) {
+                gd_hip_linear_params head = p, tail = p;
+                int e;
+                head.M = head_rows;
+                tail.M = tail_rows;
+                e = launch_tile<4, 4>(stream, xp, (const gd_half *)w, (const gd_half *)bias, rp, (const gd_half *)norm_w,
+                                      yp, head, (uint32_t)vector_store, units);
+                if (e != (int)hipSuccess) return e;
+                return launch_tile<2, 2>(stream, xp + (size_t)head_rows * p.ldx, (const gd_half *)w,
+                                         (const gd_half *)bias, rp != nullptr ? rp + (size_t)head_rows * p.ldr : nullptr,
+                                         (const gd_half *)norm_w, yp + (size_t)head_rows * p.ldy, tail,
+                                         (uint32_t)vector_store, 2u * units);
+            }
+        }
+        return launch_tile<4, 4>(stream, xp, (const gd_half *)w, (const gd_half *)bias, rp, (const gd_half *)norm_w, yp, p,
+                                 (uint32_t)vector_store, units);
+    }
+    return launch_tile<2, 2>(stream, xp, (const gd_half *)w, (const gd_half *)bias, rp, (const gd_half *)norm_w, yp, p,
+                             (uint32_t)vector_store, 2u * units);
 }

@@ -397,6 +397,24 @@ gd_status gd_backend_qkv_rope_append(gd_backend *backend, const gd_backend_tenso
                                      const gd_backend_tensor_view *k_cache, const gd_backend_tensor_view *v_cache,
                                      uint32_t n_heads, uint32_t head_dim, const gd_backend_rope_args *args);
 
+/* Packed-prefill form of qkv_split_rope + kv_cache_append_packed in one launch: qkv [N, 3*H*D] of N packed tokens,
+ * q, k, v [N,H,D] as gd_backend_qkv_split_rope_forward writes them, and the rotated keys and copied values of token
+ * t of sequence b (rows cu_seqlens[b] .. cu_seqlens[b+1]) also into row cache_pos[b] + t of k_cache / v_cache
+ * [B,Tmax,H,D], under the rules of gd_backend_kv_cache_append_packed (nothing is appended unless cu_seqlens starts at
+ * 0; a sequence with a negative position or whose rows do not fit behind it keeps its caches).  Same arithmetic as
+ * the two separate operators (values bit for bit; rotated elements within one F16 unit in the last place of theirs);
+ * the appended rows are the rows written to k / v and are not read back from memory.  NeoX pairing,
+ * head_dim % 16 == 0, F16 only (GD_ERR_UNSUPPORTED otherwise: use the separate operators).  No reference counterpart
+ * (reference order of the two operators: examples/gpt_lm/gpt_lm_shared.c:896-917). */
+gd_status gd_backend_qkv_rope_append_packed(gd_backend *backend, const gd_backend_tensor_view *qkv,
+                                            const gd_backend_tensor_view *pos_ids,
+                                            const gd_backend_tensor_view *cache_pos,
+                                            const gd_backend_tensor_view *cu_seqlens, const gd_backend_tensor_view *q,
+                                            const gd_backend_tensor_view *k, const gd_backend_tensor_view *v,
+                                            const gd_backend_tensor_view *k_cache,
+                                            const gd_backend_tensor_view *v_cache, uint32_t n_heads, uint32_t head_dim,
+                                            const gd_backend_rope_args *args);
+
 /* out[i,:] = src[rows[i],:]; replaces the reference's per-sequence slice +
  * concat when the last prompt rows are selected
  * (examples/gpt_lm/gpt_lm_shared.c:1117-1169).  Row index out of range -> row

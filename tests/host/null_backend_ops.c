@@ -31,6 +31,7 @@ GD_NULL_OP(gd_backend_matmul_nt)
 GD_NULL_OP(gd_backend_minimax_m3_index_topk)
 GD_NULL_OP(gd_backend_minimax_m3_sparse_attention)
 GD_NULL_OP(gd_backend_qkv_rope_append)
+GD_NULL_OP(gd_backend_qkv_rope_append_packed)
 GD_NULL_OP(gd_backend_qkv_split_rope_forward)
 GD_NULL_OP(gd_backend_rand_uniform)
 GD_NULL_OP(gd_backend_rms_norm_forward)

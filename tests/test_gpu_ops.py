@@ -1328,6 +1328,53 @@ def test_qkv_rope_append_equals_separate_ops(backend, arena, oracle, B, H, D):
 
 # ---- sampling front end -----------------------------------------------------------------------------------------
 
+@pytest.mark.parametrize("H,D", [(8, 64), (16, 128), (3, 32)])
+def test_qkv_rope_append_packed_equals_separate_ops(backend, arena, oracle, gda, H, D):
+    """The packed-prefill form (rotation, split and append of all prompt rows in one launch) against
+    gd_backend_qkv_split_rope_forward followed by gd_backend_kv_cache_append_packed: v and the value cache bit for
+    bit, q, k and the key cache to one unit in the last place, with the append kernel's skip rules: a sequence with a negative position, one whose rows do not fit behind
+    its position, an empty sequence; then a cu_seqlens that does not start at 0 (nothing is appended)."""
+    lens = np.array([5, 0, 17, 9, 1, 30], np.int32)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    B, N, Tmax = len(lens), int(cu[-1]), 40
+    cache_pos = np.array([0, 3, 20, -1, 39, 11], np.int32)   # 17 rows behind 20 fit exactly; 30 behind 11 do not
+    qkv = oracle.normal_f16((N, 3 * H * D), 2800 + D, 1.0)
+    pos = oracle.uniform_i32(N, 2801, 0, 4000)
+    k0, v0 = oracle.normal_f16((B, Tmax, H, D), 2802), oracle.normal_f16((B, Tmax, H, D), 2803)
+    tqkv, tpos, tcp = arena.from_numpy(qkv), arena.from_numpy(pos), arena.from_numpy(cache_pos)
+    for cu_used in (cu, cu + 1):
+        tcu = arena.from_numpy(cu_used.astype(np.int32))
+        q1, k1, v1 = (arena.from_numpy(np.full((N, H, D), 7.0, np.float16)) for _ in range(3))
+        kc1, vc1 = arena.from_numpy(k0), arena.from_numpy(v0)
+        backend.qkv_rope_append_packed(tqkv, tpos, tcp, tcu, q1, k1, v1, kc1, vc1, H, D)
+        q2, k2, v2 = (arena.from_numpy(np.full((N, H, D), 7.0, np.float16)) for _ in range(3))
+        kc2, vc2 = arena.from_numpy(k0), arena.from_numpy(v0)
+        backend.qkv_split_rope_forward(tqkv, tpos, q2, k2, v2, H, D)
+        backend.kv_cache_append_packed(kc2, vc2, tcp, tcu, k2, v2)
+        # values are moved bit for bit; the rotation runs in another instantiation of the kernel, where the compiler may
+        # contract the angle arithmetic differently: one F16 unit in the last place in a few elements per thousand
+        for a, b in ((v1, v2), (vc1, vc2)):
+            assert np.array_equal(_bits(a.read()), _bits(b.read()))
+        for a, b in ((q1, q2), (k1, k2), (kc1, kc2)):
+            a, b = a.read(), b.read()
+            ulp = np.spacing(np.maximum(np.abs(a), np.abs(b)).astype(np.float16)).astype(np.float32)
+            assert np.all(np.abs(a.astype(np.float32) - b.astype(np.float32)) <= ulp)
+            assert np.count_nonzero(_bits(a) != _bits(b)) <= max(2, a.size // 300)
+        if cu_used[0] == 0:
+            got = kc1.read()
+            assert np.array_equal(_bits(got[2, 20:37]), _bits(k1.read()[cu[2]:cu[3]]))       # appended: the rows of k
+            assert np.array_equal(_bits(got[0, 0:5]), _bits(k1.read()[cu[0]:cu[1]]))
+            assert np.array_equal(_bits(got[4, 39]), _bits(k1.read()[cu[4]]))
+            assert np.array_equal(_bits(got[3]), _bits(k0[3])) and np.array_equal(_bits(got[5]), _bits(k0[5]))  # skipped
+            assert np.array_equal(_bits(got[2, :20]), _bits(k0[2, :20])) and np.array_equal(_bits(got[2, 37:]), _bits(k0[2, 37:]))
+        else:
+            assert np.array_equal(_bits(kc1.read()), _bits(k0)) and np.array_equal(_bits(vc1.read()), _bits(v0))
+    qo, ko, vo = oracle.qkv_split_rope(qkv, pos, H, D)
+    _close(q1.read(), qo, atol=4e-3)
+    _close(k1.read(), ko, atol=4e-3)
+    assert np.array_equal(_bits(v1.read()), _bits(vo))
+
+
 def _reference_sampling_step(oracle, logits, hist, hist_len, finished, rng, p, stop, H):
     """One pass of the reference's loop body over the rows (examples/gpt_lm/gpt_lm_shared.c:1606-1680 reordered as
     sample -> stop / full test -> append), with the oracle's restatement of its sampler.  Returns the new rng, the
