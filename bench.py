@@ -35,8 +35,9 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 MFMA_F16_PEAK_TFLOPS = 2500.0  # published dense F16 matrix rate
 # HBM bytes per sdpa_decode launch at this shape from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
-# profiles/sdpa_decode_config2_pmc.md (fetch scaled by the factor a 64 MiB device copy shows in the same run)
-SDPA_TRAFFIC_BYTES = 67300600
+# profiles/sdpa_decode_config2_pmc.md (fetch scaled by the factor a 64 MiB device copy shows in the same run); the
+# kernels with cacheable and with streaming loads read the same counters
+SDPA_TRAFFIC_BYTES = 67301600
 
 
 # A hardware queue's ring holds 16384 dispatch packets.  rocprofv3's queue interception has ended the profiled process
@@ -193,7 +194,10 @@ def sdpa_roofline(dec, D, pkg, iters=200):
             "distinct_cache_bytes_rotated": len(sets) * 2 * cache_bytes,
             "with_streaming_loads": {"kernel": kernel_nt, "us_per_launch": round(sec_nt * 1e6, 3),
                                      "achieved": round(algo_bytes / sec_nt / 1e9, 1),
-                                     "frac": round(algo_bytes / sec_nt / 1e9 / HBM_PEAK_GBS, 4)}}
+                                     "frac": round(algo_bytes / sec_nt / 1e9 / HBM_PEAK_GBS, 4),
+                                     "traffic": SDPA_TRAFFIC_BYTES,
+                                     "traffic_source": "counter runs of this kernel in the same profile: the same "
+                                                       "FETCH_SIZE / WRITE_SIZE as with cacheable loads"}}
 
 
 def kernel_only(pkg, launches=20, copy_mib=64):
