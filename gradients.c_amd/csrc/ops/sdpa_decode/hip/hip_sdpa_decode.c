@@ -187,7 +187,7 @@ static gd_status dispatch(gd_backend *backend, const gd_backend_tensor_view *q, 
             const uint32_t u = pfx ? (group == 1u ? 2u : 4u)
                                    : (group == 1u ? ((p.unroll == 8u || p.unroll == 2u) ? p.unroll : 4u) : 4u);
             const uint32_t rec[12] = {1u, p.dh, group, w, u, pfx ? 0u : p.nontemporal, pfx ? 1u : 0u,
-                                      p.nsplit, p.hkv, p.batch, p.chunk, 0u};
+                                      p.nsplit, p.hkv, p.batch, p.chunk, !pfx && p.window == 0u ? 1u : 0u};
             memcpy(backend->last_sdpa, rec, sizeof(rec));
         }
         return gd_hip_finish_op(backend, gd_hip_launch_sdpa_decode_split(
@@ -265,8 +265,11 @@ gd_status gd_backend_sdpa_decode_last_kernel(gd_backend *backend, char *out, siz
     if (backend == NULL || out == NULL || capacity == 0u) return GD_ERR_INVALID_ARGUMENT;
     r = backend->last_sdpa;
     if (r[0] == 1u)
+        /* template arguments as a kernel trace prints them: D, G, wavefronts, trip length, streaming loads[, prefix
+         * [, pieces, first rows requested ahead of the position]] */
         snprintf(out, capacity, "gd_sdpa_decode_split_kernel<%u,%u,%u,%u,%s%s> [grid %u x %u x %u, %u keys per workgroup%s]",
-                 r[1], r[2], r[3], r[4], r[5] ? "true" : "false", r[6] ? ",true" : "", r[7], r[8], r[9], r[10],
+                 r[1], r[2], r[3], r[4], r[5] ? "true" : "false",
+                 r[6] ? ",true" : (r[11] ? ",false,false,true" : ""), r[7], r[8], r[9], r[10],
                  r[7] > 1u ? ", combine kernel" : "");
     else if (r[0] == 4u)
         snprintf(out, capacity, "gd_sdpa_decode_split_kernel<%u,%u,%u,%u,%s,%s,true> [grid %u x %u x %u, pieces of %u keys, "

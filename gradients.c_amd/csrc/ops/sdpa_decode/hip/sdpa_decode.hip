@@ -153,14 +153,20 @@ static int launch_split(hipStream_t stream, const void *q, const void *k, const 
                         void *out, float *ws, const gd_hip_sdpa_decode_params &p)
 {
     dim3 grid(p.nsplit, p.hkv, p.batch);
-#define GD_GO(W, U)                                                                                   \
-    do {                                                                                              \
-        if (p.nontemporal)                                                                            \
-            gd_sdpa_decode_split_kernel<D, G, W, U, true><<<grid, W * 64, 0, stream>>>(                \
-                (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, pos, (gd_half *)out, ws, p); \
-        else                                                                                          \
-            gd_sdpa_decode_split_kernel<D, G, W, U, false><<<grid, W * 64, 0, stream>>>(               \
-                (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, pos, (gd_half *)out, ws, p); \
+#define GD_GO(W, U)                                                                                          \
+    do {                                                                                                     \
+        if (p.nontemporal && p.window == 0u)                                                                 \
+            gd_sdpa_decode_split_kernel<D, G, W, U, true, false, false, true><<<grid, W * 64, 0, stream>>>(   \
+                (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, pos, (gd_half *)out, ws, p);        \
+        else if (p.nontemporal)                                                                              \
+            gd_sdpa_decode_split_kernel<D, G, W, U, true><<<grid, W * 64, 0, stream>>>(                       \
+                (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, pos, (gd_half *)out, ws, p);        \
+        else if (p.window == 0u)                                                                             \
+            gd_sdpa_decode_split_kernel<D, G, W, U, false, false, false, true><<<grid, W * 64, 0, stream>>>(  \
+                (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, pos, (gd_half *)out, ws, p);        \
+        else                                                                                                 \
+            gd_sdpa_decode_split_kernel<D, G, W, U, false><<<grid, W * 64, 0, stream>>>(                      \
+                (const gd_half *)q, (const gd_half *)k, (const gd_half *)v, pos, (gd_half *)out, ws, p);        \
     } while (0)
     if (p.prefix_len > 0u) {
         /* one instantiation per wavefront count: the tunables for trip length and streaming loads do not apply */

@@ -13,7 +13,7 @@
  * runs, [0, a_len) and [b0, live); the kernel walks a virtual index over both (v < a_len: key v, else key
  * v - a_len + b0) and the split of the range counts virtual indices.  Without PFX there is one run and the index is
  * the key row itself. */
-template <int D, int G, int WAVES, int UNROLL, bool NT, bool PFX = false, bool PIECES = false>
+template <int D, int G, int WAVES, int UNROLL, bool NT, bool PFX = false, bool PIECES = false, bool AHEAD = false>
 __global__ void __launch_bounds__(WAVES * 64)
 gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__restrict__ kc,
                             const gd_half *__restrict__ vc, const int32_t *__restrict__ pos_ptr,
@@ -55,7 +55,7 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
      * the same arithmetic everywhere, so all workgroups agree): rows of about one length (the longest within 1.25
      * of the mean) are cut into p.even_pieces equal parts instead (one part: the row stays whole and nothing is
      * merged), which is the one-workgroup-per-row kernel again. */
-    int split, hkv, b, pos, chunk = (int)p.chunk;
+    int split, hkv, b, pos, pos_lane = 0, chunk = (int)p.chunk;
     if (PIECES) {
         constexpr int RS = GD_HIP_SDPA_PIECES_MAX_BATCH / 64;
         split = blockIdx.z, hkv = blockIdx.x, b = blockIdx.y;
@@ -80,9 +80,67 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
             chunk = max((((longest + (int)p.even_pieces - 1) >> (p.even_pieces >> 1)) + 31) & ~31, 32);
     } else {
         split = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z;
-        pos = gd_decode_pos(pos_ptr, p, b);
+        if (AHEAD) {
+            /* the position is requested through a lane address the compiler cannot prove uniform, so that it stays
+             * in a vector register (no wait) until the wavefront's first rows have been requested */
+            pos_lane = p.cache_pos;
+            if (p.pos_mode != GD_HIP_SDPA_POS_SCALAR) {
+                int idx = p.pos_mode == GD_HIP_SDPA_POS_VECTOR ? b : 0;
+                asm volatile("" : "+v"(idx));
+                pos_lane = pos_ptr[idx];
+            }
+            pos = 0;
+        } else {
+            pos = gd_decode_pos(pos_ptr, p, b);
+        }
     }
-    if (pos < 0) return;
+
+    /* Addresses: one scalar base per cache for this (batch row, kv head), plus a 32-bit byte offset per lane
+     * made by one 24-bit multiply-add (the host checks that tmax, the row pitch and their product fit).  The
+     * four wavefronts of a SIMD start together and share its issue slots, so every vector instruction in
+     * front of the first row loads delays all of them. */
+    const size_t slab = ((size_t)b * p.tmax * p.hkv + (size_t)hkv) * (size_t)(D * 2);
+    const unsigned char *kslab = reinterpret_cast<const unsigned char *>(kc) + slab;
+    const unsigned char *vslab = reinterpret_cast<const unsigned char *>(vc) + slab;
+    /* rows first .. first + UNROLL * KPB of the wavefront, no row past `last`: all K rows of a trip are requested
+     * before its V rows (the scores need every K row, the accumulation takes the V rows one by one) */
+    auto load_rows = [&](gd_half8 (&kv)[UNROLL], gd_half8 (&vv)[UNROLL], int s0, int last, int a_len_, int b0_)
+        __attribute__((always_inline)) {
+        uint32_t off[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            int row = min(s0 + u * KPB + slot, last);
+            if (PFX) row = row < a_len_ ? row : row - a_len_ + b0_;
+            off[u] = __umul24((uint32_t)row, pitch) + lane_off;
+        }
+        /* every cache row is read exactly once per launch: optionally mark the loads streaming */
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const gd_half8 *kp = reinterpret_cast<const gd_half8 *>(kslab + off[u]);
+            kv[u] = NT ? __builtin_nontemporal_load(kp) : *kp;
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const gd_half8 *vp = reinterpret_cast<const gd_half8 *>(vslab + off[u]);
+            vv[u] = NT ? __builtin_nontemporal_load(vp) : *vp;
+        }
+    };
+    gd_half8 kA[UNROLL], vA[UNROLL], kB[UNROLL], vB[UNROLL];
+    /* Without a window the wavefront's first rows do not depend on the row's position: they are requested here,
+     * behind the request for the position and in front of its first use, so that the two round trips overlap.  What
+     * the position then says does not exist (rows from the live length on; they lie inside the cache, so the loads
+     * are harmless) is masked in the first trip's arithmetic, values included: such rows may hold anything.  AHEAD
+     * is chosen by the launcher (no window, no prefix, not the PIECES form). */
+    constexpr bool ahead = AHEAD && !PIECES && !PFX;
+    __builtin_amdgcn_sched_barrier(0);
+    if (ahead) load_rows(kA, vA, split * chunk + wave * KPW, (int)p.tmax - 1, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (ahead) pos = __builtin_amdgcn_readfirstlane(pos_lane);
+    /* (the early exits below read a loaded register, which keeps the loads above in front of the branches) */
+    if (pos < 0) {
+        if (ahead) asm volatile("" ::"v"(kA[0]), "v"(vA[0]));
+        return;
+    }
     int live, first, a_len, b0;
     const int n_vis = visible(pos, live, first, a_len, b0);
     const int r0 = PFX ? split * chunk : first + split * chunk;
@@ -95,6 +153,7 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
     const uint32_t npieces = ((uint32_t)max(n_vis, 0) + (uint32_t)chunk - 1u) / (uint32_t)chunk;
     const bool partial = PIECES ? npieces > 1u : p.nsplit > 1u;
     if (r0 >= r1) {
+        if (ahead) asm volatile("" ::"v"(kA[0]), "v"(vA[0]));
         if (PIECES) {
             /* a piece the row does not have; the first piece of a row without a visible key stores zeros */
             if (split != 0) return;
@@ -113,45 +172,17 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
         return;
     }
 
-    /* Addresses: one scalar base per cache for this (batch row, kv head), plus a 32-bit byte offset per lane
-     * made by one 24-bit multiply-add (the host checks that tmax, the row pitch and their product fit).  The
-     * four wavefronts of a SIMD start together and share its issue slots, so every vector instruction in
-     * front of the first row loads delays all of them. */
-    const size_t slab = ((size_t)b * p.tmax * p.hkv + (size_t)hkv) * (size_t)(D * 2);
-    const unsigned char *kslab = reinterpret_cast<const unsigned char *>(kc) + slab;
-    const unsigned char *vslab = reinterpret_cast<const unsigned char *>(vc) + slab;
-
     /* Row loads of trip t+1 are issued before the arithmetic of trip t (two register buffers), so
-     * the memory pipe stays busy while the wavefront computes.  All K rows of a trip are requested before
-     * its V rows: the scores need every K row, the accumulation takes the V rows one by one.  s0: the
-     * wavefront's first row of the trip (scalar); rows past the range re-read the last row and are masked
-     * in the arithmetic. */
+     * the memory pipe stays busy while the wavefront computes.  s0: the wavefront's first row of the trip (scalar);
+     * rows past the range re-read the last row and are masked in the arithmetic. */
     auto load_trip = [&](gd_half8 (&kv)[UNROLL], gd_half8 (&vv)[UNROLL], int s0) __attribute__((always_inline)) {
-        uint32_t off[UNROLL];
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            int row = min(s0 + u * KPB + slot, r1 - 1);
-            if (PFX) row = row < a_len ? row : row - a_len + b0;
-            off[u] = __umul24((uint32_t)row, pitch) + lane_off;
-        }
-        /* every cache row is read exactly once per launch: optionally mark the loads streaming */
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const gd_half8 *kp = reinterpret_cast<const gd_half8 *>(kslab + off[u]);
-            kv[u] = NT ? __builtin_nontemporal_load(kp) : *kp;
-        }
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const gd_half8 *vp = reinterpret_cast<const gd_half8 *>(vslab + off[u]);
-            vv[u] = NT ? __builtin_nontemporal_load(vp) : *vp;
-        }
+        load_rows(kv, vv, s0, r1 - 1, a_len, b0);
     };
 
     /* trips are decided per wavefront (scalar branches), rows past the range are masked per lane */
     const int jw = r0 + wave * KPW;
     const bool any_rows = jw < r1;
-    gd_half8 kA[UNROLL], vA[UNROLL], kB[UNROLL], vB[UNROLL];
-    if (any_rows) load_trip(kA, vA, jw);
+    if (any_rows && !ahead) load_trip(kA, vA, jw);
     __builtin_amdgcn_sched_barrier(0); /* nothing below moves in front of the first loads */
 
     /* query rows of the G heads that share this kv head stay in F16: products of two halfs are
@@ -174,8 +205,16 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
         for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
     }
 
-    auto compute_trip = [&](const gd_half8 (&kv)[UNROLL], const gd_half8 (&vv)[UNROLL], int s0)
+    bool unchecked = ahead; /* the buffers hold rows that were requested before the live length was known */
+    auto compute_trip = [&](const gd_half8 (&kv)[UNROLL], const gd_half8 (&vin)[UNROLL], int s0)
         __attribute__((always_inline)) {
+        gd_half8 vv[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            vv[u] = vin[u];
+            if (unchecked && !(s0 + u * KPB + slot < r1)) vv[u] = (gd_half8)(gd_half)0.f;
+        }
+        unchecked = false;
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             /* scores of the UNROLL rows, then one rescale of the running state for all of them */

@@ -217,6 +217,13 @@ def test_decode_positions_equals_scalar_f32(backend, arena, oracle, gda):
     _close(got, oracle.sdpa_decode(q, k, v, c["cache_pos"], c["scale"]), 1e-5, 1e-6)
 
 
+def _split_kernel_args(name):
+    """Template arguments of the split-KV kernel as gd_backend_sdpa_decode_last_kernel prints them: head size, query
+    heads per kv head, wavefronts, trip length, streaming loads[, prefix[, pieces, first rows ahead of the position]]."""
+    assert name.startswith("gd_sdpa_decode_split_kernel<"), name
+    return name[name.index("<") + 1:name.index(">")].split(",")
+
+
 def _decode_case(backend, arena, oracle, B, H, Hkv, D, Tmax, pos, scale, window=0, seed=100, chunk=0):
     q = oracle.normal_f16((B, 1, H, D), seed)
     k = oracle.normal_f16((B, Tmax, Hkv, D), seed + 1)
@@ -282,7 +289,7 @@ def test_decode_isolated_config_full_size(backend, oracle):
             finally:
                 backend.set_tunable("sdpa_merge", 1)
             name = backend.sdpa_decode_last_kernel()
-            assert form in name and ",true>" in name, name
+            assert form in name and _split_kernel_args(name)[4] == "true", name
             _close(out.read(), want)
     finally:
         backend.free(big)
@@ -426,7 +433,7 @@ def test_decode_streaming_loads_give_the_same_bits(backend, arena, oracle, H, Hk
     backend.set_tunable("sdpa_waves", waves)
     try:
         plain = _decode_case(backend, arena, oracle, 8, H, Hkv, D, 300, pos, 1.0 / np.sqrt(D), seed=230 + H + D, chunk=96)
-        assert ",false>" in backend.sdpa_decode_last_kernel()
+        assert _split_kernel_args(backend.sdpa_decode_last_kernel())[4] == "false"
         backend.set_tunable("sdpa_nontemporal", 1)
         try:
             hinted = _decode_case(backend, arena, oracle, 8, H, Hkv, D, 300, pos, 1.0 / np.sqrt(D), seed=230 + H + D, chunk=96)
@@ -435,7 +442,8 @@ def test_decode_streaming_loads_give_the_same_bits(backend, arena, oracle, H, Hk
             backend.set_tunable("sdpa_nontemporal", -1)
     finally:
         backend.set_tunable("sdpa_waves", 0)
-    assert ",true>" in name and (H != Hkv or f",{waves}," in name), name
+    args = _split_kernel_args(name)
+    assert args[4] == "true" and (H != Hkv or args[2] == str(waves)) and args[-1] == "true", name   # ..., no window: first rows ahead
     assert np.array_equal(_bits(plain), _bits(hinted))
 
 
