@@ -519,3 +519,41 @@ def test_ragged_prefill_then_128_resident_steps(gda, oracle):
     finally:
         dev.close()
         ref.close()
+
+
+def test_resident_steps_over_long_ragged_caches_take_the_pieces_form(gda, oracle):
+    """Graph-replayed decode steps whose attention runs in the form that cuts long rows into pieces merged inside the
+    kernel (a (row, kv head) pair per compute unit, caches of 1024 rows or more): the default architecture with 32
+    sequences, 1100-row caches and prompts of 1..1000 tokens, 12 fused resident steps (one eager, eleven replays of the
+    captured graph: the rows' arrival counters must be back at zero after every replay).  The oracle follows five of
+    the sequences, the longest and the shortest among them, fed the device's own tokens."""
+    from gradients_c_amd import decoder as D
+    V, Dm, L, H, Dh, Hm, T, B, steps = 2048, 512, 3, 8, 64, 1536, 1100, 32, 12
+    rng = np.random.default_rng(45)
+    lens = rng.integers(1, 1001, B).astype(np.int32)
+    lens[5], lens[11] = 1, 1000
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    prompt = oracle.uniform_i32(int(cu[-1]), 4501, 0, V - 1)
+    rows = [5, 11, 0, 20, 31]
+    dev = D.GptDecoder(D.gpt_config(V, Dm, L, H, Dh, Hm, T, B, 0, False, 4500), max_prefill_tokens=int(cu[-1]))
+    ref = oracle.Decoder(V, Dm, L, H, Dh, Hm, T, len(rows), 0, 4500, False)
+    try:
+        _, first, gap0 = dev.prefill(prompt, cu, want_logits=False)
+        sub = np.concatenate([prompt[cu[r]:cu[r + 1]] for r in rows])
+        sub_cu = np.concatenate([[0], np.cumsum(lens[rows])]).astype(np.int32)
+        _, nx_r, gp_r = ref.prefill(sub, sub_cu)
+        ties = _assert_ids(first[rows], nx_r, gap0[rows], gp_r, "prefill")
+        ids, gaps, _ = dev.run_resident(first, steps)
+        name = dev.ctx.backend().sdpa_decode_last_kernel()
+        if B * H >= dev.ctx.backend().device_info()[1]:
+            assert "rows merged by the last piece" in name, name
+        tok = first[rows].copy()
+        for s in range(steps):
+            _, nx_r, gp_r = ref.step(tok)
+            ties += _assert_ids(ids[s][rows], nx_r, gaps[s][rows], gp_r, f"step {s}")
+            tok = ids[s][rows].copy()
+        assert np.array_equal(dev.positions, lens + steps)
+        print("near-ties:", ties, name)
+    finally:
+        dev.close()
+        ref.close()
