@@ -95,6 +95,15 @@ gd_status gd_backend_create_default(gd_backend **out_backend)
     const char *hv;
     if (out_backend == NULL) return GD_ERR_INVALID_ARGUMENT;
     *out_backend = NULL;
+    /* How the HIP runtime replays a captured graph is its own choice, read from the environment when it starts: from
+     * dispatch packets it recorded when the graph was instantiated (its default), or node by node through its usual
+     * launch path.  The decode step is a chain of 17 short kernels (122 at 24 layers), and on MI355X the node-by-node
+     * path ends each of them with lighter cache maintenance: 0.1082 against 0.1117 ms per step of the gpt_lm default
+     * decoder at batch 64.  So the variable is set here, in front of the process's first HIP call, unless the user
+     * has set it; if something else has started the runtime already, this has no effect and nothing breaks.
+     * GD_HIP_KEEP_GRAPH_REPLAY_MODE=1 leaves the runtime's default alone. */
+    if (getenv("DEBUG_CLR_GRAPH_PACKET_CAPTURE") == NULL && getenv("GD_HIP_KEEP_GRAPH_REPLAY_MODE") == NULL)
+        (void)setenv("DEBUG_CLR_GRAPH_PACKET_CAPTURE", "0", 0);
     if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
         (void)hipGetLastError();
         return GD_ERR_UNSUPPORTED; /* "no GPU": the reference tests skip on this status */
