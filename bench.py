@@ -676,6 +676,7 @@ def main():
                 others[name] = fn()
             except Exception as e:  # the headline line must survive a failing secondary workload; the error is reported
                 others[name] = {"error": f"{type(e).__name__}: {e}"}
+                print(f"bench.py: {name} failed: {type(e).__name__}: {e}", file=sys.stderr)
     cpu = None if a.no_cpu_baseline else cpu_baseline(oracle, shape)
 
     ms_per_step = elapsed * 1e3 / a.steps

@@ -1,8 +1,8 @@
 /*
  * The split-KV decode attention kernel of gfx950 (F16, one query token per row, head size 64 or 128), shared by
  * its two translation units: sdpa_decode.hip (one workgroup per (piece, kv head, row), a combine kernel behind it
- * when rows are cut) and sdpa_decode_pieces.hip (PIECES: persistent workgroups that walk the pieces of a ragged
- * batch and merge a row in the kernel).  Replaces the reference kernels
+ * when rows are cut) and sdpa_decode_pieces.hip (PIECES: the rows of a ragged batch in pieces, one workgroup each,
+ * merged inside the kernel by the last piece of a row to arrive).  Replaces the reference kernels
  * src/ops/sdpa_decode/metal_sdpa_decode.metal:86-175 (Tq=1 window fast path) and :177-281 (general path).
  */
 #ifndef GD_SDPA_DECODE_SPLIT_KERNEL_H
@@ -23,6 +23,9 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
     constexpr int KPW = 64 / LPK;   /* key rows per wavefront load */
     constexpr int KPB = KPW * WAVES;
     constexpr int STEP = KPB * UNROLL;
+    /* AHEAD (chosen by the launcher: no window, no prefix, not the PIECES form): the wavefront's first rows are
+     * requested before the row's position is known, see below */
+    constexpr bool ahead = AHEAD && !PIECES && !PFX;
     /* Every kernel argument this path reads is requested from the argument segment here, in one batch with
      * one wait.  Left to the compiler, each load sits in front of its first use behind the early exits, and
      * a wavefront goes through five dependent round trips before its first K/V load. */
@@ -80,7 +83,7 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
             chunk = max((((longest + (int)p.even_pieces - 1) >> (p.even_pieces >> 1)) + 31) & ~31, 32);
     } else {
         split = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z;
-        if (AHEAD) {
+        if (ahead) {
             /* the position is requested through a lane address the compiler cannot prove uniform, so that it stays
              * in a vector register (no wait) until the wavefront's first rows have been requested */
             pos_lane = p.cache_pos;
@@ -129,9 +132,7 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
     /* Without a window the wavefront's first rows do not depend on the row's position: they are requested here,
      * behind the request for the position and in front of its first use, so that the two round trips overlap.  What
      * the position then says does not exist (rows from the live length on; they lie inside the cache, so the loads
-     * are harmless) is masked in the first trip's arithmetic, values included: such rows may hold anything.  AHEAD
-     * is chosen by the launcher (no window, no prefix, not the PIECES form). */
-    constexpr bool ahead = AHEAD && !PIECES && !PFX;
+     * are harmless) is masked in the first trip's arithmetic, values included: such rows may hold anything. */
     __builtin_amdgcn_sched_barrier(0);
     if (ahead) load_rows(kA, vA, split * chunk + wave * KPW, (int)p.tmax - 1, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
