@@ -570,8 +570,10 @@ static gd_status block_tail_prefill(gd_gpt_decoder *d, const gpt_block *b, const
         TRY(linear_forward(ctx, &b->up_gate, &mlp_normed, &up_gate));
         TRY(gd_swiglu_split(ctx, &up_gate, &gated));
     }
-    return fused_project_rows(d, rows, &gated, Hm, &b->down_proj, NULL, &b->down_proj.bias, &attn_resid, NULL, 0U, 0U,
-                              Dm, out);
+    /* through the [N,K] twin of the down projection's [K,N] weight, as the decode step does: the same products and
+     * sums, and the kernel's small tiles (the rows of the last, partly filled round) are a third faster on [N,K] */
+    return fused_project_rows(d, rows, &gated, Hm, &b->down_proj, &b->down_t, &b->down_proj.bias, &attn_resid, NULL, 0U,
+                              0U, Dm, out);
 }
 
 /* attention input -> block output, shared by decode and prefill (reference :1052-1070, 941-958) */

@@ -18,7 +18,9 @@
  * slots - which the transposing LDS read can do for any choice of rows.
  *
  * Softmax in the exp2 domain: s = (q.k) * scale * log2(e), F32 throughout; probabilities are rounded to F16
- * only as the operand of the second product, the row sum accumulates the unrounded values.
+ * only as the operand of the second product, the row sum accumulates the unrounded values.  The scaling rides in
+ * the multiply-add in front of the exp2, and the running maximum of a row moves (O and the row sum rescaled) only
+ * when a block raises it by more than 8 binary orders: the result does not depend on the reference point.
  *
  * LDS layouts (16-byte chunks, CPR = D/8 per row).  K: chunk c of key row r at position c ^ (r & 15)
  * (D = 128) or c ^ ((r >> 1) & 7) (D = 64): the 16 lanes of a fragment read hit 16 different bank groups.
@@ -215,47 +217,59 @@ gd_sdpa_varlen_mfma_kernel(const gd_half *__restrict__ q, const gd_half *__restr
             }
         }
 
-        /* scale, mask, block maximum */
+        /* scale, mask, block maximum.  The scores stay unscaled in their registers: scale2 > 0, so the maximum of the
+         * raw values is the raw value of the maximum, and the scaling rides in the multiply-add in front of the exp2. */
         const bool full = jb + (int)BKEYS <= T_len &&
                           (causal ? (prefix == 0 && jb + 63 <= wi0 && (window == 0 || wi0 + 31 - jb < window))
                                   : (window == 0));
-        float mloc = GD_VL_NEG_INF;
+        float mraw = GD_VL_NEG_INF;
+        if (!full) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+            for (int t = 0; t < 2; ++t) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                float s = st[t][e] * scale2;
-                if (!full) {
+                for (int e = 0; e < 16; ++e) {
                     const int j = jb + 32 * t + 8 * (e >> 2) + 4 * (int)h + (e & 3);
                     /* plain causal attention (no window, no prefix): one comparison against min(i, T_len - 1) */
                     if (plain_causal ? j > jmax : (j >= T_len || !gd_vl_allowed(i, j, causal, window, prefix)))
-                        s = GD_VL_NEG_INF;
+                        st[t][e] = GD_VL_NEG_INF;
                 }
-                st[t][e] = s;
-                mloc = fmaxf(mloc, s);
             }
         }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) mraw = fmaxf(mraw, st[t][e]);
+        float mloc = mraw * scale2; /* -inf stays -inf */
         mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
-        const float mnew = fmaxf(m, mloc);
-        const float msafe = mnew == GD_VL_NEG_INF ? 0.f : mnew;
-        const float corr = __builtin_amdgcn_exp2f(m - msafe); /* m = -inf -> 0 */
+        /* The running maximum is only a reference point: the result does not depend on it as long as nothing
+         * overflows.  It moves (and O and the row sum are rescaled) only when some row of the wavefront has found a
+         * score more than 8 binary orders above its reference, or has none yet; until then the probabilities of a
+         * block may reach 2^8, which F16 holds with its full precision, and 64 multiplications per block are saved. */
+        const bool moves = mloc > m + 8.f || (m == GD_VL_NEG_INF && mloc != GD_VL_NEG_INF);
+        if (__builtin_amdgcn_ballot_w64(moves) != 0ull) {
+            const float mnew = fmaxf(m, mloc);
+            const float msafe_new = mnew == GD_VL_NEG_INF ? 0.f : mnew;
+            const float corr = __builtin_amdgcn_exp2f(m - msafe_new); /* m = -inf -> 0 */
+            l *= corr;
+            m = mnew;
+#pragma unroll
+            for (int t = 0; t < DTILES; ++t)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o[t][e] *= corr;
+        }
+        const float msafe = m == GD_VL_NEG_INF ? 0.f : m;
         float psum = 0.f;
         gd_half8 pf[4];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const float pe = __builtin_amdgcn_exp2f(st[t][e] - msafe);
+                const float pe = __builtin_amdgcn_exp2f(fmaf(st[t][e], scale2, -msafe));
                 psum += pe;
                 pf[2 * t + (e >> 3)][e & 7] = (gd_half)pe;
             }
         }
-        l = l * corr + psum;
-        m = mnew;
-#pragma unroll
-        for (int t = 0; t < DTILES; ++t)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) o[t][e] *= corr;
+        l += psum;
 
         /* O^T += V^T P^T: four 16-key steps, DTILES channel tiles */
 #pragma unroll
