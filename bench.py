@@ -576,6 +576,9 @@ def build_parser():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph-replay", choices=("nodes", "runtime"), default="nodes",
+                    help="how the HIP runtime replays the captured decode step: node by node through its usual launch "
+                         "path (GD_HIP_GRAPH_NODE_REPLAY=1, default here) or its own default (recorded dispatch packets)")
     ap.add_argument("--batches", type=int, default=0,
                     help="how many times the K steps are timed (the median batch is reported); default 5 for the headline "
                          "line, 3 for --workload 3.  Kernel traces use --batches 1: a profiled run that would "
@@ -611,6 +614,11 @@ def main():
                  "weight replica on a single device (sequences are independent, so more GPUs would only add "
                  "replicas); run with --gpus 1")
     refuse_if_profiled_run_would_wrap_the_queue(a)
+    # graphs replayed node by node (the library's GD_HIP_GRAPH_NODE_REPLAY=1: it sets the HIP runtime's
+    # DEBUG_CLR_GRAPH_PACKET_CAPTURE=0 in front of the first HIP call): +3.3 % on the 17-kernel step of the headline,
+    # nothing at the 24-layer decoders, -11 % on the batch-1 step.  --graph-replay runtime keeps the runtime's default.
+    if a.graph_replay == "nodes":
+        os.environ.setdefault("GD_HIP_GRAPH_NODE_REPLAY", "1")
     pkg, oracle = _package()
     pkg.lib()
     if a.kernel_only:
@@ -689,6 +697,8 @@ def main():
                                "uniform random ids, full stack incl. greedy argmax, device-resident token feedback",
                    "batch": B, "cache_tokens": T, "sdpa_window": 0, "prefill_seconds": round(prefill_s, 3),
                    "timed_batches": batches, "reported": "median batch",
+                   "graph_replay": "node by node (GD_HIP_GRAPH_NODE_REPLAY=1)" if os.environ.get("GD_HIP_GRAPH_NODE_REPLAY") == "1"
+                                   else "runtime default",
                    "ms_per_step_of_each_batch": [round(t * 1e3 / a.steps, 5) for t in times]},
         "roofline": roof, "cpu_baseline": cpu, "others": others,
     }

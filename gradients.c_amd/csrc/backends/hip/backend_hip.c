@@ -99,11 +99,15 @@ gd_status gd_backend_create_default(gd_backend **out_backend)
      * dispatch packets it recorded when the graph was instantiated (its default), or node by node through its usual
      * launch path.  The decode step is a chain of 17 short kernels (122 at 24 layers), and on MI355X the node-by-node
      * path ends each of them with lighter cache maintenance: 0.1082 against 0.1117 ms per step of the gpt_lm default
-     * decoder at batch 64.  So the variable is set here, in front of the process's first HIP call, unless the user
-     * has set it; if something else has started the runtime already, this has no effect and nothing breaks.
-     * GD_HIP_KEEP_GRAPH_REPLAY_MODE=1 leaves the runtime's default alone. */
-    if (getenv("DEBUG_CLR_GRAPH_PACKET_CAPTURE") == NULL && getenv("GD_HIP_KEEP_GRAPH_REPLAY_MODE") == NULL)
-        (void)setenv("DEBUG_CLR_GRAPH_PACKET_CAPTURE", "0", 0);
+     * decoder at batch 64, while a batch-1 step becomes host-bound (79.5 against 70.6 us).  A process that wants it
+     * says so with GD_HIP_GRAPH_NODE_REPLAY=1: the runtime's variable is then set here, in front of the process's
+     * first HIP call, unless the user has set it; if something else has started the runtime already, this has no
+     * effect and nothing breaks.  Without the request the runtime's default stays. */
+    {
+        const char *want = getenv("GD_HIP_GRAPH_NODE_REPLAY");
+        if (want != NULL && want[0] == '1' && want[1] == '\0' && getenv("DEBUG_CLR_GRAPH_PACKET_CAPTURE") == NULL)
+            (void)setenv("DEBUG_CLR_GRAPH_PACKET_CAPTURE", "0", 0);
+    }
     if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
         (void)hipGetLastError();
         return GD_ERR_UNSUPPORTED; /* "no GPU": the reference tests skip on this status */

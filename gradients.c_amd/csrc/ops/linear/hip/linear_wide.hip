@@ -34,7 +34,7 @@ static void launch_wide_half(hipStream_t stream, const void *x, const void *w, c
 template <int NT, int MT, int EPI>
 static void launch_persistent(hipStream_t stream, const void *x, const void *w, const void *bias, const void *residual,
                               const void *norm_w, void *y, const gd_hip_linear_params &p, const gd_hip_rope_epilogue &rope,
-                              uint32_t units)
+                              uint32_t units, bool narrow)
 {
     constexpr bool PAIRED = EPI != GD_WIDE_EPI_PLAIN;
     /* as deep as LDS allows next to the sums of the wavefronts (NT x MT x 8 KB): 8 x RING x 2 KB; an eighth group for
@@ -42,13 +42,20 @@ static void launch_persistent(hipStream_t stream, const void *x, const void *w, 
     constexpr int RING = NT * MT <= 4 ? 7 : 5;
     const uint32_t cols = PAIRED ? 8u * NT : 16u * NT;
     const uint32_t outs = EPI == GD_WIDE_EPI_ROPE ? p.N / 2u : (EPI == GD_WIDE_EPI_SWIGLU ? p.swiglu_cols : p.N);
-    const uint32_t n_tiles = outs / cols;
+    uint32_t n_tiles = outs / cols, tile_w = cols;
+    /* fewer full tiles than compute units (5632 gated outputs: 176 tiles of 32): narrower tiles, one per unit, so
+     * that every unit streams its share of the weights (22 columns each).  Not for the rope epilogue, whose tiles
+     * must not straddle heads. */
+    if (EPI != GD_WIDE_EPI_ROPE && n_tiles < units && narrow && 2u * ((outs + units - 1u) / units) > cols) {
+        tile_w = (outs + units - 1u) / units; /* more than half of a tile's columns stay in use */
+        n_tiles = (outs + tile_w - 1u) / tile_w;
+    }
     uint32_t groups = n_tiles < units ? n_tiles : units;
     if ((n_tiles + groups - 1u) / groups > 8u) groups = (n_tiles + 7u) / 8u;
     dim3 grid(groups, (p.M + 16u * MT - 1u) / (16u * MT));
     gd_linear_wide_persistent_kernel<NT, MT, 4, RING, EPI, 8><<<grid, 512, 0, stream>>>(
         (const gd_half *)x, (const gd_half *)w, (const gd_half *)bias, (const gd_half *)residual,
-        (const gd_half *)norm_w, (gd_half *)y, p, n_tiles, rope);
+        (const gd_half *)norm_w, (gd_half *)y, p, n_tiles, tile_w, rope);
 }
 
 /* Returns 1 when the launch was taken (hipGetLastError() then tells how it went), 0 when this kernel family does
@@ -97,7 +104,7 @@ extern "C" int gd_hip_try_launch_linear_wide(hipStream_t stream, const void *x, 
     if (p.prologue != GD_HIP_PRO_RMS_NORM || ppw > 4u) return 0;
     /* K = 2048: the persistent form, where its LDS holds the sums of MT x NT tiles next to the ring */
 #define GD_P(NT, MT, EPI) \
-    do { launch_persistent<NT, MT, EPI>(stream, x, w, bias, residual, norm_w, y, p, rope, units); return 1; } while (0)
+    do { launch_persistent<NT, MT, EPI>(stream, x, w, bias, residual, norm_w, y, p, rope, units, tiles != 4u); return 1; } while (0)
     if (p.K == 2048u && persistent) {
         if (epi == GD_WIDE_EPI_PLAIN && (p.N % 64u) == 0u && mt <= 2u) {
             if (mt == 1u) GD_P(4, 1, GD_WIDE_EPI_PLAIN);

@@ -510,7 +510,7 @@ __global__ void __launch_bounds__(512)
 gd_linear_wide_persistent_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__ w,
                                  const gd_half *__restrict__ bias, const gd_half *__restrict__ residual,
                                  const gd_half *__restrict__ norm_w, gd_half *__restrict__ y, gd_hip_linear_params p,
-                                 uint32_t n_tiles, gd_hip_rope_epilogue rope)
+                                 uint32_t n_tiles, uint32_t tile_w, gd_hip_rope_epilogue rope)
 {
     constexpr int WAVES = 8;
     constexpr int SMAX = 2 * PMAX;
@@ -539,9 +539,18 @@ gd_linear_wide_persistent_kernel(const gd_half *__restrict__ x, const gd_half *_
     const int tiles = (int)(t_end - t_begin);
     const uint32_t pair_offset = EPI == GD_WIDE_EPI_ROPE ? p.rope_head_dim / 2u : (EPI == GD_WIDE_EPI_SWIGLU ? p.swiglu_cols : 0u);
     const uint32_t per_head = EPI == GD_WIDE_EPI_ROPE ? (p.rope_head_dim / 2u) / OUT_COLS : 1u;
+    /* Tiles are tile_w output columns apart (rope: always OUT_COLS).  With fewer full tiles than compute units the
+     * host makes them narrower (tile_w = ceil(outputs / units) < OUT_COLS), so that every unit streams its share of
+     * the weights: a tile then uses the first tile_w of its OUT_COLS columns; the others repeat the last used weight
+     * row (same cache lines: no traffic) and are not stored. */
+    const uint32_t outs = EPI == GD_WIDE_EPI_ROPE ? p.N / 2u : (EPI == GD_WIDE_EPI_SWIGLU ? p.swiglu_cols : p.N);
     auto tile_n0 = [&](uint32_t tile) __attribute__((always_inline)) -> uint32_t {
         if (EPI == GD_WIDE_EPI_ROPE) return (tile / per_head) * p.rope_head_dim + (tile % per_head) * OUT_COLS;
-        return tile * OUT_COLS;
+        return tile * tile_w;
+    };
+    auto tile_valid = [&](uint32_t n0) __attribute__((always_inline)) -> uint32_t {
+        if (EPI == GD_WIDE_EPI_ROPE) return OUT_COLS;
+        return min(tile_w, outs - n0);
     };
     const uint32_t m0 = blockIdx.y * (16u * MT);
 
@@ -559,7 +568,9 @@ gd_linear_wide_persistent_kernel(const gd_half *__restrict__ x, const gd_half *_
     auto issue_group = [&](int gi, int slot) __attribute__((always_inline)) {
         const int ti = gi / NG, g = gi % NG, pair = g / NT, j = g % NT;
         const uint32_t n0 = tile_n0(t_begin + (uint32_t)ti);
-        const uint32_t nbase = (PAIRED && j >= NT / 2) ? pair_offset + n0 + 16u * (uint32_t)(j - NT / 2) : n0 + 16u * (uint32_t)j;
+        const uint32_t nbase = (PAIRED && j >= NT / 2) ? pair_offset + n0 : n0;
+        const uint32_t jc = 16u * (uint32_t)((PAIRED && j >= NT / 2) ? j - NT / 2 : j); /* first column of the column tile */
+        const uint32_t last = tile_valid(n0) - 1u;
         /* the base is the same in every lane; said explicitly, it stays in scalar registers inside the tile loop */
         const uint64_t sp = (uint64_t)(uintptr_t)(wb + (size_t)pair * 128u);
         /* (the builtin returns a signed int: through uint32_t, or a low half with its top bit set would sign-extend
@@ -568,8 +579,8 @@ gd_linear_wide_persistent_kernel(const gd_half *__restrict__ x, const gd_half *_
             ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(sp >> 32)) << 32) |
             (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)sp));
         const uint32_t a = __builtin_amdgcn_readfirstlane(ring_base + (uint32_t)slot * 2048u);
-        gd_lin_load_lds16(src, (nbase + lrow[0]) * p.ldw * 2u + lchunk, a);
-        gd_lin_load_lds16(src, (nbase + lrow[1]) * p.ldw * 2u + lchunk, a + 1024u);
+        gd_lin_load_lds16(src, (nbase + min(jc + lrow[0], last)) * p.ldw * 2u + lchunk, a);
+        gd_lin_load_lds16(src, (nbase + min(jc + lrow[1], last)) * p.ldw * 2u + lchunk, a + 1024u);
     };
     /* ---- requested in front of the ring and counted by hand (gd_wide_request16): the bias values and positions of
      *      all tiles of this workgroup (TPW * OUT_COLS <= 512: at most one column per thread) and the activation
@@ -578,7 +589,8 @@ gd_linear_wide_persistent_kernel(const gd_half *__restrict__ x, const gd_half *_
     static_assert(TPW * OUT_COLS <= 512, "one bias column per thread");
     uint32_t rq_b1 = 0u, rq_b2 = 0u, rq_pos = 0u, rq_cpos = 0u;
     const bool has_col = (int)threadIdx.x < tiles * (int)OUT_COLS;
-    const uint32_t b_col = tile_n0(t_begin + (has_col ? threadIdx.x / OUT_COLS : 0u)) + threadIdx.x % OUT_COLS;
+    const uint32_t b_n0 = tile_n0(t_begin + (has_col ? threadIdx.x / OUT_COLS : 0u));
+    const uint32_t b_col = b_n0 + min(threadIdx.x % OUT_COLS, tile_valid(b_n0) - 1u);
     if (p.epilogue != GD_HIP_EPI_NONE) {
         rq_b1 = gd_wide_request2(bias, b_col * 2u);
         if (PAIRED) rq_b2 = gd_wide_request2(bias, (pair_offset + b_col) * 2u);
@@ -714,12 +726,14 @@ gd_linear_wide_persistent_kernel(const gd_half *__restrict__ x, const gd_half *_
                 *reinterpret_cast<gd_float4 *>(s_sum + (((wave * MT + mt) * NT + j) * 64 + lane) * 4) = acc[mt][j];
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         const uint32_t n0 = tile_n0(t_begin + (uint32_t)ti);
+        const uint32_t valid = tile_valid(n0);
 #pragma unroll
         for (int i = 0; i < EPT; ++i) {
             const int idx = (int)threadIdx.x + 512 * i;
             const int jj = idx >> 8, mt = jj / NTO, j = jj % NTO, rl = idx & 63, rr = (idx >> 6) & 3;
             if (jj >= NTO * MT) continue;
             const uint32_t col = n0 + 16u * j + (rl & 15);
+            const bool col_used = 16u * (uint32_t)j + (uint32_t)(rl & 15) < valid;
             const uint32_t lrow_i = 16u * mt + 4u * (rl >> 4) + rr, row = m0 + lrow_i;
             float v1 = 0.f, v2 = 0.f;
 #pragma unroll
@@ -727,7 +741,7 @@ gd_linear_wide_persistent_kernel(const gd_half *__restrict__ x, const gd_half *_
                 v1 += s_sum[(((wv * MT + mt) * NT + j) * 64 + rl) * 4 + rr];
                 if (PAIRED) v2 += s_sum[(((wv * MT + mt) * NT + j + NT / 2) * 64 + rl) * 4 + rr];
             }
-            if (row >= p.M) continue;
+            if (row >= p.M || !col_used) continue;
             const gd_half b1 = s_bias[0][ti * (int)OUT_COLS + 16 * j + (rl & 15)];
             const gd_half b2 = s_bias[1][ti * (int)OUT_COLS + 16 * j + (rl & 15)];
             gd_half h1, h2 = (gd_half)0.f;

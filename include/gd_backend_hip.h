@@ -560,6 +560,8 @@ gd_status gd_backend_device_info(const gd_backend *backend, char *name, size_t n
  * "linear_wide" (GD_HIP_LINEAR_WIDE): the kernel built around the weight stream for few-row projections over [N,K]
  * weights (whole-line loads through an LDS ring, every row tile of up to 64 rows in one workgroup): 1 = wherever it
  * covers the call, 0 = never, -1 (default) = from 4 MiB of weights on.
+ * "linear_tiles" = 4 also keeps the persistent form of those kernels on full-width column tiles where it would
+ * otherwise deal an output with fewer full tiles than compute units out in narrower ones (same results to the bit).
  * "linear_no_lds_stream" = 1: the few-row projection always loads its weight fragments straight into registers,
  * also where it would stage the weight stream through LDS (same results to the bit; for comparing the two).
  * Unknown name -> GD_ERR_INVALID_ARGUMENT. */

@@ -42,7 +42,7 @@ def test_greedy_text_equals_the_reference_generation(gda):
     assert (top2[:, 1] - top2[:, 0]).min() > 0.1          # no near-tie in the reference run: ids must be identical
     rc, out, err = run("--checkpoint", CKPT, "--tokenizer-path", VOCAB, "--prompt", "the quick brown fox",
                        "--max-new-tokens", "12", "--ids")
-    assert rc == 0, err
+    assert rc == 0, (rc, err, out[-400:])
     ids, text = parse(out)
     assert ids == ref_ids.tolist()
     tok = T.Tokenizer(VOCAB, 1, 1)
@@ -56,7 +56,7 @@ def test_sampled_run_equals_the_library_call(gda):
             "--max-new-tokens", "20", "--temperature", "0.9", "--min-p", "0.02", "--repetition-penalty", "1.2",
             "--logits-softcap", "15", "--seed", "5", "--ids")
     rc, out, err = run(*args)
-    assert rc == 0, err
+    assert rc == 0, (rc, err, out[-400:])
     ids, text = parse(out)
     tok = T.Tokenizer(VOCAB, 1, 1)
     prompt = tok.encode("hello <eot> 123 tokenizer test")

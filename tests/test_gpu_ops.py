@@ -1176,6 +1176,49 @@ def test_few_row_projection_weight_stream_through_lds(backend, arena, oracle, gd
         _close(got[0], u)
 
 
+@pytest.mark.parametrize("kind,N,M", [("swiglu", 5632, 16), ("swiglu", 5632, 32), ("plain", 12288, 16), ("plain", 12288, 32)])
+def test_few_row_projection_narrow_tiles_fill_every_compute_unit(backend, arena, oracle, gda, kind, N, M):
+    """Outputs with fewer full column tiles than compute units (5632 gated columns: 176 tiles of 32) are dealt out in
+    narrower tiles, one per compute unit (22 columns each), whose unused columns repeat the last weight row and are not
+    stored.  Same bits as the full-width tiles (tunable linear_tiles = 4) and as the stream kernel; nothing is written
+    outside the output."""
+    K = 2048
+    rows = 2 * N if kind == "swiglu" else N
+    x = oracle.normal_f16((M, K), 5300 + M, 1.2)
+    nw = (1.0 + 0.1 * oracle.normal_f16((K,), 5301).astype(np.float32)).astype(np.float16)
+    w = oracle.normal_f16((rows, K), 5302, 0.05)
+    bias = oracle.normal_f16((rows,), 5303, 0.4)
+    tx, tw, tb, tn = (arena.from_numpy(a) for a in (x, w, bias, nw))
+    got = {}
+    try:
+        for name, wide, tiles in (("narrow", 1, 0), ("full", 1, 4), ("stream", 0, 0)):
+            backend.set_tunable("linear_wide", wide)
+            backend.set_tunable("linear_tiles", tiles)
+            backend.set_tunable("linear_waves", 0 if wide else 8)
+            y = arena.alloc((M, N), gda.F16)
+            behind = arena.alloc((8192,), gda.F16)  # whatever is written past the output lands here
+            backend.fill(y, 0x7e00)
+            backend.fill(behind, 0x7e00)
+            backend.fused_linear(tx, tw, tb, None, tn, y, True, 2, 2, 1e-5, epilogue=1 if kind == "swiglu" else 0)
+            got[name] = y.read()
+            assert backend.linear_last_kernel() == ("wide" if wide else "stream")
+            assert np.all(_bits(behind.read()) == 0x7e00), name
+    finally:
+        backend.set_tunable("linear_wide", -1)
+        backend.set_tunable("linear_tiles", 0)
+        backend.set_tunable("linear_waves", 0)
+    assert not np.isnan(got["narrow"].astype(np.float32)).any()
+    assert np.array_equal(_bits(got["narrow"]), _bits(got["full"]))
+    assert np.array_equal(_bits(got["narrow"]), _bits(got["stream"]))
+    u = oracle.linear_nt(oracle.rms_norm(x, nw, 1e-5), w, bias)
+    if kind == "plain":
+        _close(got["narrow"], u)
+    else:
+        through = (np.abs(u[:, :N].astype(np.float64)) + np.abs(bias[:N].astype(np.float64))) * \
+                  (1.0 + np.abs(u[:, N:].astype(np.float64)) + np.abs(bias[N:].astype(np.float64)))
+        _close(got["narrow"], oracle.swiglu_split(u), through=through)
+
+
 # (33 rows or more with the rotation take the stream kernel by design)
 @pytest.mark.parametrize("kind,K,tiles,M", [(kind, K, tiles, M) for kind in ("plain", "swiglu", "rope")
                                             for (K, tiles) in ((1024, 0), (1536, 0), (2048, 1), (2048, 0))
