@@ -44,9 +44,11 @@ static void launch_persistent(hipStream_t stream, const void *x, const void *w, 
     const uint32_t outs = EPI == GD_WIDE_EPI_ROPE ? p.N / 2u : (EPI == GD_WIDE_EPI_SWIGLU ? p.swiglu_cols : p.N);
     uint32_t n_tiles = outs / cols, tile_w = cols;
     /* fewer full tiles than compute units (5632 gated outputs: 176 tiles of 32): narrower tiles, one per unit, so
-     * that every unit streams its share of the weights (22 columns each).  Not for the rope epilogue, whose tiles
-     * must not straddle heads. */
-    if (EPI != GD_WIDE_EPI_ROPE && n_tiles < units && narrow && 2u * ((outs + units - 1u) / units) > cols) {
+     * that every unit streams its share of the weights (22 columns each; the 3072 rotation pairs of a 6144-row qkv
+     * weight: 12 pairs each).  Narrow rope tiles straddle heads: only when half the head size is a power of two. */
+    const uint32_t hd2 = p.rope_head_dim / 2u;
+    const bool may_straddle = EPI != GD_WIDE_EPI_ROPE || (hd2 != 0u && (hd2 & (hd2 - 1u)) == 0u);
+    if (may_straddle && n_tiles < units && narrow && 2u * ((outs + units - 1u) / units) > cols) {
         tile_w = (outs + units - 1u) / units; /* more than half of a tile's columns stay in use */
         n_tiles = (outs + tile_w - 1u) / tile_w;
     }

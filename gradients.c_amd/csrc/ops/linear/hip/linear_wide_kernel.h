@@ -538,20 +538,24 @@ gd_linear_wide_persistent_kernel(const gd_half *__restrict__ x, const gd_half *_
     const uint32_t t_end = (uint32_t)(((uint64_t)(blockIdx.x + 1u) * n_tiles) / gridDim.x);
     const int tiles = (int)(t_end - t_begin);
     const uint32_t pair_offset = EPI == GD_WIDE_EPI_ROPE ? p.rope_head_dim / 2u : (EPI == GD_WIDE_EPI_SWIGLU ? p.swiglu_cols : 0u);
-    const uint32_t per_head = EPI == GD_WIDE_EPI_ROPE ? (p.rope_head_dim / 2u) / OUT_COLS : 1u;
-    /* Tiles are tile_w output columns apart (rope: always OUT_COLS).  With fewer full tiles than compute units the
-     * host makes them narrower (tile_w = ceil(outputs / units) < OUT_COLS), so that every unit streams its share of
-     * the weights: a tile then uses the first tile_w of its OUT_COLS columns; the others repeat the last used weight
-     * row (same cache lines: no traffic) and are not stored. */
+    /* Outputs are numbered 0 .. outs-1: output columns (plain), gated columns (swiglu: value row o, gate row
+     * swiglu_cols + o) or rotation pairs (rope: pair o of the q, k, v sections lies in weight rows first_row(o) and
+     * first_row(o) + D/2).  Tile t covers outputs t * tile_w .. + tile_w - 1.  tile_w is OUT_COLS, or, when that would
+     * give fewer tiles than compute units, what the host makes it (ceil(outs / units)), so that every unit streams its
+     * share of the weights: a narrow tile uses the first tile_w of its OUT_COLS columns; the others repeat the last
+     * used weight row (same cache lines: no traffic) and are not stored.  Narrow rope tiles may straddle heads, so
+     * the row of a pair is computed per lane (the host narrows them only when D/2 is a power of two). */
     const uint32_t outs = EPI == GD_WIDE_EPI_ROPE ? p.N / 2u : (EPI == GD_WIDE_EPI_SWIGLU ? p.swiglu_cols : p.N);
-    auto tile_n0 = [&](uint32_t tile) __attribute__((always_inline)) -> uint32_t {
-        if (EPI == GD_WIDE_EPI_ROPE) return (tile / per_head) * p.rope_head_dim + (tile % per_head) * OUT_COLS;
-        return tile * tile_w;
+    const uint32_t hd2 = EPI == GD_WIDE_EPI_ROPE ? p.rope_head_dim / 2u : 1u;
+    const bool hd2_pow2 = (hd2 & (hd2 - 1u)) == 0u;
+    const uint32_t hd2_shift = 31u - (uint32_t)__builtin_clz(hd2);
+    auto first_row = [&](uint32_t o) __attribute__((always_inline)) -> uint32_t {
+        if (EPI != GD_WIDE_EPI_ROPE) return o;
+        if (hd2_pow2) return ((o >> hd2_shift) << (hd2_shift + 1u)) | (o & (hd2 - 1u));
+        return (o / hd2) * p.rope_head_dim + o % hd2;
     };
-    auto tile_valid = [&](uint32_t n0) __attribute__((always_inline)) -> uint32_t {
-        if (EPI == GD_WIDE_EPI_ROPE) return OUT_COLS;
-        return min(tile_w, outs - n0);
-    };
+    auto tile_o0 = [&](uint32_t tile) __attribute__((always_inline)) -> uint32_t { return tile * tile_w; };
+    auto tile_valid = [&](uint32_t o0) __attribute__((always_inline)) -> uint32_t { return min(tile_w, outs - o0); };
     const uint32_t m0 = blockIdx.y * (16u * MT);
 
     /* ---- the weight stream: group = (tile, pair, column tile), two instructions of 8 rows x 128 bytes ---- */
@@ -567,10 +571,10 @@ gd_linear_wide_persistent_kernel(const gd_half *__restrict__ x, const gd_half *_
     /* requests group number `gi` of the wavefront's stream (gi = tile_index * NG + pair * NT + j) into ring slot */
     auto issue_group = [&](int gi, int slot) __attribute__((always_inline)) {
         const int ti = gi / NG, g = gi % NG, pair = g / NT, j = g % NT;
-        const uint32_t n0 = tile_n0(t_begin + (uint32_t)ti);
-        const uint32_t nbase = (PAIRED && j >= NT / 2) ? pair_offset + n0 : n0;
+        const uint32_t o0 = tile_o0(t_begin + (uint32_t)ti);
+        const uint32_t nbase = (PAIRED && j >= NT / 2) ? pair_offset : 0u;
         const uint32_t jc = 16u * (uint32_t)((PAIRED && j >= NT / 2) ? j - NT / 2 : j); /* first column of the column tile */
-        const uint32_t last = tile_valid(n0) - 1u;
+        const uint32_t last = tile_valid(o0) - 1u;
         /* the base is the same in every lane; said explicitly, it stays in scalar registers inside the tile loop */
         const uint64_t sp = (uint64_t)(uintptr_t)(wb + (size_t)pair * 128u);
         /* (the builtin returns a signed int: through uint32_t, or a low half with its top bit set would sign-extend
@@ -579,8 +583,8 @@ gd_linear_wide_persistent_kernel(const gd_half *__restrict__ x, const gd_half *_
             ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(sp >> 32)) << 32) |
             (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)sp));
         const uint32_t a = __builtin_amdgcn_readfirstlane(ring_base + (uint32_t)slot * 2048u);
-        gd_lin_load_lds16(src, (nbase + min(jc + lrow[0], last)) * p.ldw * 2u + lchunk, a);
-        gd_lin_load_lds16(src, (nbase + min(jc + lrow[1], last)) * p.ldw * 2u + lchunk, a + 1024u);
+        gd_lin_load_lds16(src, (nbase + first_row(o0 + min(jc + lrow[0], last))) * p.ldw * 2u + lchunk, a);
+        gd_lin_load_lds16(src, (nbase + first_row(o0 + min(jc + lrow[1], last))) * p.ldw * 2u + lchunk, a + 1024u);
     };
     /* ---- requested in front of the ring and counted by hand (gd_wide_request16): the bias values and positions of
      *      all tiles of this workgroup (TPW * OUT_COLS <= 512: at most one column per thread) and the activation
@@ -589,8 +593,8 @@ gd_linear_wide_persistent_kernel(const gd_half *__restrict__ x, const gd_half *_
     static_assert(TPW * OUT_COLS <= 512, "one bias column per thread");
     uint32_t rq_b1 = 0u, rq_b2 = 0u, rq_pos = 0u, rq_cpos = 0u;
     const bool has_col = (int)threadIdx.x < tiles * (int)OUT_COLS;
-    const uint32_t b_n0 = tile_n0(t_begin + (has_col ? threadIdx.x / OUT_COLS : 0u));
-    const uint32_t b_col = b_n0 + min(threadIdx.x % OUT_COLS, tile_valid(b_n0) - 1u);
+    const uint32_t b_o0 = tile_o0(t_begin + (has_col ? threadIdx.x / OUT_COLS : 0u));
+    const uint32_t b_col = first_row(b_o0 + min(threadIdx.x % OUT_COLS, tile_valid(b_o0) - 1u));
     if (p.epilogue != GD_HIP_EPI_NONE) {
         rq_b1 = gd_wide_request2(bias, b_col * 2u);
         if (PAIRED) rq_b2 = gd_wide_request2(bias, (pair_offset + b_col) * 2u);
@@ -725,15 +729,15 @@ gd_linear_wide_persistent_kernel(const gd_half *__restrict__ x, const gd_half *_
             for (int j = 0; j < NT; ++j)
                 *reinterpret_cast<gd_float4 *>(s_sum + (((wave * MT + mt) * NT + j) * 64 + lane) * 4) = acc[mt][j];
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        const uint32_t n0 = tile_n0(t_begin + (uint32_t)ti);
-        const uint32_t valid = tile_valid(n0);
+        const uint32_t o0 = tile_o0(t_begin + (uint32_t)ti);
+        const uint32_t valid = tile_valid(o0);
 #pragma unroll
         for (int i = 0; i < EPT; ++i) {
             const int idx = (int)threadIdx.x + 512 * i;
             const int jj = idx >> 8, mt = jj / NTO, j = jj % NTO, rl = idx & 63, rr = (idx >> 6) & 3;
             if (jj >= NTO * MT) continue;
-            const uint32_t col = n0 + 16u * j + (rl & 15);
             const bool col_used = 16u * (uint32_t)j + (uint32_t)(rl & 15) < valid;
+            const uint32_t col = first_row(o0 + 16u * j + (rl & 15));
             const uint32_t lrow_i = 16u * mt + 4u * (rl >> 4) + rr, row = m0 + lrow_i;
             float v1 = 0.f, v2 = 0.f;
 #pragma unroll

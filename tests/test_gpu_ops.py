@@ -1219,6 +1219,52 @@ def test_few_row_projection_narrow_tiles_fill_every_compute_unit(backend, arena,
         _close(got["narrow"], oracle.swiglu_split(u), through=through)
 
 
+@pytest.mark.parametrize("M", [16, 32])
+def test_few_row_qkv_rope_narrow_tiles_straddle_heads(backend, arena, oracle, gda, M):
+    """The 3072 rotation pairs of a 16-head, 128-wide qkv projection are 192 full tiles of 16 pairs; on 256 compute units
+    they are dealt out 12 pairs to a tile, which then straddle heads (pair -> weight row computed per lane).  Same
+    bits as the full tiles (tunable linear_tiles = 4) and as the stream kernel, q and both caches."""
+    K, H, D, Tmax = 2048, 16, 128, 6
+    N = 3 * H * D
+    x = oracle.normal_f16((M, K), 5400 + M, 1.2)
+    nw = (1.0 + 0.1 * oracle.normal_f16((K,), 5401).astype(np.float32)).astype(np.float16)
+    w = oracle.normal_f16((N, K), 5402, 0.05)
+    bias = oracle.normal_f16((N,), 5403, 0.4)
+    tx, tw, tb, tn = (arena.from_numpy(a) for a in (x, w, bias, nw))
+    pos = oracle.uniform_i32(M, 5404, 0, 3000)
+    cpos = oracle.uniform_i32(M, 5405, 0, Tmax - 1)
+    cpos[1] = -1
+    tp, tc = arena.from_numpy(pos), arena.from_numpy(cpos)
+    k0, v0 = oracle.normal_f16((M, Tmax, H, D), 5406), oracle.normal_f16((M, Tmax, H, D), 5407)
+    got = {}
+    try:
+        for name, wide, tiles in (("narrow", 1, 0), ("full", 1, 4), ("stream", 0, 0)):
+            backend.set_tunable("linear_wide", wide)
+            backend.set_tunable("linear_tiles", tiles)
+            backend.set_tunable("linear_waves", 0 if wide else 8)
+            q, kc, vc = arena.alloc((M, H, D), gda.F16), arena.from_numpy(k0), arena.from_numpy(v0)
+            backend.fill(q, 0x7e00)
+            backend.fused_qkv_rope_append(tx, tw, tb, tn, tp, tc, q, kc, vc, H, D, 2, 2, 1e-5)
+            got[name] = (q.read(), kc.read(), vc.read())
+            assert backend.linear_last_kernel() == ("wide" if wide else "stream")
+    finally:
+        backend.set_tunable("linear_wide", -1)
+        backend.set_tunable("linear_tiles", 0)
+        backend.set_tunable("linear_waves", 0)
+    for other in ("full", "stream"):
+        for a, b in zip(got["narrow"], got[other]):
+            assert np.array_equal(_bits(a), _bits(b)), other
+    u = oracle.linear_nt(oracle.rms_norm(x, nw, 1e-5), w, bias)
+    qo, ko, vo = oracle.qkv_split_rope(u, pos, H, D)
+    _close(got["narrow"][0], qo, atol=4e-3)
+    for b in range(M):
+        if 0 <= cpos[b] < Tmax:
+            _close(got["narrow"][1][b, cpos[b]], ko[b], atol=4e-3)
+            _close(got["narrow"][2][b, cpos[b]], vo[b])
+        else:
+            assert np.array_equal(_bits(got["narrow"][1][b]), _bits(k0[b]))
+
+
 # (33 rows or more with the rotation take the stream kernel by design)
 @pytest.mark.parametrize("kind,K,tiles,M", [(kind, K, tiles, M) for kind in ("plain", "swiglu", "rope")
                                             for (K, tiles) in ((1024, 0), (1536, 0), (2048, 1), (2048, 0))
