@@ -707,3 +707,10 @@ def main():
 
 if __name__ == "__main__":
     main()
+    # The line is out: leave without the interpreter's and the HIP runtime's teardown, whose order at process exit is
+    # not ours to control (one small program of this repository once ended with SIGSEGV after its work was done).  Not
+    # under a profiler, which writes its traces at exit.
+    sys.stdout.flush()
+    sys.stderr.flush()
+    if not profiler_attached():
+        os._exit(0)
