@@ -1176,7 +1176,9 @@ def test_few_row_projection_weight_stream_through_lds(backend, arena, oracle, gd
         _close(got[0], u)
 
 
-@pytest.mark.parametrize("kind,N,M", [("swiglu", 5632, 16), ("swiglu", 5632, 32), ("plain", 12288, 16), ("plain", 12288, 32)])
+# (5600 gated and 12352 plain columns leave a last tile with 12 and 4 columns in use)
+@pytest.mark.parametrize("kind,N,M", [("swiglu", 5632, 16), ("swiglu", 5632, 32), ("plain", 12288, 16), ("plain", 12288, 32),
+                                      ("swiglu", 5600, 16), ("plain", 12352, 32)])
 def test_few_row_projection_narrow_tiles_fill_every_compute_unit(backend, arena, oracle, gda, kind, N, M):
     """Outputs with fewer full column tiles than compute units (5632 gated columns: 176 tiles of 32) are dealt out in
     narrower tiles, one per compute unit (22 columns each), whose unused columns repeat the last weight row and are not
