@@ -16,8 +16,9 @@ Prints ONE JSON line: whole-job tokens/s, plus
                 shape, rotating over more distinct K/V caches than the 256 MB memory-side cache holds:
                 algorithmic bytes / mean launch time vs 8 TB/s;
   cpu_baseline  the CPU oracle's decoder running the same step shape on the host cores;
-  others        the remaining BASELINE.json configs measured in the same process: configs[0] (batch 1,
-                32-token prompt, 64 greedy tokens), configs[1] (isolated append + sdpa_decode, ragged),
+  others        the remaining BASELINE.json configs: configs[0] (batch 1, 32-token prompt, 64 greedy
+                tokens; in a child process under the runtime's default graph replay when this process
+                replays node by node), and in the same process configs[1] (isolated append + sdpa_decode, ragged),
                 configs[3] (scaled decoder, B=16, long ragged caches), configs[4] (packed prefill of 32
                 prompts + 128 greedy steps), each with its own roofline fraction.
 """
