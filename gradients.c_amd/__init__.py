@@ -139,6 +139,7 @@ _SIGNATURES = {
     "gd_backend_qkv_split_rope_forward": [_vp, _TV, _TV, _TV, _TV, _TV, C.c_uint32, C.c_uint32, C.POINTER(RopeArgs)],
     "gd_backend_swiglu_split_forward": [_vp, _TV, _TV],
     "gd_backend_sdpa_varlen": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, C.POINTER(SdpaVarlenArgs)],
+    "gd_backend_sdpa_varlen_cached": [_vp, _TV, _TV, _TV, _TV, _TV, C.POINTER(SdpaVarlenArgs)],
     "gd_backend_sdpa_decode": [_vp, _TV, _TV, _TV, _TV, _TV, C.POINTER(SdpaDecodeArgs)],
     "gd_backend_sdpa_decode_at": [_vp, _TV, _TV, _TV, _TV, C.POINTER(SdpaDecodeArgs)],
     "gd_backend_sdpa_decode_positions": [_vp, _TV, _TV, _TV, _TV, _TV, C.POINTER(SdpaDecodeArgs)],
@@ -153,6 +154,9 @@ _SIGNATURES = {
     "gd_backend_qkv_rope_append": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, C.c_uint32, C.c_uint32, C.POINTER(RopeArgs)],
     "gd_backend_qkv_rope_append_packed": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, _TV, _TV, _TV, C.c_uint32, C.c_uint32,
                                           C.POINTER(RopeArgs)],
+    "gd_backend_rope_table_packed": [_vp, _TV, _TV, _TV, _TV, _TV, _TV, C.c_uint32, C.c_uint32, C.POINTER(RopeArgs)],
+    "gd_backend_linear_qkv_rope_packed": [_vp, _MV, _MV, _VV, _TV, _TV, _TV, _TV, _TV, _TV, _MV, C.c_uint32, C.c_uint32,
+                                          C.c_uint32],
     "gd_backend_rand_uniform": [_vp, _vp, C.c_size_t, C.c_size_t, C.c_uint32, C.c_uint64, C.c_float, C.c_float],
     "gd_backend_concat_to_full": [_vp, _TV, _TV, C.POINTER(ConcatArgs)],
     "gd_backend_gather_rows": [_vp, _TV, _TV, _TV],
@@ -472,8 +476,20 @@ class Backend:
     def qkv_rope_append_packed(self, qkv, pos, cache_pos, cu, q, k, v, k_cache, v_cache, n_heads, head_dim, theta=10000.0):
         a = RopeArgs(theta, head_dim, 0)
         _check(self.call("gd_backend_qkv_rope_append_packed", qkv.view(), pos.view(), cache_pos.view(), cu.view(), q.view(),
-                         k.view(), v.view(), k_cache.view(), v_cache.view(), n_heads, head_dim, C.byref(a)),
+                         k.view() if k is not None else None, v.view() if v is not None else None, k_cache.view(),
+                         v_cache.view(), n_heads, head_dim, C.byref(a)),
                "gd_backend_qkv_rope_append_packed")
+
+    def rope_table_packed(self, pos, cache_pos, cu, cos_rows, sin_rows, cache_rows, head_dim, tmax, theta=10000.0):
+        a = RopeArgs(theta, head_dim, 0)
+        _check(self.call("gd_backend_rope_table_packed", pos.view(), cache_pos.view(), cu.view(), cos_rows.view(),
+                         sin_rows.view(), cache_rows.view(), head_dim, tmax, C.byref(a)), "gd_backend_rope_table_packed")
+
+    def linear_qkv_rope_packed(self, x, w, bias, cos_rows, sin_rows, cache_rows, q, k_cache, v_cache, work, n_heads,
+                               head_dim, bias_mode):
+        _check(self.call("gd_backend_linear_qkv_rope_packed", x.matrix(), w.matrix(), bias.vector() if bias else None,
+                         cos_rows.view(), sin_rows.view(), cache_rows.view(), q.view(), k_cache.view(), v_cache.view(),
+                         work.matrix(), n_heads, head_dim, bias_mode), "gd_backend_linear_qkv_rope_packed")
 
     def fused_qkv_rope_append(self, x, w, bias, norm_weight, pos, cache_pos, q, k_cache, v_cache, n_heads, head_dim,
                               bias_mode, prologue, eps=0.0, theta=10000.0):
@@ -490,6 +506,11 @@ class Backend:
         a = SdpaVarlenArgs(scale, int(causal), window, prefix, max_seqlen, 0)
         _check(self.call("gd_backend_sdpa_varlen", q.view(), k.view(), v.view(), cu.view(), out.view(), None,
                          C.byref(a)), "gd_backend_sdpa_varlen")
+
+    def sdpa_varlen_cached(self, q, k_cache, v_cache, cu, out, scale, causal=True, window=0, prefix=0, max_seqlen=0):
+        a = SdpaVarlenArgs(scale, int(causal), window, prefix, max_seqlen, 0)
+        _check(self.call("gd_backend_sdpa_varlen_cached", q.view(), k_cache.view(), v_cache.view(), cu.view(), out.view(),
+                         C.byref(a)), "gd_backend_sdpa_varlen_cached")
 
     def sdpa_decode(self, q, k, v, pos, out, scale, window=0, prefix=0):
         a = SdpaDecodeArgs(scale, window, prefix, 0)

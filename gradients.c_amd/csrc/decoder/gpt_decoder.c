@@ -175,7 +175,8 @@ size_t gd_gpt_scratch_bytes(const gd_gpt_config *c, int32_t max_prefill_tokens)
     const size_t picked = c->m3_block_size > 0 ? (size_t)c->n_heads * 16U * 4U + 256U : 0U; /* block ids of a row */
     const size_t per_row = 2U * (13U * (size_t)c->d_model + 2U * (size_t)c->mlp_hidden) + 14U * 256U + picked;
     const size_t layers = rows * per_row * (size_t)c->n_layers;
-    return layers + layers / 10U + rows * ((size_t)c->d_model * 4U + (size_t)c->mlp_hidden * 2U) +
+    const size_t angles = (rows + 32U) * ((size_t)c->head_dim * 4U + 4U) + 3U * 256U; /* cos, sin and cache row per prompt row */
+    return layers + layers / 10U + rows * ((size_t)c->d_model * 4U + (size_t)c->mlp_hidden * 2U) + angles +
            (size_t)c->batch * (size_t)c->vocab * 4U + ((size_t)64 << 20);
 }
 
@@ -613,17 +614,83 @@ static gd_status block_decode(gd_gpt_decoder *d, int32_t l, const gd_tensor *x, 
     return block_tail(d, b, x, &attn_flat, out);
 }
 
+/* angles and cache rows of the packed prompt rows (gd_backend_rope_table_packed), shared by the layers of a prefill */
+typedef struct prefill_rope_rows {
+    gd_tensor cos_rows, sin_rows, cache_rows;
+} prefill_rope_rows;
+
+static bool mview(const gd_tensor *t, int64_t rows, int64_t cols, gd_backend_matrix_view *m);
+static void vview(const gd_tensor *t, gd_backend_vector_view *v);
+static gd_status scratch_f16(gd_context *ctx, int64_t rows, int64_t cols, gd_tensor *out);
+
+/* the qkv projection can carry rotation, split and cache append in its epilogue (gd_backend_linear_qkv_rope_packed) */
+static bool prefill_rope_in_projection(const gd_gpt_decoder *d)
+{
+    const gd_gpt_config *c = &d->cfg;
+    const bool m3 = c->m3_block_size > 0 && c->m3_topk_blocks > 0 &&
+                    (int64_t)c->max_seq > (int64_t)c->m3_block_size * 8 &&
+                    (int64_t)c->m3_block_size * c->m3_topk_blocks * 2 < (int64_t)c->max_seq;
+    return !m3 && (c->head_dim == 64 || c->head_dim == 128) && (c->d_model % 256) == 0 &&
+           d->blocks[0].qkv_proj.transposed && d->blocks[0].qkv_proj.weight.dtype == GD_DTYPE_F16 &&
+           (uint64_t)c->batch * (uint64_t)c->max_seq * (uint64_t)c->d_model * 2U < 0xffffffffULL;
+}
+
 static gd_status block_prefill(gd_gpt_decoder *d, int32_t l, const gd_tensor *x, const gd_tensor *positions,
-                               const gd_tensor *cu, const gd_tensor *cache_positions, gd_tensor *out)
+                               const gd_tensor *cu, const gd_tensor *cache_positions, const prefill_rope_rows *rows,
+                               gd_tensor *out)
 {
     gd_context *ctx = d->ctx;
     const gpt_block *b = &d->blocks[l];
     const gd_gpt_config *c = &d->cfg;
     const gd_rope_config rope = {c->rope_theta, c->head_dim, false};
     const gd_sdpa_varlen_config sdpa = {0.0f, true, c->sdpa_window, 0, c->max_seq};
+    const bool m3 = c->m3_block_size > 0 && c->m3_topk_blocks > 0 &&
+                    (int64_t)c->max_seq > (int64_t)c->m3_block_size * 8 &&
+                    (int64_t)c->m3_block_size * c->m3_topk_blocks * 2 < (int64_t)c->max_seq;
+    /* the prefill appends every sequence at cache position 0 (gd_gpt_decoder_prefill), so the attention can read the
+     * keys and values of a sequence where the append has just put them, and the packed k / v are never written */
+    const bool from_caches = !m3 && (c->head_dim == 64 || c->head_dim == 128) &&
+                             (uint64_t)c->batch * (uint64_t)c->max_seq * (uint64_t)c->n_heads * (uint64_t)c->head_dim * 2U <
+                                 0xffffffffULL;
     gd_tensor normed, qkv, q, k, v, attn, attn_flat;
     int64_t flat_shape[2] = {x->shape[0], c->d_model};
+    bool attended = false;
     TRY(gd_rms_norm(ctx, x, &b->attn_norm_w, c->rms_eps, &normed));
+    if (rows != NULL && from_caches && x->shape[0] >= 256) {
+        /* rotation, split and cache append in the epilogue of the projection's tiles; attention from the caches */
+        const gd_backend_sdpa_varlen_args va = {(float)(1.0 / sqrt((double)c->head_dim)), 1U, (uint32_t)c->sdpa_window, 0U,
+                                                (uint32_t)c->max_seq, 0U};
+        const int64_t N = x->shape[0];
+        int64_t dims[3] = {N, c->n_heads, c->head_dim};
+        gd_backend_matrix_view xm, wm, workm;
+        gd_backend_vector_view bv;
+        gd_backend_tensor_view vcos, vsin, vrows, vq, vkc, vvc, vcu, vo;
+        gd_status st;
+        TRY(gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F16, gd_shape_make(3U, dims), 256U, &q));
+        TRY(scratch_f16(ctx, N, 3 * (int64_t)c->d_model, &qkv));
+        mview(&normed, N, c->d_model, &xm);
+        mview(&b->qkv_proj.weight, b->qkv_proj.weight.shape[0], b->qkv_proj.weight.shape[1], &wm);
+        mview(&qkv, N, 3 * (int64_t)c->d_model, &workm);
+        vview(&b->qkv_proj.bias, &bv);
+        tview(&rows->cos_rows, &vcos);
+        tview(&rows->sin_rows, &vsin);
+        tview(&rows->cache_rows, &vrows);
+        tview(&q, &vq);
+        tview(&d->k_cache[l], &vkc);
+        tview(&d->v_cache[l], &vvc);
+        tview(cu, &vcu);
+        /* bias mode 2: gd_linear_transposed_weight is matmul_nt + add, two roundings */
+        st = gd_backend_linear_qkv_rope_packed(gd_context_backend(ctx), &xm, &wm, &bv, &vcos, &vsin, &vrows, &vq, &vkc, &vvc,
+                                               &workm, (uint32_t)c->n_heads, (uint32_t)c->head_dim, 2U);
+        if (st == GD_OK) {
+            TRY(gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F16, gd_shape_make(3U, dims), 256U, &attn));
+            tview(&attn, &vo);
+            TRY(gd_backend_sdpa_varlen_cached(gd_context_backend(ctx), &vq, &vkc, &vvc, &vcu, &vo, &va));
+            TRY(gd_reshape(ctx, &attn, gd_shape_make(2U, flat_shape), &attn_flat));
+            return block_tail_prefill(d, b, x, &attn_flat, out);
+        }
+        if (st != GD_ERR_UNSUPPORTED) return st;
+    }
     TRY(linear_forward(ctx, &b->qkv_proj, &normed, &qkv));
     if ((c->head_dim % 16) == 0 && qkv.dtype == GD_DTYPE_F16) {
         /* rotation, split and cache append in one pass over the projection: the appended rows are not read back */
@@ -631,26 +698,39 @@ static gd_status block_prefill(gd_gpt_decoder *d, int32_t l, const gd_tensor *x,
         int64_t dims[3] = {x->shape[0], c->n_heads, c->head_dim};
         gd_backend_tensor_view vqkv, vpos, vcp, vcu, vq, vk, vv, vkc, vvc;
         TRY(gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F16, gd_shape_make(3U, dims), 256U, &q));
-        TRY(gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F16, gd_shape_make(3U, dims), 256U, &k));
-        TRY(gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F16, gd_shape_make(3U, dims), 256U, &v));
+        if (!from_caches) {
+            TRY(gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F16, gd_shape_make(3U, dims), 256U, &k));
+            TRY(gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F16, gd_shape_make(3U, dims), 256U, &v));
+            tview(&k, &vk);
+            tview(&v, &vv);
+        }
         tview(&qkv, &vqkv);
         tview(positions, &vpos);
         tview(cache_positions, &vcp);
         tview(cu, &vcu);
         tview(&q, &vq);
-        tview(&k, &vk);
-        tview(&v, &vv);
         tview(&d->k_cache[l], &vkc);
         tview(&d->v_cache[l], &vvc);
-        TRY(gd_backend_qkv_rope_append_packed(gd_context_backend(ctx), &vqkv, &vpos, &vcp, &vcu, &vq, &vk, &vv, &vkc, &vvc,
+        TRY(gd_backend_qkv_rope_append_packed(gd_context_backend(ctx), &vqkv, &vpos, &vcp, &vcu, &vq,
+                                              from_caches ? NULL : &vk, from_caches ? NULL : &vv, &vkc, &vvc,
                                               (uint32_t)c->n_heads, (uint32_t)c->head_dim, &ra));
+        if (from_caches) {
+            const gd_backend_sdpa_varlen_args va = {(float)(1.0 / sqrt((double)c->head_dim)), 1U, (uint32_t)c->sdpa_window,
+                                                    0U, (uint32_t)c->max_seq, 0U};
+            gd_backend_tensor_view vo;
+            TRY(gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F16, gd_shape_make(3U, dims), 256U, &attn));
+            tview(&attn, &vo);
+            TRY(gd_backend_sdpa_varlen_cached(gd_context_backend(ctx), &vq, &vkc, &vvc, &vcu, &vo, &va));
+            attended = true;
+        }
     } else {
         TRY(gd_qkv_split_rope(ctx, &qkv, positions, c->n_heads, c->head_dim, &rope, &q, &k, &v));
         TRY(gd_kv_cache_append_packed(ctx, &d->k_cache[l], &d->v_cache[l], cache_positions, cu, &k, &v));
     }
     /* MiniMax-M3: picked blocks when the context is long enough for that to matter (reference :588-600, 918-933) */
-    if (c->m3_block_size > 0 && c->m3_topk_blocks > 0 && (int64_t)c->max_seq > (int64_t)c->m3_block_size * 8 &&
-        (int64_t)c->m3_block_size * c->m3_topk_blocks * 2 < (int64_t)c->max_seq) {
+    if (attended) {
+        /* done above, from the caches */
+    } else if (m3) {
         const gd_minimax_m3_sparse_config m3 = {0.0f, c->m3_block_size, c->m3_topk_blocks, c->m3_init_blocks,
                                                 c->m3_local_blocks, c->max_seq};
         gd_tensor picked;
@@ -722,6 +802,8 @@ gd_status gd_gpt_decoder_prefill(gd_gpt_decoder *d, const int32_t *ids, const in
 {
     gd_context *ctx;
     gd_tensor t_ids, t_pos, t_cu, t_cache_pos, t_last, x, y, last_hidden, t_logits, t_next, t_gaps;
+    prefill_rope_rows rope_rows;
+    bool have_rows = false;
     gd_status st = GD_OK;
     int32_t *positions, *zero, *last_rows;
     int32_t B, N, b, r, l;
@@ -753,8 +835,31 @@ gd_status gd_gpt_decoder_prefill(gd_gpt_decoder *d, const int32_t *ids, const in
         if (st == GD_OK) st = data_i32(ctx, zero, B, &t_cache_pos);
         if (st == GD_OK) st = data_i32(ctx, last_rows, B, &t_last);
         if (st == GD_OK) st = gd_embedding(ctx, &d->token_embedding, &t_ids, &x);
+        if (st == GD_OK && N >= 256 && prefill_rope_in_projection(d)) {
+            /* once for all layers: the angles of every row's position and the cache row its k and v go to */
+            const gd_backend_rope_args ra = {d->cfg.rope_theta, (uint32_t)d->cfg.head_dim, 0U};
+            int64_t tdims[2] = {((int64_t)N + 31) / 32 * 32, d->cfg.head_dim / 2}, rdims[1] = {N};
+            gd_backend_tensor_view vpos, vcp, vcu, vcos, vsin, vrows;
+            st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F32, gd_shape_make(2U, tdims), 256U, &rope_rows.cos_rows);
+            if (st == GD_OK)
+                st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_F32, gd_shape_make(2U, tdims), 256U, &rope_rows.sin_rows);
+            if (st == GD_OK)
+                st = gd_tensor_empty(ctx, GD_ARENA_SCRATCH, GD_DTYPE_I32, gd_shape_make(1U, rdims), 256U, &rope_rows.cache_rows);
+            if (st == GD_OK) {
+                tview(&t_pos, &vpos);
+                tview(&t_cache_pos, &vcp);
+                tview(&t_cu, &vcu);
+                tview(&rope_rows.cos_rows, &vcos);
+                tview(&rope_rows.sin_rows, &vsin);
+                tview(&rope_rows.cache_rows, &vrows);
+                st = gd_backend_rope_table_packed(gd_context_backend(ctx), &vpos, &vcp, &vcu, &vcos, &vsin, &vrows,
+                                                  (uint32_t)d->cfg.head_dim, (uint32_t)d->cfg.max_seq, &ra);
+                have_rows = st == GD_OK;
+                if (st == GD_ERR_UNSUPPORTED) st = GD_OK;
+            }
+        }
         for (l = 0; l < d->cfg.n_layers && st == GD_OK; ++l) {
-            st = block_prefill(d, l, &x, &t_pos, &t_cu, &t_cache_pos, &y);
+            st = block_prefill(d, l, &x, &t_pos, &t_cu, &t_cache_pos, have_rows ? &rope_rows : NULL, &y);
             x = y;
         }
         if (st == GD_OK) st = gd_gather_rows(ctx, &x, &t_last, &last_hidden);

@@ -215,6 +215,114 @@ gd_status gd_backend_fused_qkv_rope_append(gd_backend *backend, const gd_backend
         backend->linear_wide, &backend->last_linear_family));
 }
 
+int gd_hip_launch_linear_tile_rope(hipStream_t stream, const void *x, const void *w, const void *bias,
+                                   const gd_hip_linear_params *params, const float *cos_rows, const float *sin_rows,
+                                   const int32_t *cache_row, void *q, void *k_cache, void *v_cache, uint32_t hd,
+                                   uint32_t half_d, int compute_units);
+uint32_t gd_hip_linear_tile_rope_head_rows(uint32_t M, uint32_t N, int compute_units);
+int gd_hip_launch_qkv_rope_rows(hipStream_t stream, const void *qkv, const float *cos_rows, const float *sin_rows,
+                                const int32_t *cache_row, void *q, void *k_cache, void *v_cache, uint64_t row0,
+                                uint64_t rows, uint32_t heads, uint32_t head_dim);
+
+/* qkv projection of a packed prefill with rotation, split and cache append in the projection's epilogue (see the
+ * header): the row tiles that fill whole rounds of 256 x 256 tiles go through the tile kernel's rotation epilogue;
+ * the rest goes through the plain projection into `work` and the table-driven rotation kernel. */
+gd_status gd_backend_linear_qkv_rope_packed(gd_backend *backend, const gd_backend_matrix_view *x,
+                                            const gd_backend_matrix_view *w, const gd_backend_vector_view *bias,
+                                            const gd_backend_tensor_view *cos_rows, const gd_backend_tensor_view *sin_rows,
+                                            const gd_backend_tensor_view *cache_rows, const gd_backend_tensor_view *q,
+                                            const gd_backend_tensor_view *k_cache, const gd_backend_tensor_view *v_cache,
+                                            const gd_backend_matrix_view *work, uint32_t n_heads, uint32_t head_dim,
+                                            uint32_t bias_mode)
+{
+    gd_hip_linear_params p;
+    uint64_t area;
+    uint32_t i, head_rows;
+    int e;
+    if (backend == NULL || !gd_hip_matrix_ok(x) || !gd_hip_matrix_ok(w) || !gd_hip_matrix_ok(work) ||
+        (bias != NULL && !gd_hip_vector_ok(bias)) || !gd_hip_view_ok(cos_rows) || !gd_hip_view_ok(sin_rows) ||
+        !gd_hip_view_ok(cache_rows) || !gd_hip_view_ok(q) || !gd_hip_view_ok(k_cache) || !gd_hip_view_ok(v_cache) ||
+        n_heads == 0u || head_dim == 0u || cos_rows->rank != 2u || sin_rows->rank != 2u || cache_rows->rank != 1u ||
+        q->rank != 3u || k_cache->rank != 4u || v_cache->rank != 4u || bias_mode > 2u || (bias_mode != 0u) != (bias != NULL))
+        return GD_ERR_INVALID_ARGUMENT;
+    if (x->dtype != GD_BACKEND_DTYPE_F16 || w->dtype != GD_BACKEND_DTYPE_F16 || work->dtype != GD_BACKEND_DTYPE_F16 ||
+        q->dtype != GD_BACKEND_DTYPE_F16 || k_cache->dtype != GD_BACKEND_DTYPE_F16 ||
+        v_cache->dtype != GD_BACKEND_DTYPE_F16 || (bias != NULL && bias->dtype != GD_BACKEND_DTYPE_F16) ||
+        cos_rows->dtype != GD_BACKEND_DTYPE_F32 || sin_rows->dtype != GD_BACKEND_DTYPE_F32 ||
+        cache_rows->dtype != GD_BACKEND_DTYPE_I32)
+        return GD_ERR_UNSUPPORTED;
+    area = (uint64_t)n_heads * head_dim;
+    for (i = 0u; i < 4u; ++i) {
+        if (k_cache->shape[i] != v_cache->shape[i]) return GD_ERR_INVALID_ARGUMENT;
+    }
+    if (area * 3u > 0xffffffffu || w->rows != (uint32_t)(area * 3u) || w->cols != x->cols || x->rows == 0u ||
+        (bias != NULL && bias->length != w->rows) || work->rows != x->rows || work->cols != w->rows ||
+        q->shape[0] != (int64_t)x->rows || q->shape[1] != (int64_t)n_heads || q->shape[2] != (int64_t)head_dim ||
+        k_cache->shape[2] != (int64_t)n_heads || k_cache->shape[3] != (int64_t)head_dim ||
+        cache_rows->shape[0] != (int64_t)x->rows || cos_rows->shape[0] != ((int64_t)x->rows + 31) / 32 * 32 ||
+        sin_rows->shape[0] != cos_rows->shape[0] || cos_rows->shape[1] != (int64_t)(head_dim / 2u) ||
+        (uint64_t)cos_rows->shape[0] * (head_dim / 2u) > 0x7fffffffull ||
+        sin_rows->shape[1] != (int64_t)(head_dim / 2u) || (cache_rows->offset & 3u) != 0u)
+        return GD_ERR_INVALID_ARGUMENT;
+    /* the tile kernel's rotation epilogue: head size 64 or 128, heads * head_dim a multiple of 256 (every 128-column
+     * block of a wavefront inside q, k or v), K a multiple of 64, 16-byte aligned rows everywhere, caches whose rows a
+     * 31-bit row number reaches */
+    if ((head_dim != 64u && head_dim != 128u) || (area % 256u) != 0u || (x->cols % 64u) != 0u || x->cols < 128u ||
+        ((x->offset | x->row_bytes | w->offset | w->row_bytes | work->offset | work->row_bytes | q->offset |
+          k_cache->offset | v_cache->offset | cos_rows->offset | sin_rows->offset) & 15u) != 0u ||
+        (uint64_t)k_cache->shape[0] * (uint64_t)k_cache->shape[1] > (uint64_t)INT32_MAX ||
+        work->row_bytes != (size_t)w->rows * 2u) /* the row kernel reads packed rows */
+        return GD_ERR_UNSUPPORTED;
+    p.M = x->rows;
+    p.N = w->rows;
+    p.K = x->cols;
+    p.ldx = (uint32_t)(x->row_bytes / 2u);
+    p.ldw = (uint32_t)(w->row_bytes / 2u);
+    p.ldy = (uint32_t)(work->row_bytes / 2u);
+    p.epilogue = bias != NULL ? bias_mode : GD_HIP_EPI_NONE;
+    p.w_is_nk = 1u;
+    p.prologue = GD_HIP_PRO_NONE;
+    p.has_residual = 0u;
+    p.ldr = 0u;
+    p.eps = 0.0f;
+    p.swiglu_cols = 0u;
+    p.rope_heads = p.rope_head_dim = p.rope_tmax = 0u;
+    p.rope_freq_scale = 0.0f;
+    p.force_tiles = (uint16_t)backend->linear_tiles;
+    p.force_waves = (uint16_t)backend->linear_waves;
+    p.no_lds_stream = (uint32_t)backend->linear_no_lds_stream;
+    head_rows = gd_hip_linear_tile_rope_head_rows(p.M, p.N, backend->compute_units);
+    if (head_rows != 0u) {
+        gd_hip_linear_params head = p;
+        head.M = head_rows;
+        e = gd_hip_launch_linear_tile_rope(backend->stream, gd_hip_matrix_ptr(x), gd_hip_matrix_ptr(w),
+                                           bias != NULL ? gd_hip_vector_ptr(bias) : NULL, &head,
+                                           (const float *)gd_hip_view_ptr(cos_rows), (const float *)gd_hip_view_ptr(sin_rows),
+                                           (const int32_t *)gd_hip_view_ptr(cache_rows), gd_hip_view_ptr(q),
+                                           gd_hip_view_ptr(k_cache), gd_hip_view_ptr(v_cache), (uint32_t)area,
+                                           head_dim / 2u, backend->compute_units);
+        if (e != 0) return gd_hip_finish_op(backend, e);
+        backend->last_linear_family = GD_HIP_LINEAR_FAMILY_TILE;
+    }
+    if (head_rows < p.M) {
+        gd_hip_linear_params tail = p;
+        char *work_rows = (char *)gd_hip_matrix_ptr(work) + (size_t)head_rows * work->row_bytes;
+        tail.M = p.M - head_rows;
+        e = gd_hip_launch_linear(backend->stream, (const char *)gd_hip_matrix_ptr(x) + (size_t)head_rows * x->row_bytes,
+                                 gd_hip_matrix_ptr(w), bias != NULL ? gd_hip_vector_ptr(bias) : NULL, NULL, NULL, work_rows,
+                                 &tail, 1, 0, 1, 2 * backend->compute_units, NULL, backend->linear_wide,
+                                 &backend->last_linear_family);
+        if (e != 0) return gd_hip_finish_op(backend, e);
+        e = gd_hip_launch_qkv_rope_rows(backend->stream, work_rows, (const float *)gd_hip_view_ptr(cos_rows),
+                                        (const float *)gd_hip_view_ptr(sin_rows),
+                                        (const int32_t *)gd_hip_view_ptr(cache_rows), gd_hip_view_ptr(q),
+                                        gd_hip_view_ptr(k_cache), gd_hip_view_ptr(v_cache), head_rows, tail.M, n_heads,
+                                        head_dim);
+        if (e != 0) return gd_hip_finish_op(backend, e);
+    }
+    return gd_hip_finish_op(backend, 0);
+}
+
 /* Which kernel family the last projection call on this backend took: "stream", "wide", "tile" or "scalar". */
 gd_status gd_backend_linear_last_kernel(gd_backend *backend, char *out, size_t capacity)
 {

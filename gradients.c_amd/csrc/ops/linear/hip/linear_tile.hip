@@ -45,6 +45,7 @@
  */
 #include "../../_shared/hip_device.h"
 #include "hip_linear_types.h"
+#include "../../qkv_split_rope/hip/rope_device.h"
 #include <type_traits>
 
 #define GD_TILE_BK 64u
@@ -67,6 +68,19 @@ extern "C" __attribute__((visibility("default"))) int gd_hip_linear_tile_timelin
 #else
 #define GD_TILE_NOTE(slot, value) do { } while (0)
 #endif
+
+/* Rotation + cache append epilogue of the packed prefill's qkv projection (ROPE instantiation): the tile kernel
+ * writes rotated q rows to q [M, hd], rotated k rows and v rows into cache row cache_row[m] of the K / V caches
+ * (row pitch hd), and no [M, 3*hd] intermediate.  cos / sin hold, F32, the angles of row m's position for the half_d
+ * pairs of a head (NeoX pairing: column c of a head with column c + half_d) in the layout of the table kernel
+ * (gd_rope_table_at in ops/qkv_split_rope/hip/qkv_split_rope.hip). */
+struct gd_tile_rope {
+    const float *cos, *sin;
+    const int32_t *cache_row; /* [M]; negative: the row's k and v go nowhere */
+    gd_half *q, *k_cache, *v_cache;
+    uint32_t hd;     /* heads * head_dim, a multiple of 256 */
+    uint32_t half_d; /* 32 or 64 */
+};
 
 __device__ __forceinline__ uint32_t gd_tile_slot(uint32_t row, uint32_t c)
 {
@@ -95,12 +109,12 @@ __device__ __forceinline__ void gd_tile_load_lds16(const gd_half *uniform_base, 
                  : "memory");
 }
 
-template <int WM, int WN, bool W_NK, int PRO>
+template <int WM, int WN, bool W_NK, int PRO, bool ROPE = false>
 __global__ void __launch_bounds__(256)
 gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__ w, const gd_half *__restrict__ bias,
                       const gd_half *__restrict__ residual, const gd_half *__restrict__ norm_w,
                       gd_half *__restrict__ y, gd_hip_linear_params p, uint32_t tiles_m, uint32_t tiles_n,
-                      uint32_t vector_store)
+                      uint32_t vector_store, gd_tile_rope rp)
 {
     constexpr uint32_t BM = 64u * WM, BN = 64u * WN;
     constexpr int A_PER = BM / 32;                 /* 16-byte chunks of the activation tile per thread */
@@ -664,6 +678,128 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
         pass(std::integral_constant<int, (WM > 2 ? 3 : 0)>{});
     };
 
+    /* ROPE instantiation (whole tiles only; the launcher sees to that): the wavefront's 128 columns lie inside q, k
+     * or v (hd is a multiple of 256) and hold whole heads, so both columns of a rotation pair (c, c + half_d) are in
+     * one lane's accumulators: tiles j and j + half_d / 32.  Rounding points as in the separate operators: the
+     * projection is rounded to F16 (with its bias), rotated in F32 with the angles of the row's position, rounded
+     * again.  Rotated quads then take the path of epilogue_own; a row piece goes to row m of q or to row
+     * cache_row[m] of the K or V cache. */
+    auto epilogue_own_rope = [&](auto mode_tag) __attribute__((always_inline)) {
+        if (decltype(mode_tag)::value != GD_HIP_EPI_NONE) load_bias();
+        unsigned char *own = epi + wave * 8192u;
+        const uint32_t rr = lane >> 4, v = lane & 15u;
+        const uint32_t col0 = n0 + wn * (WN * 32u);
+        const uint32_t region = col0 >= 2u * rp.hd ? 2u : (col0 >= rp.hd ? 1u : 0u); /* q, k, v */
+        gd_half *dst = rp.q;
+        if (region == 1u) dst = rp.k_cache;
+        if (region == 2u) dst = rp.v_cache;
+        dst += col0 - region * rp.hd + v * 8u;
+        const uint32_t row_w = m0 + wm * (WM * 32u);
+        typedef float gd_float4v __attribute__((ext_vector_type(4)));
+        /* what a pass needs from memory: the angles of its 32 rows (region q or k) and the destination rows of the
+         * lane's 8 row pieces.  Both are requested one pass ahead so that their latency passes behind the pass in
+         * front: the angles into the registers the running pass has just used them from, the rows into a second
+         * set. */
+        /* element offset of the lane's first angle of pass I in the angle tables, which are laid out for this read
+         * (blocks of 32 rows, groups of 8 pairs, the low and the high 4 pairs of all 32 rows: the 64 lanes of a load
+         * read 1 KB of consecutive memory; group g of the block lies 256 elements behind group g - 1); a signed
+         * 32-bit number (the launcher keeps the tables below 2^31 elements), so that the loads take the table's base
+         * from scalar registers and the constant steps as immediate offsets */
+        auto table_at = [&](int I) __attribute__((always_inline)) {
+            return (int32_t)(((row_w >> 5) + (uint32_t)I) * (rp.half_d * 32u) + frag_c * 128u + frag_row * 4u);
+        };
+        auto request_rows = [&](int I, int32_t (&drow)[8]) __attribute__((always_inline)) {
+#pragma unroll
+            for (uint32_t it = 0; it < 8u; ++it) {
+                const uint32_t r = row_w + (uint32_t)I * 32u + it * 4u + rr;
+                drow[it] = region == 0u ? (int32_t)r : rp.cache_row[r];
+            }
+        };
+        auto pass = [&](auto pass_tag, auto t_tag, gd_float4v (&cs)[8], gd_float4v (&sn)[8], const int32_t (&drow)[8],
+                        int32_t (&drow_next)[8]) __attribute__((always_inline)) {
+            constexpr int I = decltype(pass_tag)::value;
+            constexpr int T = decltype(t_tag)::value; /* accumulator tiles per half head */
+            constexpr bool MORE = I + 1 < WM;
+            if (MORE) request_rows(I + 1, drow_next);
+            auto stage = [&](int j, int pr, gd_half4 a, gd_half4 b) __attribute__((always_inline)) {
+                const uint32_t c = (uint32_t)j * 4u + 2u * (uint32_t)pr + frag_c;
+                *reinterpret_cast<gd_half8 *>(own + (frag_row * 16u + (c ^ (frag_row & 15u))) * 16u) = pair_chunk(a, b);
+            };
+            if (region < 2u) {
+                const int32_t tnext = table_at(I + 1);
+#pragma unroll
+                for (int t = 0; t < T; ++t) {
+#pragma unroll
+                    for (int pr = 0; pr < 2; ++pr) {
+                        gd_half4 olo[WN / (2 * T)][2], ohi[WN / (2 * T)][2];
+#pragma unroll
+                        for (int s2 = 0; s2 < 2; ++s2) {
+                            const int q = 2 * pr + s2;
+#pragma unroll
+                            for (int g = 0; g < WN / (2 * T); ++g) {
+                                const int jlo = g * 2 * T + t, jhi = jlo + T;
+                                const gd_half4 lo = quad_f16(mode_tag, acc[I][jlo], jlo, q);
+                                const gd_half4 hi = quad_f16(mode_tag, acc[I][jhi], jhi, q);
+#pragma unroll
+                                for (int r = 0; r < 4; ++r) {
+                                    gd_half a, b;
+                                    gd_rope_rotate((float)lo[r], (float)hi[r], cs[t * 4 + q][r], sn[t * 4 + q][r], &a, &b);
+                                    olo[g][s2][r] = a;
+                                    ohi[g][s2][r] = b;
+                                }
+                            }
+                            if (MORE) {
+                                cs[t * 4 + q] = *reinterpret_cast<const gd_float4v *>(rp.cos + (tnext + 256 * (t * 4 + q)));
+                                sn[t * 4 + q] = *reinterpret_cast<const gd_float4v *>(rp.sin + (tnext + 256 * (t * 4 + q)));
+                            }
+                        }
+#pragma unroll
+                        for (int g = 0; g < WN / (2 * T); ++g) {
+                            stage(g * 2 * T + t, pr, olo[g][0], olo[g][1]);
+                            stage(g * 2 * T + t + T, pr, ohi[g][0], ohi[g][1]);
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < WN; ++j)
+#pragma unroll
+                    for (int pr = 0; pr < 2; ++pr)
+                        stage(j, pr, quad_f16(mode_tag, acc[I][j], j, 2 * pr), quad_f16(mode_tag, acc[I][j], j, 2 * pr + 1));
+            }
+            gd_half8 h[8];
+#pragma unroll
+            for (uint32_t it = 0; it < 8u; ++it) {
+                const uint32_t e = it * 4u + rr;
+                h[it] = *reinterpret_cast<const gd_half8 *>(own + (e * 16u + (v ^ (e & 15u))) * 16u);
+            }
+#pragma unroll
+            for (uint32_t it = 0; it < 8u; ++it) {
+                if (drow[it] >= 0) *reinterpret_cast<gd_half8 *>(dst + (size_t)(uint32_t)drow[it] * rp.hd) = h[it];
+            }
+        };
+        auto passes = [&](auto t_tag) __attribute__((always_inline)) {
+            constexpr int T = decltype(t_tag)::value;
+            gd_float4v cs[8], sn[8];
+            int32_t even[8], odd[8];
+            request_rows(0, even);
+            if (region < 2u) {
+                const int32_t t0 = table_at(0);
+#pragma unroll
+                for (int t = 0; t < T * 4; ++t) {
+                    cs[t] = *reinterpret_cast<const gd_float4v *>(rp.cos + (t0 + 256 * t));
+                    sn[t] = *reinterpret_cast<const gd_float4v *>(rp.sin + (t0 + 256 * t));
+                }
+            }
+            pass(std::integral_constant<int, 0>{}, t_tag, cs, sn, even, odd);
+            pass(std::integral_constant<int, 1>{}, t_tag, cs, sn, odd, even);
+            pass(std::integral_constant<int, (WM > 2 ? 2 : 0)>{}, t_tag, cs, sn, even, odd);
+            pass(std::integral_constant<int, (WM > 2 ? 3 : 0)>{}, t_tag, cs, sn, odd, even);
+        };
+        if (rp.half_d == 64u) passes(std::integral_constant<int, (WN >= 4 ? 2 : 1)>{});
+        else passes(std::integral_constant<int, 1>{});
+    };
+
         /* interior tile: every staged chunk is in range, so the main loop carries no guards */
         const bool interior = m0 + BM <= p.M && n0 + out_bn <= p.N && (p.K % GD_TILE_BK) == 0u;
 
@@ -743,7 +879,9 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
         GD_TILE_NOTE(3, __builtin_amdgcn_s_memtime() - timeline_c0);
 #endif
         auto finish = [&](auto mode_tag) __attribute__((always_inline)) {
-            if (WM == 4 && WN == 4 && vector_store && m0 + BM <= p.M && n0 + out_bn <= p.N) {
+            if constexpr (ROPE) {
+                epilogue_own_rope(mode_tag);
+            } else if (WM == 4 && WN == 4 && vector_store && m0 + BM <= p.M && n0 + out_bn <= p.N) {
                 if (gated) epilogue_own_gated(mode_tag);
                 else epilogue_own(mode_tag);
             } else {
@@ -776,7 +914,8 @@ static int launch_tile_one(hipStream_t stream, const gd_half *x, const gd_half *
     const uint32_t tiles_m = (p.M + BM - 1u) / BM, tiles_n = (p.N + out_bn - 1u) / out_bn;
     /* persistent workgroups: at most `workgroups` of them (a multiple of 8 keeps the tile -> XCD relation) */
     const uint32_t grid = tiles_m * tiles_n < workgroups ? tiles_m * tiles_n : workgroups;
-    kernel<<<grid, 256, lds, stream>>>(x, w, bias, residual, norm_w, y, p, tiles_m, tiles_n, vector_store);
+    kernel<<<grid, 256, lds, stream>>>(x, w, bias, residual, norm_w, y, p, tiles_m, tiles_n, vector_store,
+                                       gd_tile_rope{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0u, 0u});
     return (int)hipGetLastError();
 }
 
@@ -844,4 +983,52 @@ extern "C" int gd_hip_launch_linear_tile(hipStream_t stream, const void *x, cons
     }
     return launch_tile<2, 2>(stream, xp, (const gd_half *)w, (const gd_half *)bias, rp, (const gd_half *)norm_w, yp, p,
                              (uint32_t)vector_store, 2u * units);
+}
+
+/* The qkv projection of a packed prefill with rotation and cache append in the epilogue (gd_tile_rope): x [M,K],
+ * w [3*hd, K], whole 256 x 256 tiles only.  Requires: M % 256 == 0, hd % 256 == 0, K % 64 == 0, K >= 128, 16-byte
+ * aligned rows of x, w, q and the caches, half_d 32 or 64 (head size 64 or 128). */
+extern "C" int gd_hip_launch_linear_tile_rope(hipStream_t stream, const void *x, const void *w, const void *bias,
+                                              const gd_hip_linear_params *params, const float *cos_rows,
+                                              const float *sin_rows, const int32_t *cache_row, void *q, void *k_cache,
+                                              void *v_cache, uint32_t hd, uint32_t half_d, int compute_units)
+{
+    const gd_hip_linear_params &p = *params;
+    constexpr size_t lds = (size_t)2u * (256u + 256u) * 8u * 16u + (size_t)64u * 256u * 2u;
+    static bool configured = false;
+    auto kernel = gd_linear_tile_kernel<4, 4, true, GD_HIP_PRO_NONE, true>;
+    if (p.M == 0u) return (int)hipSuccess;
+    if ((p.M % 256u) != 0u || (hd % 256u) != 0u || p.N != 3u * hd || (p.K % 64u) != 0u || p.K < 128u || !p.w_is_nk ||
+        p.prologue != GD_HIP_PRO_NONE || p.has_residual || p.swiglu_cols != 0u || (half_d != 32u && half_d != 64u))
+        return (int)hipErrorInvalidValue;
+    if (!configured) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        configured = true;
+    }
+    const uint32_t units = ((uint32_t)(compute_units > 0 ? compute_units : 256) + 7u) & ~7u;
+    const uint32_t tiles_m = p.M / 256u, tiles_n = p.N / 256u;
+    const uint32_t grid = tiles_m * tiles_n < units ? tiles_m * tiles_n : units;
+    kernel<<<grid, 256, lds, stream>>>((const gd_half *)x, (const gd_half *)w, (const gd_half *)bias, nullptr, nullptr,
+                                       nullptr, p, tiles_m, tiles_n, 1u,
+                                       gd_tile_rope{cos_rows, sin_rows, cache_row, (gd_half *)q, (gd_half *)k_cache,
+                                                    (gd_half *)v_cache, hd, half_d});
+    return (int)hipGetLastError();
+}
+
+/* Row tiles of 256 that fill whole rounds of `units` workgroups for an [M, N] output in 256-column tiles: the rows
+ * the rope form takes; the rest (a partly filled last round, a ragged last row tile) goes through the plain
+ * projection and the table-driven rotation kernel. */
+extern "C" uint32_t gd_hip_linear_tile_rope_head_rows(uint32_t M, uint32_t N, int compute_units)
+{
+    const uint32_t units = ((uint32_t)(compute_units > 0 ? compute_units : 256) + 7u) & ~7u;
+    const uint32_t tiles_n = (N + 255u) / 256u, whole_m = M / 256u;
+    const uint64_t tiles = (uint64_t)whole_m * tiles_n;
+    const uint64_t rounds = tiles / units;
+    uint32_t head_m = rounds != 0u ? (uint32_t)(rounds * units / tiles_n) : 0u;
+    /* a few tiles beyond whole rounds cost less than they would in small tiles only when the remainder is nearly a
+     * round itself */
+    if (tiles - (uint64_t)head_m * tiles_n >= (uint64_t)units * 3u / 4u) head_m = whole_m;
+    return head_m * 256u;
 }

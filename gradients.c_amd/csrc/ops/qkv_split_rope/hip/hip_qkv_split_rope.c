@@ -113,18 +113,59 @@ gd_status gd_backend_qkv_rope_append_packed(gd_backend *backend, const gd_backen
     if (tokens <= 0 || batch <= 0 || batch > (int64_t)INT32_MAX || pos_ids->shape[0] != tokens ||
         cache_pos->shape[0] != batch || cu_seqlens->shape[0] != batch + 1 || k_cache->shape[2] != (int64_t)n_heads ||
         k_cache->shape[3] != (int64_t)head_dim || (uint64_t)qkv->shape[1] != (uint64_t)n_heads * head_dim * 3u ||
-        !out_ok(q, tokens, n_heads, head_dim) || !out_ok(k, tokens, n_heads, head_dim) ||
-        !out_ok(v, tokens, n_heads, head_dim) || k_cache->shape[1] > (int64_t)INT32_MAX || !(args->theta > 0.0f) ||
+        !out_ok(q, tokens, n_heads, head_dim) || (k == NULL) != (v == NULL) ||
+        (k != NULL && (!out_ok(k, tokens, n_heads, head_dim) || !out_ok(v, tokens, n_heads, head_dim))) ||
+        k_cache->shape[1] > (int64_t)INT32_MAX || !(args->theta > 0.0f) ||
         args->n_dims != head_dim || ((pos_ids->offset | cache_pos->offset | cu_seqlens->offset) & 3u) != 0u ||
         (uint64_t)tokens * n_heads * head_dim / 2u > 0x7fffffffull * 256u)
         return GD_ERR_INVALID_ARGUMENT;
     /* vector kernel only: NeoX pairing, head size a multiple of 16, 16-byte aligned tensors */
     if (args->interleaved != 0u || (head_dim % 16u) != 0u ||
-        ((qkv->offset | q->offset | k->offset | v->offset | k_cache->offset | v_cache->offset) & 15u) != 0u)
+        ((qkv->offset | q->offset | (k != NULL ? k->offset | v->offset : 0u) | k_cache->offset | v_cache->offset) & 15u) != 0u)
         return GD_ERR_UNSUPPORTED;
     return gd_hip_finish_op(backend, gd_hip_launch_qkv_rope_append_packed(
         backend->stream, gd_hip_view_ptr(qkv), (const int32_t *)gd_hip_view_ptr(pos_ids),
         (const int32_t *)gd_hip_view_ptr(cache_pos), (const int32_t *)gd_hip_view_ptr(cu_seqlens), (uint32_t)batch,
-        gd_hip_view_ptr(q), gd_hip_view_ptr(k), gd_hip_view_ptr(v), gd_hip_view_ptr(k_cache), gd_hip_view_ptr(v_cache),
-        (uint64_t)tokens, n_heads, head_dim, (uint32_t)k_cache->shape[1], args->theta));
+        gd_hip_view_ptr(q), k != NULL ? gd_hip_view_ptr(k) : NULL, v != NULL ? gd_hip_view_ptr(v) : NULL,
+        gd_hip_view_ptr(k_cache), gd_hip_view_ptr(v_cache), (uint64_t)tokens, n_heads, head_dim,
+        (uint32_t)k_cache->shape[1], args->theta));
+}
+
+int gd_hip_launch_rope_table_packed(hipStream_t stream, const int32_t *pos, const int32_t *cu, const int32_t *seq_pos,
+                                    uint32_t batch, float *cos_rows, float *sin_rows, int32_t *cache_row, uint64_t tokens,
+                                    uint32_t head_dim, uint32_t tmax, float theta);
+
+/* Angles and cache rows of the packed prompt rows, once per prefill (see the header). */
+gd_status gd_backend_rope_table_packed(gd_backend *backend, const gd_backend_tensor_view *pos_ids,
+                                       const gd_backend_tensor_view *cache_pos, const gd_backend_tensor_view *cu_seqlens,
+                                       const gd_backend_tensor_view *cos_rows, const gd_backend_tensor_view *sin_rows,
+                                       const gd_backend_tensor_view *cache_rows, uint32_t head_dim, uint32_t tmax,
+                                       const gd_backend_rope_args *args)
+{
+    int64_t tokens, batch;
+    if (backend == NULL || args == NULL || !gd_hip_view_ok(pos_ids) || !gd_hip_view_ok(cache_pos) ||
+        !gd_hip_view_ok(cu_seqlens) || !gd_hip_view_ok(cos_rows) || !gd_hip_view_ok(sin_rows) ||
+        !gd_hip_view_ok(cache_rows) || pos_ids->rank != 1u || cache_pos->rank != 1u || cu_seqlens->rank != 1u ||
+        cos_rows->rank != 2u || sin_rows->rank != 2u || cache_rows->rank != 1u || head_dim == 0u || tmax == 0u)
+        return GD_ERR_INVALID_ARGUMENT;
+    if (pos_ids->dtype != GD_BACKEND_DTYPE_I32 || cache_pos->dtype != GD_BACKEND_DTYPE_I32 ||
+        cu_seqlens->dtype != GD_BACKEND_DTYPE_I32 || cache_rows->dtype != GD_BACKEND_DTYPE_I32 ||
+        cos_rows->dtype != GD_BACKEND_DTYPE_F32 || sin_rows->dtype != GD_BACKEND_DTYPE_F32)
+        return GD_ERR_UNSUPPORTED;
+    tokens = pos_ids->shape[0];
+    batch = cache_pos->shape[0];
+    if (tokens <= 0 || batch <= 0 || cu_seqlens->shape[0] != batch + 1 || cache_rows->shape[0] != tokens ||
+        cos_rows->shape[0] != (tokens + 31) / 32 * 32 || sin_rows->shape[0] != cos_rows->shape[0] || (head_dim % 16u) != 0u ||
+        cos_rows->shape[1] != (int64_t)(head_dim / 2u) || sin_rows->shape[1] != (int64_t)(head_dim / 2u) ||
+        (uint64_t)batch * (uint64_t)tmax > (uint64_t)INT32_MAX || !(args->theta > 0.0f) || args->n_dims != head_dim ||
+        ((pos_ids->offset | cache_pos->offset | cu_seqlens->offset | cache_rows->offset | cos_rows->offset |
+          sin_rows->offset) & 3u) != 0u ||
+        ((cos_rows->offset | sin_rows->offset) & 15u) != 0u || (uint64_t)cos_rows->shape[0] * (head_dim / 2u) > 0x7fffffffull)
+        return GD_ERR_INVALID_ARGUMENT;
+    if (args->interleaved != 0u) return GD_ERR_UNSUPPORTED;
+    return gd_hip_finish_op(backend, gd_hip_launch_rope_table_packed(
+        backend->stream, (const int32_t *)gd_hip_view_ptr(pos_ids), (const int32_t *)gd_hip_view_ptr(cu_seqlens),
+        (const int32_t *)gd_hip_view_ptr(cache_pos), (uint32_t)batch, (float *)gd_hip_view_ptr(cos_rows),
+        (float *)gd_hip_view_ptr(sin_rows), (int32_t *)gd_hip_view_ptr(cache_rows), (uint64_t)tokens, head_dim, tmax,
+        args->theta));
 }

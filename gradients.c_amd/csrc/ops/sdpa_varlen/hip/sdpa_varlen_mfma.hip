@@ -35,6 +35,8 @@ struct gd_hip_sdpa_varlen_params {
     uint32_t n_rows, batch, hq, hkv, dh;
     uint32_t causal, window, prefix_len, max_seqlen;
     float scale;
+    uint32_t kv_tmax; /* 0: k and v are packed like q; otherwise caches [batch, kv_tmax, hkv, dh], token t of
+                         segment b in cache row t of sequence b */
 };
 
 __device__ __forceinline__ bool gd_vl_allowed(int i, int j, int causal, int window, int prefix_len)
@@ -126,6 +128,10 @@ gd_sdpa_varlen_mfma_kernel(const gd_half *__restrict__ q, const gd_half *__restr
     }
     if (b == p.batch || end > (int)p.n_rows) return;
     const int T_len = end - start;
+    if (p.kv_tmax != 0u && (uint32_t)T_len > p.kv_tmax) return; /* a segment its cache cannot hold: out stays */
+    /* first and last row of K and V this workgroup may touch */
+    const uint32_t kv_first = p.kv_tmax != 0u ? b * p.kv_tmax : (uint32_t)start;
+    const uint32_t kv_last = p.kv_tmax != 0u ? b * p.kv_tmax + (p.kv_tmax - 1u) : p.n_rows - 1u;
     const int i0 = (int)((pair - seen) * BQ);
     const int causal = (int)p.causal, window = (int)p.window, prefix = (int)p.prefix_len;
 
@@ -158,7 +164,7 @@ gd_sdpa_varlen_mfma_kernel(const gd_half *__restrict__ q, const gd_half *__restr
         for (int t = 0; t < LOADS; ++t) {
             const uint32_t r0 = (wave * (uint32_t)LOADS + (uint32_t)t) * RPL;
             const uint32_t r = r0 + lane / CPR, pos = lane % CPR;
-            const uint32_t grow = min((uint32_t)(start + jb) + r, p.n_rows - 1u); /* stays inside the tensor */
+            const uint32_t grow = min(kv_first + (uint32_t)jb + r, kv_last); /* stays inside the tensor */
             const uint32_t ck = pos ^ (D == 128 ? (r & 15u) : ((r >> 1) & 7u));
             const uint32_t cv = pos ^ (D == 128 ? ((r & 3u) << 2) : (((r >> 1) & 1u) << 2));
             const uint32_t dst = lds_base + (stage * 2u * TILE_CHUNKS + r0 * CPR) * 16u;
@@ -323,9 +329,10 @@ gd_sdpa_varlen_mfma_kernel(const gd_half *__restrict__ q, const gd_half *__restr
 extern "C" int gd_hip_launch_sdpa_varlen_mfma(hipStream_t stream, const void *q, const void *k, const void *v,
                                               const int32_t *cu, void *out, uint32_t n_rows, uint32_t batch,
                                               uint32_t hq, uint32_t hkv, uint32_t dh, uint32_t causal, uint32_t window,
-                                              uint32_t prefix_len, uint32_t max_seqlen, float scale)
+                                              uint32_t prefix_len, uint32_t max_seqlen, float scale,
+                                              uint32_t kv_tmax)
 {
-    gd_hip_sdpa_varlen_params p = {n_rows, batch, hq, hkv, dh, causal, window, prefix_len, max_seqlen, scale};
+    gd_hip_sdpa_varlen_params p = {n_rows, batch, hq, hkv, dh, causal, window, prefix_len, max_seqlen, scale, kv_tmax};
     const uint64_t pairs = (uint64_t)(n_rows + 127u) / 128u + batch; /* upper bound of sum ceil(len_b / 128) */
     const uint64_t blocks = pairs * hq;
     if (n_rows == 0u || blocks == 0u) return (int)hipSuccess;

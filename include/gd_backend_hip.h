@@ -245,6 +245,20 @@ gd_status gd_backend_sdpa_varlen(gd_backend *backend, const gd_backend_tensor_vi
                                  const gd_backend_tensor_view *stats,
                                  const gd_backend_sdpa_varlen_args *args);
 
+/* gd_backend_sdpa_varlen whose keys and values are read from the caches the packed prefill has just appended them
+ * to: k_cache / v_cache [B,Tmax,Hkv,D] with B = number of segments, token t of segment b in cache row t of sequence
+ * b (the prefill appends at position 0).  Same kernel, same arithmetic and masks as gd_backend_sdpa_varlen on packed
+ * k / v holding the same rows; what it saves is writing the packed k / v and reading them back.  A segment longer
+ * than Tmax leaves its rows of `out` untouched.  F16, head size 64 or 128, caches below 4 GiB
+ * (GD_ERR_UNSUPPORTED otherwise: use gd_backend_sdpa_varlen on packed rows).  No reference counterpart (the
+ * reference's prefill reads the packed rows: examples/gpt_lm/gpt_lm_shared.c:896-940). */
+gd_status gd_backend_sdpa_varlen_cached(gd_backend *backend, const gd_backend_tensor_view *q,
+                                        const gd_backend_tensor_view *k_cache,
+                                        const gd_backend_tensor_view *v_cache,
+                                        const gd_backend_tensor_view *cu_seqlens,
+                                        const gd_backend_tensor_view *out,
+                                        const gd_backend_sdpa_varlen_args *args);
+
 /* backend.h:680-685, 710-729.  q/out [B,Tq,Hq,D], caches [B,Tmax,Hkv,D].
  * `sdpa_decode` takes a rank-0 I32 position tensor, `_at` a host scalar in
  * args->cache_pos, `_positions` an I32 [B] tensor.  A negative position leaves
@@ -403,7 +417,8 @@ gd_status gd_backend_qkv_rope_append(gd_backend *backend, const gd_backend_tenso
  * [B,Tmax,H,D], under the rules of gd_backend_kv_cache_append_packed (nothing is appended unless cu_seqlens starts at
  * 0; a sequence with a negative position or whose rows do not fit behind it keeps its caches).  Same arithmetic as
  * the two separate operators (values bit for bit; rotated elements within one F16 unit in the last place of theirs);
- * the appended rows are the rows written to k / v and are not read back from memory.  NeoX pairing,
+ * the appended rows are the rows written to k / v and are not read back from memory.  k and v may both be NULL: then
+ * the rows only go into the caches (for a caller that reads them there: gd_backend_sdpa_varlen_cached).  NeoX pairing,
  * head_dim % 16 == 0, F16 only (GD_ERR_UNSUPPORTED otherwise: use the separate operators).  No reference counterpart
  * (reference order of the two operators: examples/gpt_lm/gpt_lm_shared.c:896-917). */
 gd_status gd_backend_qkv_rope_append_packed(gd_backend *backend, const gd_backend_tensor_view *qkv,
@@ -414,6 +429,45 @@ gd_status gd_backend_qkv_rope_append_packed(gd_backend *backend, const gd_backen
                                             const gd_backend_tensor_view *k_cache,
                                             const gd_backend_tensor_view *v_cache, uint32_t n_heads, uint32_t head_dim,
                                             const gd_backend_rope_args *args);
+
+/* The packed prefill's rotation and cache append inside the qkv projection, in two calls.
+ *
+ * gd_backend_rope_table_packed, once per prefill: for the N packed prompt rows the angles of their positions,
+ * cos_rows / sin_rows [ceil(N/32)*32, head_dim/2] F32 (pair p of row n: angle = float(pos_ids[n]) * exp2(p *
+ * -2*log2(theta) / head_dim), as gd_backend_qkv_split_rope_forward computes them; stored for the reads of the
+ * projection's epilogue, not row by row: element (n, p) sits at (((n/32) * (head_dim/16) + p/8) * 2 + (p/4)%2) * 128 +
+ * (n%32) * 4 + p%4; the rows behind N are not written), and cache_rows [N] I32: the row of a
+ * [B,Tmax,H,D] cache seen as [B*Tmax, H*D] that token t of sequence b goes to, b*tmax + cache_pos[b] + t, under the
+ * rules of gd_backend_kv_cache_append_packed (nothing unless cu_seqlens starts at 0; a sequence with a negative
+ * position or whose rows do not fit behind it is skipped), -1 for a row that is not appended.  NeoX pairing only.
+ *
+ * gd_backend_linear_qkv_rope_packed, once per layer: x [N,K] times w [3*H*D, K] (plus bias; bias_mode 0 none,
+ * 1 added in F32 before the rounding as gd_backend_linear does, 2 added in F16 to the rounded product), the
+ * projection rounded to F16, q and k rotated in F32 with the table's angles and rounded again, then rotated q to
+ * q [N,H,D] and rotated k and copied v to row cache_rows[n] of k_cache / v_cache: the results of
+ * gd_backend_linear + gd_backend_qkv_split_rope_forward + gd_backend_kv_cache_append_packed (values bit for bit,
+ * rotated elements within one F16 unit in the last place), with no [N, 3*H*D] intermediate written and read back:
+ * the rotation rides in the epilogue of the 256 x 256 tiles.  The rows of a last, partly filled round of tiles go
+ * through the plain projection into `work` [N, 3*H*D] (only those rows of it are written) and a rotation kernel
+ * driven by the same table.  Packed k / v rows are not produced: read them from the caches
+ * (gd_backend_sdpa_varlen_cached).  F16, [N,K] weights, head size 64 or 128, H*D a multiple of 256, K a multiple
+ * of 64, 16-byte aligned rows (GD_ERR_UNSUPPORTED otherwise: use the separate operators).  No reference counterpart
+ * (reference order of the operators: examples/gpt_lm/gpt_lm_shared.c:880-917). */
+gd_status gd_backend_rope_table_packed(gd_backend *backend, const gd_backend_tensor_view *pos_ids,
+                                       const gd_backend_tensor_view *cache_pos,
+                                       const gd_backend_tensor_view *cu_seqlens,
+                                       const gd_backend_tensor_view *cos_rows, const gd_backend_tensor_view *sin_rows,
+                                       const gd_backend_tensor_view *cache_rows, uint32_t head_dim, uint32_t tmax,
+                                       const gd_backend_rope_args *args);
+gd_status gd_backend_linear_qkv_rope_packed(gd_backend *backend, const gd_backend_matrix_view *x,
+                                            const gd_backend_matrix_view *w, const gd_backend_vector_view *bias,
+                                            const gd_backend_tensor_view *cos_rows,
+                                            const gd_backend_tensor_view *sin_rows,
+                                            const gd_backend_tensor_view *cache_rows, const gd_backend_tensor_view *q,
+                                            const gd_backend_tensor_view *k_cache,
+                                            const gd_backend_tensor_view *v_cache,
+                                            const gd_backend_matrix_view *work, uint32_t n_heads, uint32_t head_dim,
+                                            uint32_t bias_mode);
 
 /* out[i,:] = src[rows[i],:]; replaces the reference's per-sequence slice +
  * concat when the last prompt rows are selected

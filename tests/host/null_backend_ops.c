@@ -26,6 +26,7 @@ GD_NULL_OP(gd_backend_kv_cache_append_positions)
 GD_NULL_OP(gd_backend_linear)
 GD_NULL_OP(gd_backend_linear_last_kernel)
 GD_NULL_OP(gd_backend_linear_nt)
+GD_NULL_OP(gd_backend_linear_qkv_rope_packed)
 GD_NULL_OP(gd_backend_matmul)
 GD_NULL_OP(gd_backend_matmul_nt)
 GD_NULL_OP(gd_backend_minimax_m3_index_topk)
@@ -35,6 +36,7 @@ GD_NULL_OP(gd_backend_qkv_rope_append_packed)
 GD_NULL_OP(gd_backend_qkv_split_rope_forward)
 GD_NULL_OP(gd_backend_rand_uniform)
 GD_NULL_OP(gd_backend_rms_norm_forward)
+GD_NULL_OP(gd_backend_rope_table_packed)
 GD_NULL_OP(gd_backend_sample_advance)
 GD_NULL_OP(gd_backend_sdpa_decode)
 GD_NULL_OP(gd_backend_sdpa_decode_at)
@@ -42,5 +44,6 @@ GD_NULL_OP(gd_backend_sdpa_decode_last_kernel)
 GD_NULL_OP(gd_backend_sdpa_decode_positions)
 GD_NULL_OP(gd_backend_sdpa_decode_positions_noalloc)
 GD_NULL_OP(gd_backend_sdpa_varlen)
+GD_NULL_OP(gd_backend_sdpa_varlen_cached)
 GD_NULL_OP(gd_backend_swiglu_split_forward)
 GD_NULL_OP(gd_backend_swiglu_split_linear)

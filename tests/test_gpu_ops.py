@@ -642,6 +642,49 @@ def test_varlen_ignores_values_of_the_next_segment(backend, arena, oracle):
     _close(got[:70], oracle.sdpa_varlen(q, kk, vv, cu, 0.125, False, 0, 0, 0)[:70])
 
 
+@pytest.mark.parametrize("H,Hkv,D,causal,window,prefix", [
+    (4, 4, 64, True, 0, 0), (4, 2, 128, True, 0, 0), (2, 2, 128, True, 100, 0), (2, 1, 128, True, 40, 150),
+    (2, 2, 64, False, 0, 0)])
+def test_varlen_reads_keys_and_values_from_the_caches(backend, arena, oracle, gda, H, Hkv, D, causal, window, prefix):
+    """gd_backend_sdpa_varlen_cached (token t of segment b in row t of cache b) against gd_backend_sdpa_varlen on packed
+    rows holding the same keys and values: the same kernel on the same numbers, so bit for bit, and against the oracle.
+    Cache rows behind a segment's length hold NaN keys and infinite values and must not leak; a segment that fills
+    its cache to the last row; an empty segment; a segment longer than the cache leaves its rows of out untouched."""
+    lens = np.array([300, 128, 0, 577, 64, 65, 1], np.int32)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    B, N, Tmax = len(lens), int(cu[-1]), 577
+    q, k, v = oracle.normal_f16((N, H, D), 770), oracle.normal_f16((N, Hkv, D), 771), oracle.normal_f16((N, Hkv, D), 772)
+    kc = np.full((B, Tmax, Hkv, D), np.nan, np.float16)
+    vc = np.full((B, Tmax, Hkv, D), np.inf, np.float16)
+    for b in range(B):
+        kc[b, :lens[b]], vc[b, :lens[b]] = k[cu[b]:cu[b + 1]], v[cu[b]:cu[b + 1]]
+    scale = float(1.0 / np.sqrt(D))
+    tq, tcu = arena.from_numpy(q), arena.from_numpy(cu)
+    packed = arena.from_numpy(np.zeros(q.shape, np.float16))
+    backend.sdpa_varlen(tq, arena.from_numpy(k), arena.from_numpy(v), tcu, packed, scale, causal, window, prefix, 0)
+    cached = arena.from_numpy(np.zeros(q.shape, np.float16))
+    backend.sdpa_varlen_cached(tq, arena.from_numpy(kc), arena.from_numpy(vc), tcu, cached, scale, causal, window, prefix, 0)
+    got = cached.read()
+    assert np.array_equal(_bits(got), _bits(packed.read()))
+    _close(got, oracle.sdpa_varlen(q, k, v, cu, scale, causal, window, prefix, 0))
+    # a cache of 400 rows cannot hold the segment of 577: its rows stay as they were, all others are computed
+    short = arena.from_numpy(np.full(q.shape, 5.0, np.float16))
+    backend.sdpa_varlen_cached(tq, arena.from_numpy(np.ascontiguousarray(kc[:, :400])),
+                               arena.from_numpy(np.ascontiguousarray(vc[:, :400])), tcu, short, scale, causal, window, prefix, 0)
+    got_short = short.read()
+    assert np.all(got_short[cu[3]:cu[4]] == 5.0)
+    keep = np.r_[0:cu[3], cu[4]:N]
+    assert np.array_equal(_bits(got_short[keep]), _bits(got[keep]))
+    # F32 tensors, other head sizes and a batch that is not the number of segments are refused, not mis-run
+    a = gda.SdpaVarlenArgs(scale, 1, 0, 0, 0, 0)
+    k5 = arena.alloc((B + 1, 8, Hkv, D), gda.F16)
+    assert backend.call("gd_backend_sdpa_varlen_cached", tq.view(), k5.view(), k5.view(), tcu.view(), cached.view(),
+                        C.byref(a)) == gda.INVALID_ARGUMENT
+    k32 = arena.alloc((B, 8, Hkv, D), gda.F32)
+    assert backend.call("gd_backend_sdpa_varlen_cached", tq.view(), k32.view(), k32.view(), tcu.view(), cached.view(),
+                        C.byref(a)) == gda.UNSUPPORTED
+
+
 def test_varlen_max_seqlen_truncates(backend, arena, oracle):
     cu = np.array([0, 50, 60], np.int32)
     q, k, v = (oracle.normal_f16((60, 2, 64), s) for s in (710, 711, 712))
@@ -1425,6 +1468,83 @@ def test_qkv_rope_append_equals_separate_ops(backend, arena, oracle, B, H, D):
     assert np.array_equal(_bits(vc.read()), _bits(ov))
 
 
+@pytest.mark.parametrize("H,D,K,N", [(4, 128, 128, 11100), (8, 64, 192, 11010), (2, 128, 128, 300)])
+def test_linear_qkv_rope_packed_equals_separate_ops(backend, arena, oracle, gda, H, D, K, N):
+    """The packed prefill's qkv projection with rotation, split and cache append in its epilogue
+    (gd_backend_rope_table_packed once, gd_backend_linear_qkv_rope_packed per layer) against the separate operators
+    gd_backend_linear_nt -> gd_backend_qkv_split_rope_forward -> gd_backend_kv_cache_append_packed and against the
+    oracle.  11,100 rows of 6 column tiles fill one round of 256 tiles (42 row tiles through the tile kernel's rotation
+    epilogue, the rest through the plain projection and the table-driven rotation kernel); 300 rows take the second
+    path only.  Values bit for bit; rotated elements within one F16 unit in the last place; the skip rules of the
+    packed append: a sequence with a negative position, one whose rows do not fit, an empty one."""
+    rng = np.random.default_rng(2900 + N)
+    B, Tmax = 9, 2048
+    cuts = np.sort(rng.choice(np.arange(1, N), B - 2, replace=False))
+    cu = np.concatenate([[0], cuts[:3], [cuts[3]], cuts[3:], [N]]).astype(np.int32)  # sequence 4 is empty
+    lens = np.diff(cu)
+    cache_pos = np.zeros(B, np.int32)
+    cache_pos[1], cache_pos[2] = -1, 5
+    x = oracle.normal_f16((N, K), 2901, 1.0)
+    w = oracle.normal_f16((3 * H * D, K), 2902, 1.0 / np.sqrt(K))
+    bias = oracle.normal_f16((3 * H * D,), 2903, 0.1)
+    pos = oracle.uniform_i32(N, 2904, 0, 4000)
+    k0, v0 = oracle.normal_f16((B, Tmax, H, D), 2905), oracle.normal_f16((B, Tmax, H, D), 2906)
+    tx, tw, tb = arena.from_numpy(x), arena.from_numpy(w), arena.from_numpy(bias)
+    tpos, tcp, tcu = arena.from_numpy(pos), arena.from_numpy(cache_pos), arena.from_numpy(cu)
+    # separate operators
+    qkv = arena.alloc((N, 3 * H * D), gda.F16)
+    backend.linear_nt(tx, tw, tb, qkv)
+    q2, k2, v2 = (arena.from_numpy(np.full((N, H, D), 7.0, np.float16)) for _ in range(3))
+    kc2, vc2 = arena.from_numpy(k0), arena.from_numpy(v0)
+    backend.qkv_split_rope_forward(qkv, tpos, q2, k2, v2, H, D)
+    backend.kv_cache_append_packed(kc2, vc2, tcp, tcu, k2, v2)
+    # table + projection with the rotation epilogue
+    Npad = (N + 31) // 32 * 32
+    cos_rows, sin_rows = arena.alloc((Npad, D // 2), gda.F32), arena.alloc((Npad, D // 2), gda.F32)
+    cache_rows = arena.alloc((N,), gda.I32)
+    backend.rope_table_packed(tpos, tcp, tcu, cos_rows, sin_rows, cache_rows, D, Tmax)
+    rows = cache_rows.read()
+    want_rows = np.full(N, -1, np.int64)
+    for b in range(B):
+        if cache_pos[b] >= 0 and cache_pos[b] + lens[b] <= Tmax:
+            want_rows[cu[b]:cu[b + 1]] = b * Tmax + cache_pos[b] + np.arange(lens[b])
+    assert np.array_equal(rows, want_rows)
+    ang = pos[:, None].astype(np.float64) * np.exp2(np.arange(D // 2) * (-2.0 * np.log2(10000.0) / D))[None, :]
+    nn, pp = np.arange(N)[:, None], np.arange(D // 2)[None, :]   # where the tables keep element (n, p)
+    at = (((nn // 32) * (D // 16) + pp // 8) * 2 + (pp // 4) % 2) * 128 + (nn % 32) * 4 + pp % 4
+    assert np.allclose(cos_rows.read().reshape(-1)[at], np.cos(ang), atol=3e-3)
+    assert np.allclose(sin_rows.read().reshape(-1)[at], np.sin(ang), atol=3e-3)
+    q1 = arena.from_numpy(np.full((N, H, D), 7.0, np.float16))
+    kc1, vc1 = arena.from_numpy(k0), arena.from_numpy(v0)
+    work = arena.alloc((N, 3 * H * D), gda.F16)
+    backend.linear_qkv_rope_packed(tx, tw, tb, cos_rows, sin_rows, cache_rows, q1, kc1, vc1, work, H, D, 2)
+    assert np.array_equal(_bits(vc1.read()), _bits(vc2.read()))
+    for a, b in ((q1, q2), (kc1, kc2)):
+        a, b = a.read(), b.read()
+        ulp = np.spacing(np.maximum(np.abs(a), np.abs(b)).astype(np.float16)).astype(np.float32)
+        assert np.all(np.abs(a.astype(np.float32) - b.astype(np.float32)) <= ulp)
+        assert np.count_nonzero(_bits(a) != _bits(b)) <= max(2, a.size // 300)
+    skipped = [b for b in range(B) if not (cache_pos[b] >= 0 and cache_pos[b] + lens[b] <= Tmax)]
+    assert 1 in skipped
+    for b in skipped:
+        assert np.array_equal(_bits(kc1.read()[b]), _bits(k0[b])) and np.array_equal(_bits(vc1.read()[b]), _bits(v0[b]))
+    qo, ko, vo = oracle.qkv_split_rope(oracle.linear_nt(x, w, bias), pos, H, D)
+    _close(q1.read(), qo, atol=8e-3)
+    got_k, got_v = kc1.read(), vc1.read()
+    for b in (b for b in range(B) if b not in skipped):
+        _close(got_k[b, cache_pos[b]:cache_pos[b] + lens[b]], ko[cu[b]:cu[b + 1]], atol=8e-3)
+        _close(got_v[b, cache_pos[b]:cache_pos[b] + lens[b]], vo[cu[b]:cu[b + 1]], atol=8e-3)
+    # refused, not mis-run: a head size the rotation epilogue does not cover
+    q96 = arena.alloc((N, 4, 96), gda.F16)
+    kc96 = arena.alloc((B, 16, 4, 96), gda.F16)
+    c96 = arena.alloc((Npad, 48), gda.F32)
+    w96 = arena.alloc((3 * 4 * 96, K), gda.F16)
+    wk96 = arena.alloc((N, 3 * 4 * 96), gda.F16)
+    b96 = arena.alloc((3 * 4 * 96,), gda.F16)
+    assert backend.call("gd_backend_linear_qkv_rope_packed", tx.matrix(), w96.matrix(), b96.vector(), c96.view(), c96.view(),
+                        cache_rows.view(), q96.view(), kc96.view(), kc96.view(), wk96.matrix(), 4, 96, 2) == gda.UNSUPPORTED
+
+
 # ---- sampling front end -----------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("H,D", [(8, 64), (16, 128), (3, 32)])
@@ -1446,6 +1566,11 @@ def test_qkv_rope_append_packed_equals_separate_ops(backend, arena, oracle, gda,
         q1, k1, v1 = (arena.from_numpy(np.full((N, H, D), 7.0, np.float16)) for _ in range(3))
         kc1, vc1 = arena.from_numpy(k0), arena.from_numpy(v0)
         backend.qkv_rope_append_packed(tqkv, tpos, tcp, tcu, q1, k1, v1, kc1, vc1, H, D)
+        # without the packed k / v outputs (a caller that reads the rows from the caches): q and the caches as before
+        q3, kc3, vc3 = arena.from_numpy(np.full((N, H, D), 7.0, np.float16)), arena.from_numpy(k0), arena.from_numpy(v0)
+        backend.qkv_rope_append_packed(tqkv, tpos, tcp, tcu, q3, None, None, kc3, vc3, H, D)
+        for a, b in ((q3, q1), (kc3, kc1), (vc3, vc1)):
+            assert np.array_equal(_bits(a.read()), _bits(b.read()))
         q2, k2, v2 = (arena.from_numpy(np.full((N, H, D), 7.0, np.float16)) for _ in range(3))
         kc2, vc2 = arena.from_numpy(k0), arena.from_numpy(v0)
         backend.qkv_split_rope_forward(tqkv, tpos, q2, k2, v2, H, D)
