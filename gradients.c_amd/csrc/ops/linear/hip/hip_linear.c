@@ -307,12 +307,18 @@ gd_status gd_backend_linear_qkv_rope_packed(gd_backend *backend, const gd_backen
     if (head_rows < p.M) {
         gd_hip_linear_params tail = p;
         char *work_rows = (char *)gd_hip_matrix_ptr(work) + (size_t)head_rows * work->row_bytes;
-        tail.M = p.M - head_rows;
-        e = gd_hip_launch_linear(backend->stream, (const char *)gd_hip_matrix_ptr(x) + (size_t)head_rows * x->row_bytes,
-                                 gd_hip_matrix_ptr(w), bias != NULL ? gd_hip_vector_ptr(bias) : NULL, NULL, NULL, work_rows,
-                                 &tail, 1, 0, 1, 2 * backend->compute_units, NULL, backend->linear_wide,
-                                 &backend->last_linear_family);
+        /* the projection of the tail rows in whole 128-row tiles: it starts up to 127 rows early (rows of `work`
+         * nobody reads), so that no ragged row tile leaves the tile kernel's direct staging path */
+        const uint32_t tail_rows = p.M - head_rows;
+        const uint32_t up = (tail_rows + 127u) / 128u * 128u;
+        const uint32_t first = tail_rows >= 128u && up <= p.M ? p.M - up : head_rows;
+        tail.M = p.M - first;
+        e = gd_hip_launch_linear(backend->stream, (const char *)gd_hip_matrix_ptr(x) + (size_t)first * x->row_bytes,
+                                 gd_hip_matrix_ptr(w), bias != NULL ? gd_hip_vector_ptr(bias) : NULL, NULL, NULL,
+                                 (char *)gd_hip_matrix_ptr(work) + (size_t)first * work->row_bytes, &tail, 1, 0, 1,
+                                 2 * backend->compute_units, NULL, backend->linear_wide, &backend->last_linear_family);
         if (e != 0) return gd_hip_finish_op(backend, e);
+        tail.M = tail_rows;
         e = gd_hip_launch_qkv_rope_rows(backend->stream, work_rows, (const float *)gd_hip_view_ptr(cos_rows),
                                         (const float *)gd_hip_view_ptr(sin_rows),
                                         (const int32_t *)gd_hip_view_ptr(cache_rows), gd_hip_view_ptr(q),

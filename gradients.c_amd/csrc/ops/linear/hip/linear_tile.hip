@@ -421,14 +421,20 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
             if (READS) {
 #pragma unroll
                 for (uint32_t r = min(idx * RPM, NR); r < min((idx + 1u) * RPM, NR); ++r) {
-                    /* a0 b0 a1 b1 ...: the order in which the next step consumes them */
-                    if ((r & 1u) == 0u) qa[NXT][r >> 1] = direct_frag_a(cA, rks, r >> 1);
+                    /* a0 b0 a1 b1 ...: the order in which the next step consumes them; behind the shorter of the
+                     * two lists the rest of the longer one */
+                    constexpr uint32_t BOTH = 2u * (WM < WN ? WM : WN);
+                    if (r >= BOTH) {
+                        if constexpr (WM > WN) qa[NXT][r - BOTH / 2u] = direct_frag_a(cA, rks, r - BOTH / 2u);
+                        else qb[NXT][r - BOTH / 2u] = direct_frag_b(cB, rks, r - BOTH / 2u);
+                    } else if ((r & 1u) == 0u) qa[NXT][r >> 1] = direct_frag_a(cA, rks, r >> 1);
                     else qb[NXT][r >> 1] = direct_frag_b(cB, rks, r >> 1);
                 }
             }
-            if (LOADS && loads_on && idx >= NM - NL / LPM) {
+            constexpr uint32_t LI = (NL + LPM - 1u) / LPM; /* matrix instructions that carry loads */
+            if (LOADS && loads_on && idx >= NM - LI) {
 #pragma unroll
-                for (uint32_t t = (idx - (NM - NL / LPM)) * LPM; t < (idx - (NM - NL / LPM) + 1u) * LPM; ++t)
+                for (uint32_t t = (idx - (NM - LI)) * LPM; t < min((idx - (NM - LI) + 1u) * LPM, NL); ++t)
                     direct_load_item(m0, n0, KS == 3u ? kt + 2u : kt + 1u, KS == 3u ? t : NL + t);
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -560,10 +566,8 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
         if (decltype(mode_tag)::value != GD_HIP_EPI_NONE) load_bias();
         epilogue_pass(std::integral_constant<int, 0>{}, mode_tag);
         epilogue_pass(std::integral_constant<int, 1>{}, mode_tag);
-        if (WM > 2) {
-            epilogue_pass(std::integral_constant<int, (WM > 2 ? 2 : 0)>{}, mode_tag);
-            epilogue_pass(std::integral_constant<int, (WM > 2 ? 3 : 0)>{}, mode_tag);
-        }
+        if (WM > 2) epilogue_pass(std::integral_constant<int, (WM > 2 ? 2 : 0)>{}, mode_tag);
+        if (WM > 3) epilogue_pass(std::integral_constant<int, (WM > 3 ? 3 : 0)>{}, mode_tag);
     };
 
     /* Epilogue of a whole 256-column tile whose rows can take 16-byte stores: no workgroup barriers.  A wavefront
@@ -634,8 +638,8 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
         };
         pass(std::integral_constant<int, 0>{});
         pass(std::integral_constant<int, 1>{});
-        pass(std::integral_constant<int, (WM > 2 ? 2 : 0)>{});
-        pass(std::integral_constant<int, (WM > 2 ? 3 : 0)>{});
+        if (WM > 2) pass(std::integral_constant<int, (WM > 2 ? 2 : 0)>{});
+        if (WM > 3) pass(std::integral_constant<int, (WM > 3 ? 3 : 0)>{});
     };
     auto epilogue_own_gated = [&](auto mode_tag) __attribute__((always_inline)) {
         if (decltype(mode_tag)::value != GD_HIP_EPI_NONE) load_bias();
@@ -674,8 +678,8 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
         };
         pass(std::integral_constant<int, 0>{});
         pass(std::integral_constant<int, 1>{});
-        pass(std::integral_constant<int, (WM > 2 ? 2 : 0)>{});
-        pass(std::integral_constant<int, (WM > 2 ? 3 : 0)>{});
+        if (WM > 2) pass(std::integral_constant<int, (WM > 2 ? 2 : 0)>{});
+        if (WM > 3) pass(std::integral_constant<int, (WM > 3 ? 3 : 0)>{});
     };
 
     /* ROPE instantiation (whole tiles only; the launcher sees to that): the wavefront's 128 columns lie inside q, k
@@ -881,7 +885,7 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
         auto finish = [&](auto mode_tag) __attribute__((always_inline)) {
             if constexpr (ROPE) {
                 epilogue_own_rope(mode_tag);
-            } else if (WM == 4 && WN == 4 && vector_store && m0 + BM <= p.M && n0 + out_bn <= p.N) {
+            } else if (WM >= 3 && WN == 4 && vector_store && m0 + BM <= p.M && n0 + out_bn <= p.N) {
                 if (gated) epilogue_own_gated(mode_tag);
                 else epilogue_own(mode_tag);
             } else {
@@ -964,7 +968,21 @@ extern "C" int gd_hip_launch_linear_tile(hipStream_t stream, const void *x, cons
             const double whole = (double)((tiles + units - 1u) / units);
             const double cut = (double)(((uint64_t)head_m * tiles_n + units - 1u) / units) +
                                0.35 * (double)((small + 2u * units - 1u) / (2u * units));
-            if (cut + 0.1 < whole) {
+            /* a tail that small tiles would need more than one round for, and that fits one round of 192 x 256
+             * tiles (three row tiles per wavefront instead of four): one launch of those; measured on the
+             * 2048-column projections of the scaled decoder (5,653 tail rows: 720 small tiles on 512 places, or 248
+             * tiles of 192 rows, or 240 when the launch is anchored at the last row, see below) */
+            const uint32_t mid_rows = (tail_rows + 191u) / 192u * 192u;
+            const uint64_t mid = (uint64_t)(mid_rows / 192u) * tiles_n;
+            /* whole tiles only (a ragged row tile would leave the direct staging path and take twice as long as the
+             * others of its round): the launch covers the LAST mid_rows rows, so its first rows, fewer than 192,
+             * are rows of the head launch computed once more, to the same bits (the same products in the same
+             * order, the same epilogue); that needs an output the residual does not alias */
+            const bool apart = rp == nullptr || rp + (size_t)p.M * p.ldr <= yp || yp + (size_t)p.M * p.ldy <= rp;
+            const bool mid_tiles = p.w_is_nk && p.prologue == GD_HIP_PRO_NONE && p.swiglu_cols == 0u &&
+                                   small > 2u * units && mid <= units && mid_rows <= p.M && (p.N % 256u) == 0u &&
+                                   vector_store && apart;
+            if (mid_tiles || cut + 0.1 < whole) {
                 gd_hip_linear_params head = p, tail = p;
                 int e;
                 head.M = head_rows;
@@ -972,10 +990,24 @@ extern "C" int gd_hip_launch_linear_tile(hipStream_t stream, const void *x, cons
                 e = launch_tile<4, 4>(stream, xp, (const gd_half *)w, (const gd_half *)bias, rp, (const gd_half *)norm_w,
                                       yp, head, (uint32_t)vector_store, units);
                 if (e != (int)hipSuccess) return e;
-                return launch_tile<2, 2>(stream, xp + (size_t)head_rows * p.ldx, (const gd_half *)w,
-                                         (const gd_half *)bias, rp != nullptr ? rp + (size_t)head_rows * p.ldr : nullptr,
-                                         (const gd_half *)norm_w, yp + (size_t)head_rows * p.ldy, tail,
-                                         (uint32_t)vector_store, 2u * units);
+                if (mid_tiles) {
+                    const uint32_t first = p.M - mid_rows;
+                    tail.M = mid_rows;
+                    return launch_tile_one<3, 4, true, GD_HIP_PRO_NONE>(
+                        stream, xp + (size_t)first * p.ldx, (const gd_half *)w, (const gd_half *)bias,
+                        rp != nullptr ? rp + (size_t)first * p.ldr : nullptr, (const gd_half *)norm_w,
+                        yp + (size_t)first * p.ldy, tail, (uint32_t)vector_store, units);
+                }
+                /* small tiles: whole row tiles as well when the output allows it (anchored at the last row) */
+                uint32_t first = head_rows;
+                const uint32_t up = (tail_rows + 127u) / 128u * 128u;
+                if (apart && up <= p.M) {
+                    first = p.M - up;
+                    tail.M = up;
+                }
+                return launch_tile<2, 2>(stream, xp + (size_t)first * p.ldx, (const gd_half *)w, (const gd_half *)bias,
+                                         rp != nullptr ? rp + (size_t)first * p.ldr : nullptr, (const gd_half *)norm_w,
+                                         yp + (size_t)first * p.ldy, tail, (uint32_t)vector_store, 2u * units);
             }
         }
         return launch_tile<4, 4>(stream, xp, (const gd_half *)w, (const gd_half *)bias, rp, (const gd_half *)norm_w, yp, p,

@@ -1009,14 +1009,36 @@ def test_many_row_projection_prologues(backend, arena, oracle, M, K, N, nk):
     _close(y.read(), oracle.linear(oracle.rms_norm(x, nw, 1e-5), w_kn, bias))
 
 
+@pytest.mark.parametrize("K", [128, 192])
+def test_many_row_projection_tail_in_192_row_tiles(backend, arena, oracle, K):
+    """13,192 rows onto 2048 columns of an [N,K] weight: 52 x 8 tiles of 256 x 256 are 1.6 rounds on 256 compute units;
+    the first round's 8,192 rows run in those tiles, the 5,000 rows behind them (640 tiles of 128 x 128 would need more
+    than one round of them) in one launch of 27 x 8 tiles of 192 x 256, three row tiles per wavefront, the last row tile
+    ragged.  Whole output against the oracle, plain, with bias, and with bias and residual."""
+    M, N = 13192, 2048
+    x = oracle.normal_f16((M, K), 2500 + K, 1.0)
+    w = oracle.normal_f16((N, K), 2501, 0.05)
+    bias = oracle.normal_f16((N,), 2502, 0.5)
+    res = oracle.normal_f16((M, N), 2503, 1.0)
+    tx, tw, tb, tr = (arena.from_numpy(a) for a in (x, w, bias, res))
+    y = arena.alloc((M, N), 1)
+    backend.fused_linear(tx, tw, None, None, None, y, True, 0, 0)
+    _close(y.read(), oracle.linear_nt(x, w))
+    backend.fused_linear(tx, tw, tb, tr, None, y, True, 2, 0)
+    inter = oracle.linear_nt(x, w, bias)
+    _close(y.read(), oracle.add(res, inter), through=inter)
+
+
 def test_many_row_projection_full_size_sampled(backend, oracle):
     """The packed-prefill projections of BASELINE config 4 at full size (30,229 rows): the qkv projection ([N,K]
     weight, bias added after the F16 rounding) and the down projection ([K,N] weight, F32 bias, residual), operands
-    filled on the device, sampled rows (first, last, both sides of every kind of tile edge) against float64."""
+    filled on the device, sampled rows (first, last, both sides of every kind of tile edge) against float64; and the
+    attention projection with its residual on an [N,K] weight, whose 5,653 rows behind the last whole round of 256 x 256
+    tiles go to one launch of 192 x 256 tiles (rows 24,576 on; tile edges every 192 rows, the last tile ragged)."""
     M = 30229
     big = backend.buffer(900 << 20)
     try:
-        for (K, N, nk) in ((2048, 6144, True), (5632, 2048, False)):
+        for (K, N, nk) in ((2048, 6144, True), (5632, 2048, False), (2048, 2048, True)):
             big.reset()
             x, w = big.alloc((M, K), 1), big.alloc((N, K) if nk else (K, N), 1)
             backend.rand_uniform(x, 9101 + K, -1.0, 1.0)
@@ -1025,14 +1047,17 @@ def test_many_row_projection_full_size_sampled(backend, oracle):
             res = big.alloc((M, N), 1)
             backend.rand_uniform(res, 9104, -1.0, 1.0)
             y = big.alloc((M, N), 1)
-            backend.fused_linear(x, w, big.from_numpy(bias), None if nk else res, None, y, nk, 2 if nk else 1, 0)
+            with_res = not nk or N == 2048
+            backend.fused_linear(x, w, big.from_numpy(bias), res if with_res else None, None, y, nk, 2 if nk else 1, 0)
             wf = w.read().astype(np.float64)
             wf = wf.T if nk else wf
-            for r in (0, 1, 255, 256, 4095, 4096, 17000, 30207, 30208, 30228):
+            for r in (0, 1, 255, 256, 4095, 4096, 17000, 24575, 24576, 24767, 24768, 30143, 30144, 30207, 30208, 30228):
                 xr = x.rows(r, 1).read()[0].astype(np.float64)
                 t = xr @ wf
                 if nk:
                     want = (t.astype(np.float16).astype(np.float32) + bias.astype(np.float32)).astype(np.float16)
+                    if with_res:
+                        want = (res.rows(r, 1).read()[0].astype(np.float32) + want.astype(np.float32)).astype(np.float16)
                 else:
                     u = (t + bias.astype(np.float64)).astype(np.float16)
                     want = (res.rows(r, 1).read()[0].astype(np.float32) + u.astype(np.float32)).astype(np.float16)
