@@ -430,7 +430,8 @@ def long_context_workload(a, oracle, D, which, steps=None, warmup=None, batches=
     for _ in range(batches):
         if which == 3:
             t0 = time.perf_counter()    # configs[4] keeps the session set-up inside its one clock
-        dec.resident_run(steps)
+        # configs[4]: the session's first step ran inside resident_begin, so steps - 1 replays complete its `steps` steps
+        dec.resident_run(steps if which == 3 else steps - 1)
         dec.resident_sync()
         times.append(time.perf_counter() - t0)
     elapsed = _median(times)
