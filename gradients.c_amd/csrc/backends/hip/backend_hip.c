@@ -221,6 +221,11 @@ gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t 
         backend->linear_no_lds_stream = (int)value;
         return GD_OK;
     }
+    if (strcmp(name, "prefill_rope_epilogue") == 0) {
+        if (value != 0 && value != 1) return GD_ERR_INVALID_ARGUMENT;
+        backend->no_prefill_rope_epilogue = value == 0;
+        return GD_OK;
+    }
     if (strcmp(name, "sdpa_waves") == 0 || strcmp(name, "sdpa_unroll") == 0) {
         if (value != 0 && value != 4 && value != 8 && !(value == 2 && name[5] == 'u')) return GD_ERR_INVALID_ARGUMENT;
         if (name[5] == 'w') backend->sdpa_waves = (int)value;

@@ -57,6 +57,8 @@ struct gd_backend {
     int linear_tiles;    /* few-row projections: 16-column tiles per workgroup, 1 / 2 / 4 (0 = automatic) */
     int linear_waves;    /* few-row projections: wavefronts per workgroup = K split, 4 / 8 (0 = automatic) */
     int linear_no_lds_stream; /* few-row projections: 1 = never stage the weight stream through LDS (tests compare the two paths) */
+    int no_prefill_rope_epilogue; /* 1: gd_backend_linear_qkv_rope_packed answers GD_ERR_UNSUPPORTED, so a caller stays with
+                                     the separate operators (tests compare the two paths) */
 };
 
 struct gd_backend_buffer {

@@ -264,6 +264,7 @@ gd_status gd_backend_linear_qkv_rope_packed(gd_backend *backend, const gd_backen
         (uint64_t)cos_rows->shape[0] * (head_dim / 2u) > 0x7fffffffull ||
         sin_rows->shape[1] != (int64_t)(head_dim / 2u) || (cache_rows->offset & 3u) != 0u)
         return GD_ERR_INVALID_ARGUMENT;
+    if (backend->no_prefill_rope_epilogue) return GD_ERR_UNSUPPORTED; /* tunable "prefill_rope_epilogue" = 0 */
     /* the tile kernel's rotation epilogue: head size 64 or 128, heads * head_dim a multiple of 256 (every 128-column
      * block of a wavefront inside q, k or v), K a multiple of 64, 16-byte aligned rows everywhere, caches whose rows a
      * 31-bit row number reaches */

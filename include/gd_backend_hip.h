@@ -618,6 +618,8 @@ gd_status gd_backend_device_info(const gd_backend *backend, char *name, size_t n
  * otherwise deal an output with fewer full tiles than compute units out in narrower ones (same results to the bit).
  * "linear_no_lds_stream" = 1: the few-row projection always loads its weight fragments straight into registers,
  * also where it would stage the weight stream through LDS (same results to the bit; for comparing the two).
+ * "prefill_rope_epilogue" = 0: gd_backend_linear_qkv_rope_packed answers GD_ERR_UNSUPPORTED, so that a caller (the
+ * decoder's prefill) stays with the separate projection and rotation + append launches (for comparing the two).
  * Unknown name -> GD_ERR_INVALID_ARGUMENT. */
 gd_status gd_backend_set_tunable(gd_backend *backend, const char *name, int64_t value);
 

@@ -557,3 +557,55 @@ def test_resident_steps_over_long_ragged_caches_take_the_pieces_form(gda, oracle
     finally:
         dev.close()
         ref.close()
+
+
+def test_prefill_with_the_rotation_in_the_projection_matches_the_separate_launches(gda, oracle):
+    """A packed prefill of 12,100 tokens at head size 128 (d_model 512, 4 heads): 47 row tiles x 6 column tiles of the
+    qkv projection are more than a round on 256 compute units, so 42 row tiles take the tile kernel's rotation + split +
+    cache append epilogue and the remaining 1,348 rows the plain projection and the table-driven rotation kernel; the
+    attention reads keys and values from the caches.  Against the same decoder with the tunable
+    "prefill_rope_epilogue" = 0 (separate projection and rotation + append launches): first-layer values bit for bit,
+    first-layer keys to one unit in the last place, last-layer caches and logits within the decoder tests' bar; and
+    against the CPU oracle on the two shortest sequences."""
+    from gradients_c_amd import decoder as D
+    V, Dm, L, H, Dh, Hm, T, B = 2048, 512, 2, 4, 128, 1024, 2048, 8
+    lens = np.array([2048, 1900, 1500, 1700, 1200, 2000, 1100, 652], np.int32)
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    prompt = oracle.uniform_i32(int(cu[-1]), 4601, 0, V - 1)
+    dev = D.GptDecoder(D.gpt_config(V, Dm, L, H, Dh, Hm, T, B, 0, False, 4600), max_prefill_tokens=int(cu[-1]))
+    rows = [6, 7]
+    ref = oracle.Decoder(V, Dm, L, H, Dh, Hm, T, len(rows), 0, 4600, False)
+    try:
+        be = dev.ctx.backend()
+        lg_a, nx_a, gp_a = dev.prefill(prompt, cu)
+        caches_a = [(dev.read_tensor("k_cache", l), dev.read_tensor("v_cache", l)) for l in range(L)]
+        be.set_tunable("prefill_rope_epilogue", 0)
+        lg_b, nx_b, gp_b = dev.prefill(prompt, cu)
+        caches_b = [(dev.read_tensor("k_cache", l), dev.read_tensor("v_cache", l)) for l in range(L)]
+        be.set_tunable("prefill_rope_epilogue", 1)
+        for b in range(B):
+            n = lens[b]
+            ka, va, kb, vb = caches_a[0][0][b, :n], caches_a[0][1][b, :n], caches_b[0][0][b, :n], caches_b[0][1][b, :n]
+            assert np.array_equal(va.view(np.uint16), vb.view(np.uint16)), b
+            ulp = np.spacing(np.maximum(np.abs(ka), np.abs(kb)).astype(np.float16)).astype(np.float32)
+            assert np.all(np.abs(ka.astype(np.float32) - kb.astype(np.float32)) <= ulp), b
+            assert np.count_nonzero(ka.view(np.uint16) != kb.view(np.uint16)) <= max(2, ka.size // 300), b
+            for which in (0, 1):
+                xa, xb = caches_a[L - 1][which][b, :n].astype(np.float32), caches_b[L - 1][which][b, :n].astype(np.float32)
+                assert np.abs(xa - xb).max() < 8e-3, (b, which)
+        assert np.abs(lg_a.astype(np.float32) - lg_b.astype(np.float32)).max() < 8e-3
+        _assert_ids(nx_a, nx_b, gp_a, gp_b, "fused against separate launches")
+        sub = np.concatenate([prompt[cu[r]:cu[r + 1]] for r in rows])
+        sub_cu = np.concatenate([[0], np.cumsum(lens[rows])]).astype(np.int32)
+        lg_r, nx_r, gp_r = ref.prefill(sub, sub_cu)
+        assert np.abs(lg_a[rows].astype(np.float32) - lg_r.astype(np.float32)).max() < 8e-3
+        _assert_ids(nx_a[rows], nx_r, gp_a[rows], gp_r, "fused against the oracle")
+        for i, r in enumerate(rows):
+            for l in range(L):
+                kd, kr = caches_a[l][0][r, :lens[r]], ref.tensor("k_cache", l)[i, :lens[r]]
+                vd, vr = caches_a[l][1][r, :lens[r]], ref.tensor("v_cache", l)[i, :lens[r]]
+                assert np.abs(kd.astype(np.float32) - kr.astype(np.float32)).max() < 8e-3, (l, r)
+                assert np.abs(vd.astype(np.float32) - vr.astype(np.float32)).max() < 8e-3, (l, r)
+    finally:
+        dev.close()
+        ref.close()
