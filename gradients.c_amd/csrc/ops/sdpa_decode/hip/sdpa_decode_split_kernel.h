@@ -58,45 +58,11 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
      * the same arithmetic everywhere, so all workgroups agree): rows of about one length (the longest within 1.25
      * of the mean) are cut into p.even_pieces equal parts instead (one part: the row stays whole and nothing is
      * merged), which is the one-workgroup-per-row kernel again. */
-    int split, hkv, b, pos, pos_lane = 0, chunk = (int)p.chunk;
-    if (PIECES) {
-        constexpr int RS = GD_HIP_SDPA_PIECES_MAX_BATCH / 64;
-        split = blockIdx.z, hkv = blockIdx.x, b = blockIdx.y;
-        int longest = 0, total = 0, rows = 0;
-        pos = -1;
-#pragma unroll
-        for (int i = 0; i < RS; ++i) {
-            const int r = i * 64 + lane;
-            const int at = r < (int)p.batch ? pos_ptr[r] : -1;
-            int l_, f_, a_, b_;
-            const int n = at >= 0 ? max(visible(at, l_, f_, a_, b_), 0) : 0;
-            longest = max(longest, n);
-            total += n;
-            rows += at >= 0 ? 1 : 0;
-            if ((b >> 6) == i) pos = __builtin_amdgcn_readlane(at, b & 63);
-        }
-        longest = gd_wave_reduce_i32(longest, [](int x, int y) { return max(x, y); });
-        total = gd_wave_reduce_i32(total, [](int x, int y) { return x + y; });
-        rows = gd_wave_reduce_i32(rows, [](int x, int y) { return x + y; });
-        /* p.even_pieces is 0 (never), 1 or 2; p.chunk times the pieces of the grid covers the longest row there can be */
-        if (p.even_pieces != 0u && 4.f * (float)longest * (float)rows <= 5.f * (float)total)
-            chunk = max((((longest + (int)p.even_pieces - 1) >> (p.even_pieces >> 1)) + 31) & ~31, 32);
-    } else {
-        split = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z;
-        if (ahead) {
-            /* the position is requested through a lane address the compiler cannot prove uniform, so that it stays
-             * in a vector register (no wait) until the wavefront's first rows have been requested */
-            pos_lane = p.cache_pos;
-            if (p.pos_mode != GD_HIP_SDPA_POS_SCALAR) {
-                int idx = p.pos_mode == GD_HIP_SDPA_POS_VECTOR ? b : 0;
-                asm volatile("" : "+v"(idx));
-                pos_lane = pos_ptr[idx];
-            }
-            pos = 0;
-        } else {
-            pos = gd_decode_pos(pos_ptr, p, b);
-        }
-    }
+    const int split = PIECES ? blockIdx.z : blockIdx.x, hkv = PIECES ? blockIdx.x : blockIdx.y;
+    const int b = PIECES ? blockIdx.y : blockIdx.z;
+    int pos, pos_lane = 0, chunk = (int)p.chunk;
+    /* PIECES without a window or a prefix: the first piece of a row requests its first rows ahead of the positions */
+    const bool pieces_ahead = PIECES && !PFX && p.window == 0u;
 
     /* Addresses: one scalar base per cache for this (batch row, kv head), plus a 32-bit byte offset per lane
      * made by one 24-bit multiply-add (the host checks that tmax, the row pitch and their product fit).  The
@@ -129,6 +95,58 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
         }
     };
     gd_half8 kA[UNROLL], vA[UNROLL], kB[UNROLL], vB[UNROLL];
+    auto load_rows_early = [&](int s0) __attribute__((always_inline)) { load_rows(kA, vA, s0, (int)p.tmax - 1, 0, 0); };
+
+    if (PIECES) {
+        constexpr int RS = GD_HIP_SDPA_PIECES_MAX_BATCH / 64;
+        int longest = 0, total = 0, rows = 0;
+        pos = -1;
+        int at_row[RS];
+#pragma unroll
+        for (int i = 0; i < RS; ++i) {
+            const int r = i * 64 + lane;
+            at_row[i] = r < (int)p.batch ? pos_ptr[r] : -1;
+        }
+        /* The first piece of a row starts at key 0 whatever the positions say (no window, no prefix), and the first
+         * pieces hold the lowest workgroup numbers: they are the workgroups the launch starts with.  Their first rows
+         * are requested here, behind the requests for the positions and in front of their first use, so that the two
+         * round trips overlap at the start of the launch (later pieces start next to running ones, and pieces a row
+         * does not have must not load anything). */
+        __builtin_amdgcn_sched_barrier(0);
+        if (pieces_ahead && split == 0) load_rows_early(wave * KPW);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < RS; ++i) {
+            const int at = at_row[i];
+            int l_, f_, a_, b_;
+            const int n = at >= 0 ? max(visible(at, l_, f_, a_, b_), 0) : 0;
+            longest = max(longest, n);
+            total += n;
+            rows += at >= 0 ? 1 : 0;
+            if ((b >> 6) == i) pos = __builtin_amdgcn_readlane(at, b & 63);
+        }
+        longest = gd_wave_reduce_i32(longest, [](int x, int y) { return max(x, y); });
+        total = gd_wave_reduce_i32(total, [](int x, int y) { return x + y; });
+        rows = gd_wave_reduce_i32(rows, [](int x, int y) { return x + y; });
+        /* p.even_pieces is 0 (never), 1 or 2; p.chunk times the pieces of the grid covers the longest row there can be */
+        if (p.even_pieces != 0u && 4.f * (float)longest * (float)rows <= 5.f * (float)total)
+            chunk = max((((longest + (int)p.even_pieces - 1) >> (p.even_pieces >> 1)) + 31) & ~31, 32);
+    } else {
+        if (ahead) {
+            /* the position is requested through a lane address the compiler cannot prove uniform, so that it stays
+             * in a vector register (no wait) until the wavefront's first rows have been requested */
+            pos_lane = p.cache_pos;
+            if (p.pos_mode != GD_HIP_SDPA_POS_SCALAR) {
+                int idx = p.pos_mode == GD_HIP_SDPA_POS_VECTOR ? b : 0;
+                asm volatile("" : "+v"(idx));
+                pos_lane = pos_ptr[idx];
+            }
+            pos = 0;
+        } else {
+            pos = gd_decode_pos(pos_ptr, p, b);
+        }
+    }
+
     /* Without a window the wavefront's first rows do not depend on the row's position: they are requested here,
      * behind the request for the position and in front of its first use, so that the two round trips overlap.  What
      * the position then says does not exist (rows from the live length on; they lie inside the cache, so the loads
@@ -137,9 +155,10 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
     if (ahead) load_rows(kA, vA, split * chunk + wave * KPW, (int)p.tmax - 1, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
     if (ahead) pos = __builtin_amdgcn_readfirstlane(pos_lane);
+    const bool ahead_now = ahead || (pieces_ahead && split == 0); /* the first rows are on their way */
     /* (the early exits below read a loaded register, which keeps the loads above in front of the branches) */
     if (pos < 0) {
-        if (ahead) asm volatile("" ::"v"(kA[0]), "v"(vA[0]));
+        if (ahead_now) asm volatile("" ::"v"(kA[0]), "v"(vA[0]));
         return;
     }
     int live, first, a_len, b0;
@@ -154,7 +173,7 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
     const uint32_t npieces = ((uint32_t)max(n_vis, 0) + (uint32_t)chunk - 1u) / (uint32_t)chunk;
     const bool partial = PIECES ? npieces > 1u : p.nsplit > 1u;
     if (r0 >= r1) {
-        if (ahead) asm volatile("" ::"v"(kA[0]), "v"(vA[0]));
+        if (ahead_now) asm volatile("" ::"v"(kA[0]), "v"(vA[0]));
         if (PIECES) {
             /* a piece the row does not have; the first piece of a row without a visible key stores zeros */
             if (split != 0) return;
@@ -183,7 +202,7 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
     /* trips are decided per wavefront (scalar branches), rows past the range are masked per lane */
     const int jw = r0 + wave * KPW;
     const bool any_rows = jw < r1;
-    if (any_rows && !ahead) load_trip(kA, vA, jw);
+    if (any_rows && !ahead_now) load_trip(kA, vA, jw);
     __builtin_amdgcn_sched_barrier(0); /* nothing below moves in front of the first loads */
 
     /* query rows of the G heads that share this kv head stay in F16: products of two halfs are
@@ -206,7 +225,7 @@ gd_sdpa_decode_split_kernel(const gd_half *__restrict__ q, const gd_half *__rest
         for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
     }
 
-    bool unchecked = ahead; /* the buffers hold rows that were requested before the live length was known */
+    bool unchecked = ahead_now; /* the buffers hold rows that were requested before the live length was known */
     auto compute_trip = [&](const gd_half8 (&kv)[UNROLL], const gd_half8 (&vin)[UNROLL], int s0)
         __attribute__((always_inline)) {
         gd_half8 vv[UNROLL];
