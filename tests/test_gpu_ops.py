@@ -1559,6 +1559,22 @@ def test_linear_qkv_rope_packed_equals_separate_ops(backend, arena, oracle, gda,
     for b in (b for b in range(B) if b not in skipped):
         _close(got_k[b, cache_pos[b]:cache_pos[b] + lens[b]], ko[cu[b]:cu[b + 1]], atol=8e-3)
         _close(got_v[b, cache_pos[b]:cache_pos[b] + lens[b]], vo[cu[b]:cu[b + 1]], atol=8e-3)
+    # arguments that do not fit together are refused before anything is launched
+    a = gda.RopeArgs(10000.0, D, 0)
+    short = arena.alloc((N - 1,), gda.I32)
+    assert backend.call("gd_backend_rope_table_packed", tpos.view(), tcp.view(), tcu.view(), cos_rows.view(), sin_rows.view(),
+                        short.view(), D, Tmax, C.byref(a)) == gda.INVALID_ARGUMENT          # cache_rows one row short
+    assert backend.call("gd_backend_rope_table_packed", tpos.view(), tcp.view(), tcu.view(), cos_rows.view(), sin_rows.view(),
+                        cache_rows.view(), D, 0, C.byref(a)) == gda.INVALID_ARGUMENT         # caches without rows
+    inter = gda.RopeArgs(10000.0, D, 1)
+    assert backend.call("gd_backend_rope_table_packed", tpos.view(), tcp.view(), tcu.view(), cos_rows.view(), sin_rows.view(),
+                        cache_rows.view(), D, Tmax, C.byref(inter)) == gda.UNSUPPORTED      # interleaved pairing
+    assert backend.call("gd_backend_linear_qkv_rope_packed", tx.matrix(), tw.matrix(), tb.vector(), cos_rows.view(),
+                        sin_rows.view(), short.view(), q1.view(), kc1.view(), vc1.view(), work.matrix(), H, D, 2) == gda.INVALID_ARGUMENT
+    assert backend.call("gd_backend_linear_qkv_rope_packed", tx.matrix(), tw.matrix(), None, cos_rows.view(),
+                        sin_rows.view(), cache_rows.view(), q1.view(), kc1.view(), vc1.view(), work.matrix(), H, D, 2) == gda.INVALID_ARGUMENT
+    assert backend.call("gd_backend_linear_qkv_rope_packed", tx.matrix(), tw.matrix(), tb.vector(), cos_rows.view(),
+                        sin_rows.view(), cache_rows.view(), q1.view(), kc1.view(), vc1.view(), work.matrix(), H + 1, D, 2) == gda.INVALID_ARGUMENT
     # refused, not mis-run: a head size the rotation epilogue does not cover
     q96 = arena.alloc((N, 4, 96), gda.F16)
     kc96 = arena.alloc((B, 16, 4, 96), gda.F16)
