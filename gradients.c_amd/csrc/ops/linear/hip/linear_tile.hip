@@ -700,11 +700,11 @@ gd_linear_tile_kernel(const gd_half *__restrict__ x, const gd_half *__restrict__
         dst += col0 - region * rp.hd + v * 8u;
         const uint32_t row_w = m0 + wm * (WM * 32u);
         typedef float gd_float4v __attribute__((ext_vector_type(4)));
-        /* what a pass needs from memory: the angles of its 32 rows (region q or k) and the destination rows of the
+        /* What a pass needs from memory: the angles of its 32 rows (region q or k) and the destination rows of the
          * lane's 8 row pieces.  Both are requested one pass ahead so that their latency passes behind the pass in
          * front: the angles into the registers the running pass has just used them from, the rows into a second
-         * set. */
-        /* element offset of the lane's first angle of pass I in the angle tables, which are laid out for this read
+         * set.
+         * table_at: element offset of the lane's first angle of pass I in the angle tables, which are laid out for this read
          * (blocks of 32 rows, groups of 8 pairs, the low and the high 4 pairs of all 32 rows: the 64 lanes of a load
          * read 1 KB of consecutive memory; group g of the block lies 256 elements behind group g - 1); a signed
          * 32-bit number (the launcher keeps the tables below 2^31 elements), so that the loads take the table's base

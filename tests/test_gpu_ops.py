@@ -1026,7 +1026,13 @@ def test_many_row_projection_tail_in_192_row_tiles(backend, arena, oracle, K):
     _close(y.read(), oracle.linear_nt(x, w))
     backend.fused_linear(tx, tw, tb, tr, None, y, True, 2, 0)
     inter = oracle.linear_nt(x, w, bias)
-    _close(y.read(), oracle.add(res, inter), through=inter)
+    got = y.read()
+    _close(got, oracle.add(res, inter), through=inter)
+    # the 192-row launch starts at row 13192 - 27 * 192 = 8008: rows 8008..8191 are rows of the first launch computed
+    # once more.  The same rows from a call over the first 8,192 rows alone (whole 256 x 256 tiles only): same bits
+    y_head = arena.alloc((8192, N), 1)
+    backend.fused_linear(tx.rows(0, 8192), tw, tb, tr.rows(0, 8192), None, y_head, True, 2, 0)
+    assert np.array_equal(_bits(y_head.read()), _bits(got[:8192]))
 
 
 def test_many_row_projection_full_size_sampled(backend, oracle):
