@@ -37,8 +37,9 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 MFMA_F16_PEAK_TFLOPS = 2500.0  # published dense F16 matrix rate
 # HBM bytes per sdpa_decode launch at this shape from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
 # profiles/sdpa_decode_config2_pmc.md (fetch scaled by the factor a 64 MiB device copy shows in the same run); the
-# kernels with cacheable and with streaming loads read the same counters
-SDPA_TRAFFIC_BYTES = 67301600
+# kernel with cacheable loads (the one the step uses) and the one with streaming loads
+SDPA_TRAFFIC_BYTES = 67333269
+SDPA_TRAFFIC_BYTES_STREAMING = 67315867
 
 
 # A hardware queue's ring holds 16384 dispatch packets.  rocprofv3's queue interception has ended the profiled process
@@ -196,9 +197,8 @@ def sdpa_roofline(dec, D, pkg, iters=200):
             "with_streaming_loads": {"kernel": kernel_nt, "us_per_launch": round(sec_nt * 1e6, 3),
                                      "achieved": round(algo_bytes / sec_nt / 1e9, 1),
                                      "frac": round(algo_bytes / sec_nt / 1e9 / HBM_PEAK_GBS, 4),
-                                     "traffic": SDPA_TRAFFIC_BYTES,
-                                     "traffic_source": "counter runs of this kernel in the same profile: the same "
-                                                       "FETCH_SIZE / WRITE_SIZE as with cacheable loads"}}
+                                     "traffic": SDPA_TRAFFIC_BYTES_STREAMING,
+                                     "traffic_source": "counter runs of this kernel in the same profile"}}
 
 
 def kernel_only(pkg, launches=20, copy_mib=64):
